@@ -1,0 +1,240 @@
+"""The cache manager: page pools, block tables, state slots.
+
+Every entry of a model's layer order declares what it keeps
+(:class:`~pyre_amd.parts.base.KVCacheSpec`, :class:`~pyre_amd.parts.base.StateCacheSpec`
+or nothing). Entries with the same needs form a *group*:
+
+* a **page group** has a pool of pages of its own and, for each request, a block
+  table of its own. One page id addresses that page in every layer of the group
+  (`pyre/paged_cache.py:96-109` lays the reference's single pool out the same way).
+  A group with a window gives a page back as soon as no later query can see it.
+* a **state group** has one fixed-size state per (layer, slot).
+
+A request holds one *slot* from admission to its end; the slot indexes the state
+tensors. Pages are *reserved* for all tokens of a step before the step runs and
+the request's length is *committed* after it, so no kernel ever sees a half-grown
+table (`pyre/paged_cache.py:118-122,198-201` has per-layer side effects instead,
+and `tests/test_paged_cache.py:203-213` records the bug that came of it).
+
+This module is bookkeeping only and runs without a GPU; ``materialize`` allocates
+the pools' tensors.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from pyre_amd.cache.allocator import OutOfPages, PageAllocator
+from pyre_amd.parts.base import KVCacheSpec, StateCacheSpec
+
+RELEASED = -1  #: block-table entry of a page that a window has passed
+
+
+@dataclass
+class PageGroup:
+    index: int
+    spec: KVCacheSpec
+    entries: list[int]               #: positions in the layer order, ascending
+    page_size: int
+    num_pages: int
+    allocator: PageAllocator
+    k: object = None                 #: [len(entries), num_pages, nkv, page_size, hd]
+    v: object = None                 #: [len(entries), num_pages, nkv, hd, page_size]
+
+    def layer_index(self, entry: int) -> int:
+        return self.entries.index(entry)
+
+
+@dataclass
+class StateGroup:
+    index: int
+    spec: StateCacheSpec
+    entries: list[int]
+    tensor: object = None            #: [len(entries), num_slots, *shape]
+
+    def layer_index(self, entry: int) -> int:
+        return self.entries.index(entry)
+
+
+@dataclass
+class _Request:
+    slot: int
+    length: int = 0                  #: tokens committed
+    reserved: int = 0                #: tokens that pages exist for
+    tables: list[list[int]] = field(default_factory=list)  #: one per page group
+
+
+class CacheManager:
+    def __init__(self, cache_specs: list, page_size: int, num_pages: int, max_num_seqs: int,
+                 max_model_len: int):
+        """``cache_specs[i]`` is what entry i of the layer order keeps (or None)."""
+        if page_size <= 0 or num_pages <= 0 or max_num_seqs <= 0:
+            raise ValueError("page_size, num_pages and max_num_seqs must be positive")
+        self.page_size = page_size
+        self.max_num_seqs = max_num_seqs
+        self.max_model_len = max_model_len
+        self.max_pages_per_seq = -(-max_model_len // page_size)
+        self.page_groups: list[PageGroup] = []
+        self.state_groups: list[StateGroup] = []
+        #: entry -> ("kv" | "state", group index) for entries that keep something
+        self.group_of_entry: dict[int, tuple[str, int]] = {}
+        by_spec: dict[object, object] = {}
+        for entry, spec in enumerate(cache_specs):
+            if spec is None:
+                continue
+            grp = by_spec.get(spec)
+            if grp is None:
+                if isinstance(spec, KVCacheSpec):
+                    grp = PageGroup(len(self.page_groups), spec, [], page_size, num_pages,
+                                    PageAllocator(num_pages))
+                    self.page_groups.append(grp)
+                elif isinstance(spec, StateCacheSpec):
+                    grp = StateGroup(len(self.state_groups), spec, [])
+                    self.state_groups.append(grp)
+                else:
+                    raise TypeError(f"entry {entry}: unknown cache description {spec!r}")
+                by_spec[spec] = grp
+            grp.entries.append(entry)
+            self.group_of_entry[entry] = ("kv" if isinstance(grp, PageGroup) else "state", grp.index)
+        self.slots = PageAllocator(max_num_seqs, what="slot")
+        self._requests: dict[object, _Request] = {}
+
+    # ------------------------------------------------------------------ tensors
+
+    def materialize(self, device, dtype) -> None:
+        """Allocate the pools on ``device`` (keys and values in ``dtype``)."""
+        import torch
+
+        for g in self.page_groups:
+            s = g.spec
+            n = len(g.entries)
+            g.k = torch.zeros((n, g.num_pages, s.num_kv_heads, g.page_size, s.head_dim), device=device, dtype=dtype)
+            g.v = torch.zeros((n, g.num_pages, s.num_kv_heads, s.head_dim, g.page_size), device=device, dtype=dtype)
+        for g in self.state_groups:
+            dt = torch.float32 if g.spec.dtype == "float32" else dtype
+            g.tensor = torch.zeros((len(g.entries), self.max_num_seqs, *g.spec.shape), device=device, dtype=dt)
+
+    def bytes_per_page(self, dtype_bytes: int) -> int:
+        return sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * g.page_size * dtype_bytes
+                   for g in self.page_groups)
+
+    # ------------------------------------------------------------------ requests
+
+    def __contains__(self, rid) -> bool:
+        return rid in self._requests
+
+    @property
+    def live_requests(self) -> list:
+        return list(self._requests)
+
+    def has_free_slot(self) -> bool:
+        return self.slots.num_free > 0
+
+    def add_request(self, rid) -> int:
+        if rid in self._requests:
+            raise ValueError(f"request {rid!r} already exists")
+        slot = self.slots.allocate()
+        self._requests[rid] = _Request(slot, tables=[[] for _ in self.page_groups])
+        for g in self.state_groups:
+            if g.tensor is not None:
+                g.tensor[:, slot].zero_()
+        return slot
+
+    def slot(self, rid) -> int:
+        return self._requests[rid].slot
+
+    def length(self, rid) -> int:
+        return self._requests[rid].length
+
+    def _pages_to_add(self, req: _Request, new_len: int) -> int:
+        have = len(req.tables[0]) if self.page_groups else 0
+        return max(0, -(-new_len // self.page_size) - have)
+
+    def pages_needed(self, rid, n_new: int) -> int:
+        """Pages per group that ``reserve(rid, n_new)`` would take (rid may be new: None)."""
+        if not self.page_groups:
+            return 0
+        if rid is None or rid not in self._requests:
+            return -(-n_new // self.page_size)
+        req = self._requests[rid]
+        return self._pages_to_add(req, req.length + n_new)
+
+    def free_pages(self) -> int:
+        """Free pages of the tightest group."""
+        return min((g.allocator.num_free for g in self.page_groups), default=1 << 30)
+
+    def reserve(self, rid, n_new: int) -> None:
+        """Make room for the next ``n_new`` tokens of ``rid`` in every page group.
+        Takes all pages or none (:class:`OutOfPages`)."""
+        req = self._requests[rid]
+        new_len = req.length + n_new
+        if new_len > self.max_model_len:
+            raise ValueError(f"request {rid!r} would reach {new_len} tokens; the engine's limit is {self.max_model_len}")
+        add = self._pages_to_add(req, new_len)
+        if add:
+            for g in self.page_groups:
+                if g.allocator.num_free < add:
+                    raise OutOfPages(f"page pool of group {g.index} exhausted "
+                                     f"({add} needed, {g.allocator.num_free} of {g.num_pages} free)")
+            for g, table in zip(self.page_groups, req.tables):
+                table.extend(g.allocator.allocate_many(add))
+        req.reserved = max(req.reserved, new_len)
+
+    def slot_mapping(self, rid, group: int, start: int, n: int) -> list[int]:
+        """Flat cache slot (page * page_size + offset) of positions start .. start+n-1."""
+        table = self._requests[rid].tables[group]
+        ps = self.page_size
+        out = []
+        for pos in range(start, start + n):
+            page = table[pos // ps]
+            if page == RELEASED:
+                raise RuntimeError(f"position {pos} of request {rid!r} lies in a released page")
+            out.append(page * ps + pos % ps)
+        return out
+
+    def block_table(self, rid, group: int) -> list[int]:
+        return self._requests[rid].tables[group]
+
+    def commit(self, rid, n_new: int) -> None:
+        """The step has run: the request is ``n_new`` tokens longer. Pages of a
+        windowed group that no later query can see go back to the pool."""
+        req = self._requests[rid]
+        req.length += n_new
+        if req.length > req.reserved:
+            raise RuntimeError(f"request {rid!r}: committed past the reservation")
+        for g, table in zip(self.page_groups, req.tables):
+            w = g.spec.window
+            if w <= 0:
+                continue
+            # The next query sits at position req.length and sees keys > length - w.
+            dead_upto = req.length - w  # keys <= dead_upto are never read again
+            last_dead_page = (dead_upto + 1) // self.page_size - 1
+            for i in range(min(last_dead_page + 1, len(table))):
+                if table[i] != RELEASED:
+                    g.allocator.free(table[i])
+                    table[i] = RELEASED
+
+    def free_request(self, rid) -> None:
+        req = self._requests.pop(rid)
+        for g, table in zip(self.page_groups, req.tables):
+            for page in reversed(table):
+                if page != RELEASED:
+                    g.allocator.free(page)
+        self.slots.free(req.slot)
+
+    # ------------------------------------------------------------------ checks
+
+    def check_invariants(self) -> None:
+        """No page lost, held twice or free while held (used by the tests)."""
+        for gi, g in enumerate(self.page_groups):
+            held = [p for r in self._requests.values() for p in r.tables[gi] if p != RELEASED]
+            if len(held) != len(set(held)):
+                raise AssertionError(f"group {gi}: a page is held twice")
+            if len(held) != g.allocator.num_used:
+                raise AssertionError(f"group {gi}: {g.allocator.num_used} pages in use, {len(held)} held")
+            for p in held:
+                if not g.allocator.is_used(p):
+                    raise AssertionError(f"group {gi}: page {p} is held but free")
+        slots = [r.slot for r in self._requests.values()]
+        if len(slots) != len(set(slots)) or len(slots) != self.slots.num_used:
+            raise AssertionError("slot bookkeeping is inconsistent")

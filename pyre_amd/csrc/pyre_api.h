@@ -1,0 +1,51 @@
+// C entry points of the gfx950 kernel library. Pointers are device pointers
+// unless a comment says otherwise; `stream` is the HIP stream the work is put on.
+// Every function returns 0, or non-zero after storing a message that
+// pyre_last_error() returns. Element type codes: 0 = float32, 1 = bfloat16.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+extern "C" {
+
+const char* pyre_last_error();
+int pyre_abi_version();
+
+int pyre_embed(const void* table, int table_dt, const int* ids, float* out, int n, int hidden,
+               hipStream_t stream);
+
+int pyre_add_rmsnorm(float* resid, const void* delta, int delta_dt, int n_partials,
+                     long partial_stride, const void* bias, int bias_dt, const void* gain,
+                     int gain_dt, void* out, int out_dt, const int* rows, int n, int hidden,
+                     float eps, hipStream_t stream);
+
+int pyre_rope_kv_write(const void* qkv, int qkv_dt, int n_partials, long partial_stride,
+                       const void* bias, int bias_dt, void* q_out, int q_dt, void* k_cache,
+                       void* v_cache, int cache_dt, const float* cos_t, const float* sin_t,
+                       int rotary_dim, const int* positions, const int* slots, int n, int nq,
+                       int nkv, int hd, int page_size, int write_kv, hipStream_t stream);
+
+int pyre_silu_mul(const void* gu, int gu_dt, int n_partials, long partial_stride, void* out,
+                  int out_dt, int n, int inter, hipStream_t stream);
+
+int pyre_reduce_partials(const void* in, int in_dt, int n_partials, long partial_stride,
+                         const void* bias, int bias_dt, void* out, int out_dt, int n, int width,
+                         hipStream_t stream);
+
+int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, const void* W,
+                      int w_dt, long ldw, const void* bias, int bias_dt, void* out, int out_dt,
+                      long ldo, int M, int N, int K, hipStream_t stream);
+
+int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
+                      const void* v_cache, int cache_dt, const int* positions,
+                      const int* seq_of_token, const int* block_table, int table_stride, int n,
+                      int nq, int nkv, int hd, int page_size, float scale, int window,
+                      hipStream_t stream);
+
+int pyre_argmax(const float* logits, long row_stride, int* out, int m, int vocab,
+                hipStream_t stream);
+
+int pyre_sample(const float* logits, long row_stride, const float* temperature,
+                const float* uniform, int* out, int m, int vocab, hipStream_t stream);
+
+}  // extern "C"

@@ -1,0 +1,125 @@
+// Shared helpers for the gfx950 kernels: element types, conversions, reductions,
+// error reporting. Everything here is device code for 64-wide wavefronts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace pyre {
+
+constexpr int kWave = 64;
+
+// Element type codes shared with the Python binding.
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+// bfloat16 as its raw 16 bits; conversions are explicit so that every rounding
+// in a kernel is visible where it happens.
+struct bf16 {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float to_float(float v) { return v; }
+__host__ __device__ inline float to_float(bf16 v) {
+  union { uint32_t u; float f; } x;
+  x.u = static_cast<uint32_t>(v.bits) << 16;
+  return x.f;
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__host__ __device__ inline uint16_t bf16_bits(float f) {
+  union { uint32_t u; float f; } x;
+  x.f = f;
+  if ((x.u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((x.u >> 16) | 0x40u);
+  x.u += 0x7fffu + ((x.u >> 16) & 1u);
+  return static_cast<uint16_t>(x.u >> 16);
+}
+
+template <typename T> __host__ __device__ inline T from_float(float v);
+template <> __host__ __device__ inline float from_float<float>(float v) { return v; }
+template <> __host__ __device__ inline bf16 from_float<bf16>(float v) {
+  bf16 r;
+  r.bits = bf16_bits(v);
+  return r;
+}
+
+// Read element i of an array whose element type is only known at run time.
+__device__ inline float load_as_float(const void* p, int dt, size_t i) {
+  return dt == kF32 ? static_cast<const float*>(p)[i] : to_float(static_cast<const bf16*>(p)[i]);
+}
+__device__ inline void store_from_float(void* p, int dt, size_t i, float v) {
+  if (dt == kF32) static_cast<float*>(p)[i] = v;
+  else static_cast<bf16*>(p)[i] = from_float<bf16>(v);
+}
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Block-wide reductions for blocks of up to 1024 threads (16 waves). `scratch`
+// is 16 floats of LDS. Every thread receives the result; the order of the
+// additions is fixed by the thread layout alone.
+__device__ inline float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int w = threadIdx.x / kWave, nw = (blockDim.x + kWave - 1) / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[w] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += scratch[i];
+  return t;
+}
+__device__ inline float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int w = threadIdx.x / kWave, nw = (blockDim.x + kWave - 1) / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[w] = v;
+  __syncthreads();
+  float t = scratch[0];
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, scratch[i]);
+  return t;
+}
+
+// ---- host side -------------------------------------------------------------
+
+// The last error of this thread, returned to Python by pyre_last_error().
+char* error_buffer();
+
+inline int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail("%s: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+inline bool known_dtype(int dt) { return dt == kF32 || dt == kBF16; }
+
+}  // namespace pyre
+
+#define PYRE_REQUIRE(cond, ...) \
+  do {                          \
+    if (!(cond)) return pyre::fail(__VA_ARGS__); \
+  } while (0)
+
+// Calls `body` with `T` bound to the element type that `dt` names.
+#define PYRE_DISPATCH(dt, T, ...)                         \
+  do {                                                    \
+    if ((dt) == pyre::kF32) { using T = float; __VA_ARGS__; } \
+    else { using T = pyre::bf16; __VA_ARGS__; }           \
+  } while (0)

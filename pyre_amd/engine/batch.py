@@ -1,0 +1,101 @@
+"""A step's batch as flat arrays.
+
+A step is a list of entries ``(request, its next tokens, which of them want
+logits)``: portions of prompts beside single decoded tokens, in any mix
+(`pyre/model.py:251-294` runs one request with any number of tokens, `:297-342`
+many requests with one token each; here both are one call). The arrays below
+are everything the kernels need; they are packed into one int32 buffer so that a
+step costs one host-to-device copy.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+
+
+@dataclass
+class Entry:
+    rid: object
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)  #: indices into ``tokens``
+
+
+@dataclass
+class HostBatch:
+    """Host-side description of one step (numpy int32 arrays)."""
+
+    n_tokens: int
+    n_seqs: int
+    rids: list
+    tokens: np.ndarray          #: [N]
+    positions: np.ndarray       #: [N] absolute position of each token
+    seq_of_token: np.ndarray    #: [N] row of the step's block tables
+    q_start: np.ndarray         #: [S + 1] first token of each request's run
+    ctx_len: np.ndarray         #: [S] keys each request has after this step
+    state_slots: np.ndarray     #: [S] the request's state slot
+    logit_rows: np.ndarray      #: [M] token indices whose logits are wanted, in entry order
+    slots: list[np.ndarray]     #: per page group [N]: cache slot of each token
+    tables: list[np.ndarray]    #: per page group [S, P]: block tables (-1: released or unused)
+    max_q_len: int = 0
+
+    @property
+    def decode_only(self) -> bool:
+        return self.max_q_len == 1
+
+
+def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: int | None = None) -> HostBatch:
+    """Lay the entries out in the order given. ``cache`` is the
+    :class:`~pyre_amd.cache.CacheManager`; every request must already have its
+    pages reserved for this step."""
+    if not entries:
+        raise ValueError("a step needs at least one entry")
+    seen = set()
+    tokens: list[int] = []
+    positions: list[int] = []
+    seq_of_token: list[int] = []
+    q_start = [0]
+    ctx_len: list[int] = []
+    state_slots: list[int] = []
+    logit_rows: list[int] = []
+    n_groups = len(cache.page_groups)
+    slots: list[list[int]] = [[] for _ in range(n_groups)]
+    width = table_width or cache.max_pages_per_seq
+    tables = [np.full((len(entries), width), -1, dtype=np.int32) for _ in range(n_groups)]
+    max_q = 0
+    for s, e in enumerate(entries):
+        if e.rid in seen:
+            raise ValueError(f"request {e.rid!r} appears twice in one step")
+        seen.add(e.rid)
+        n = len(e.tokens)
+        if n == 0:
+            raise ValueError(f"request {e.rid!r} brings no tokens")
+        for t in e.tokens:
+            if not (0 <= int(t) < vocab_size):
+                raise ValueError(f"token id {t} of request {e.rid!r} is outside the vocabulary (0..{vocab_size - 1})")
+        start = cache.length(e.rid)
+        base = len(tokens)
+        tokens.extend(int(t) for t in e.tokens)
+        positions.extend(range(start, start + n))
+        seq_of_token.extend([s] * n)
+        q_start.append(base + n)
+        ctx_len.append(start + n)
+        state_slots.append(cache.slot(e.rid))
+        for w in e.want:
+            if not (0 <= int(w) < n):
+                raise ValueError(f"request {e.rid!r}: wanted place {w} is outside its {n} tokens")
+            logit_rows.append(base + int(w))
+        for g in range(n_groups):
+            slots[g].extend(cache.slot_mapping(e.rid, g, start, n))
+            tbl = cache.block_table(e.rid, g)
+            if len(tbl) > width:
+                raise ValueError(f"request {e.rid!r} has {len(tbl)} pages, the table holds {width}")
+            tables[g][s, :len(tbl)] = tbl
+        max_q = max(max_q, n)
+    i32 = lambda x: np.asarray(x, dtype=np.int32)  # noqa: E731
+    return HostBatch(
+        n_tokens=len(tokens), n_seqs=len(entries), rids=[e.rid for e in entries], tokens=i32(tokens),
+        positions=i32(positions), seq_of_token=i32(seq_of_token), q_start=i32(q_start),
+        ctx_len=i32(ctx_len), state_slots=i32(state_slots), logit_rows=i32(logit_rows),
+        slots=[i32(x) for x in slots], tables=tables, max_q_len=max_q)

@@ -1,0 +1,160 @@
+"""The engine: a model, its caches and one step function.
+
+``Engine.step(entries)`` runs exactly the tokens it is given, as one batch, against
+the cache that earlier steps left, and returns the float32 logits at the wanted
+places. The reference has three separate forwards for this (`pyre/model.py:188-201`
+contiguous cache and one shared start, `:251-294` one request with any number of
+tokens, `:297-342` many requests with one token each) and an empty `pyre/engine.py`.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+
+from pyre_amd.cache import CacheManager
+from pyre_amd.config.engine import EngineConfig
+from pyre_amd.config.model import ModelConfig
+from pyre_amd.engine.batch import Entry, build_host_batch
+from pyre_amd.engine.context import (TORCH_DTYPES, KVLayerView, MetaBuffers, Runtime, StateLayerView,
+                                     StepContext)
+from pyre_amd.parts.model import LayeredModel
+from pyre_amd.registry import get_architecture, load_config
+from pyre_amd.weights.loader import adopt_state, load_weights
+
+
+class Engine:
+    def __init__(self, model: LayeredModel, config: ModelConfig, engine_config: EngineConfig):
+        if not torch.cuda.is_available():
+            raise RuntimeError("pyre_amd needs a GPU: there is no CPU execution path")
+        from pyre_amd.hip import lib
+
+        lib.lib()  # fail now, and loudly, if the kernel library cannot be built or loaded
+        self.model = model
+        self.config = config
+        self.engine_config = ec = engine_config
+        self.device = torch.device(ec.device)
+        self.dtype = TORCH_DTYPES[ec.dtype]
+        spec = model.spec
+        self.max_model_len = min(ec.max_model_len or spec.max_positions, spec.max_positions)
+        self.runtime = Runtime(self.device, self.dtype, self.max_model_len)
+        specs = model.cache_specs()
+        probe = CacheManager(specs, ec.page_size, 1, ec.max_num_seqs, self.max_model_len)
+        num_pages = self._choose_num_pages(probe)
+        self.cache = CacheManager(specs, ec.page_size, num_pages, ec.max_num_seqs, self.max_model_len)
+        self.cache.materialize(self.device, self.dtype)
+        widths = [self.cache.max_pages_per_seq for _ in self.cache.page_groups]
+        self.meta = MetaBuffers(self.device, ec.max_num_batched_tokens, ec.max_num_seqs, widths)
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ construction
+
+    def _choose_num_pages(self, probe: CacheManager) -> int:
+        ec = self.engine_config
+        if ec.num_pages is not None:
+            return ec.num_pages
+        if ec.max_cached_tokens is not None:
+            return max(1, -(-ec.max_cached_tokens // ec.page_size))
+        per_page = probe.bytes_per_page(torch.empty((), dtype=self.dtype).element_size())
+        if per_page == 0:
+            return 1
+        free, _ = torch.cuda.mem_get_info(self.device)
+        want = int(free * ec.memory_fraction) // per_page
+        # No request can use more than its longest length; no pool needs more than all of them.
+        cap = ec.max_num_seqs * -(-self.max_model_len // ec.page_size)
+        return max(1, min(want, cap))
+
+    @classmethod
+    def from_folder(cls, folder: str | Path, engine_config: EngineConfig | None = None) -> "Engine":
+        """Model folder (config.json + *.safetensors) -> engine."""
+        ec = engine_config or EngineConfig()
+        config = load_config(folder)
+        model = LayeredModel(get_architecture(config.architecture).build(config))
+        tensors = load_weights(folder, model.tensor_specs(), torch.device(ec.device), TORCH_DTYPES[ec.dtype])
+        return cls._finish(model, config, ec, tensors)
+
+    @classmethod
+    def from_state(cls, config: ModelConfig, state: dict[str, torch.Tensor],
+                   engine_config: EngineConfig | None = None) -> "Engine":
+        """Tensors already in memory (random weights made on the device, tests)."""
+        ec = engine_config or EngineConfig()
+        model = LayeredModel(get_architecture(config.architecture).build(config))
+        tensors = adopt_state(state, model.tensor_specs(), torch.device(ec.device), TORCH_DTYPES[ec.dtype])
+        return cls._finish(model, config, ec, tensors)
+
+    @classmethod
+    def _finish(cls, model, config, ec, tensors) -> "Engine":
+        with torch.cuda.device(torch.device(ec.device)):
+            rt = Runtime(torch.device(ec.device), TORCH_DTYPES[ec.dtype], 0)
+            model.bind(tensors, rt)
+            tensors.clear()
+            return cls(model, config, ec)
+
+    # ------------------------------------------------------------------ the step
+
+    @property
+    def vocab_size(self) -> int:
+        return self.model.spec.vocab_size
+
+    def has(self, rid) -> bool:
+        return rid in self.cache
+
+    def step(self, entries: list[Entry]) -> torch.Tensor | None:
+        """Run one batch. Requests not seen before are admitted (a slot and empty
+        block tables); pages for all the step's tokens are reserved first, lengths
+        are committed afterwards. Returns float32 ``[sum(len(want)), vocab]`` on the
+        device, rows in the order of the entries and of each ``want`` (None if no
+        logits are wanted).
+        """
+        n_tokens = sum(len(e.tokens) for e in entries)
+        ec = self.engine_config
+        if n_tokens > ec.max_num_batched_tokens:
+            raise ValueError(f"step of {n_tokens} tokens exceeds max_num_batched_tokens={ec.max_num_batched_tokens}")
+        if len(entries) > ec.max_num_seqs:
+            raise ValueError(f"step of {len(entries)} requests exceeds max_num_seqs={ec.max_num_seqs}")
+        cache = self.cache
+        for e in entries:
+            if e.rid not in cache:
+                cache.add_request(e.rid)
+        for e in entries:
+            cache.reserve(e.rid, len(e.tokens))
+        pages = max((len(cache.block_table(e.rid, 0)) for e in entries), default=0) if cache.page_groups else 0
+        width = max(8, -(-pages // 8) * 8)
+        hb = build_host_batch(entries, cache, self.vocab_size, table_width=width)
+        with torch.cuda.device(self.device):
+            views = self.meta.upload(hb)
+            ctx = StepContext(
+                runtime=self.runtime, host=hb, n_tokens=hb.n_tokens, n_seqs=hb.n_seqs,
+                n_logits=len(hb.logit_rows), tokens=views["tokens"], positions=views["positions"],
+                seq_of_token=views["seq_of_token"], logit_rows=views["logit_rows"],
+                q_start=views["q_start"], ctx_len=views["ctx_len"], state_slots=views["state_slots"])
+            logits = self.model.forward(ctx, self._layer_views(views))
+        for e in entries:
+            cache.commit(e.rid, len(e.tokens))
+        self.steps_run += 1
+        return logits
+
+    def _layer_views(self, views) -> list:
+        cache = self.cache
+        out = []
+        for pos, call in enumerate(self.model.schedule):
+            src = call.cache_from if call.cache_from is not None else pos
+            where = cache.group_of_entry.get(src)
+            if where is None:
+                out.append(None)
+                continue
+            kind, gi = where
+            if kind == "kv":
+                g = cache.page_groups[gi]
+                li = g.layer_index(src)
+                out.append(KVLayerView(g.k[li], g.v[li], views[f"table{gi}"], views[f"slots{gi}"],
+                                       g.page_size, g.spec.window, writes=call.cache_from is None))
+            else:
+                g = cache.state_groups[gi]
+                out.append(StateLayerView(g.tensor[g.layer_index(src)], views["state_slots"]))
+        return out
+
+    def finish(self, rid) -> None:
+        """The request is over: its pages and its slot go back."""
+        self.cache.free_request(rid)

@@ -1,0 +1,66 @@
+"""ctypes binding of the kernel library: argument types, error translation.
+
+The library is loaded (and, if need be, compiled) at the first use of ``lib()``.
+There is no fallback: if it cannot be built or loaded, the caller gets the error.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+from pyre_amd.hip import build as _build
+
+ABI_VERSION = 1
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or failed to launch."""
+
+
+P, I, L, F = c_void_p, c_int, c_long, c_float
+
+_SIGNATURES = {
+    "pyre_embed": [P, I, P, P, I, I, P],
+    "pyre_add_rmsnorm": [P, P, I, I, L, P, I, P, I, P, I, P, I, I, F, P],
+    "pyre_rope_kv_write": [P, I, I, L, P, I, P, I, P, P, I, P, P, I, P, P, I, I, I, I, I, I, P],
+    "pyre_silu_mul": [P, I, I, L, P, I, I, I, P],
+    "pyre_reduce_partials": [P, I, I, L, P, I, P, I, I, I, P],
+    "pyre_gemm_generic": [P, I, L, P, P, I, L, P, I, P, I, L, I, I, I, P],
+    "pyre_attn_generic": [P, P, I, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+    "pyre_argmax": [P, L, P, I, I, P],
+    "pyre_sample": [P, L, P, P, P, I, I, P],
+}
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        path = _build.ensure_built()
+        handle = ctypes.CDLL(str(path))
+        handle.pyre_last_error.restype = ctypes.c_char_p
+        handle.pyre_abi_version.restype = c_int
+        if handle.pyre_abi_version() != ABI_VERSION:
+            # An older library from a previous checkout: rebuild once.
+            path = _build.build(force=True)
+            handle = ctypes.CDLL(str(path))
+            handle.pyre_last_error.restype = ctypes.c_char_p
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int
+        _lib = handle
+    return _lib
+
+
+def loaded_path() -> str | None:
+    return None if _lib is None else _lib._name
+
+
+def call(name: str, *args) -> None:
+    handle = lib()
+    rc = getattr(handle, name)(*args)
+    if rc != 0:
+        raise KernelError(handle.pyre_last_error().decode(errors="replace"))

@@ -1,0 +1,254 @@
+"""The kernels as functions of torch tensors.
+
+torch is the allocator and the owner of the stream here, nothing more: every
+function checks shapes, element types, device and contiguity on the host, then
+hands raw pointers to the HIP library. There is no CPU path; a tensor that is
+not on a GPU is an error.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from pyre_amd.hip.lib import KernelError, call
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def dtype_code(t: torch.Tensor | torch.dtype) -> int:
+    dt = t if isinstance(t, torch.dtype) else t.dtype
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise KernelError(f"unsupported element type {dt}; kernels take float32 and bfloat16") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operand is not on a GPU (there is no CPU path)")
+
+
+def _contig(name: str, t: torch.Tensor) -> None:
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+
+
+def _i32(name: str, t: torch.Tensor, n: int | None = None) -> None:
+    if t.dtype != torch.int32:
+        raise KernelError(f"{name} must be int32, got {t.dtype}")
+    _contig(name, t)
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name} holds {t.numel()} entries, {n} needed")
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+@dataclass
+class Partials:
+    """What a matrix product hands to its consumer: ``S`` partial sums ``[S, M, N]``
+    (``S`` = 1 unless the product was split along K) and a bias not yet added.
+    The consumer adds them up in the order 0..S-1, then the bias."""
+
+    data: torch.Tensor
+    bias: torch.Tensor | None = None
+
+    def __post_init__(self) -> None:
+        if self.data.dim() != 3 or not self.data.is_contiguous():
+            raise KernelError("partials must be a contiguous [S, M, N] tensor")
+
+    @property
+    def count(self) -> int:
+        return self.data.shape[0]
+
+    @property
+    def rows(self) -> int:
+        return self.data.shape[1]
+
+    @property
+    def width(self) -> int:
+        return self.data.shape[2]
+
+    @property
+    def stride(self) -> int:
+        return self.data.stride(0)
+
+    def _args(self, width: int):
+        if self.width != width:
+            raise KernelError(f"partials are {self.width} wide, {width} expected")
+        if self.bias is not None and self.bias.numel() != width:
+            raise KernelError(f"bias has {self.bias.numel()} entries, {width} expected")
+        return (self.data.data_ptr(), dtype_code(self.data), self.count, self.stride,
+                _ptr(self.bias), dtype_code(self.bias) if self.bias is not None else 0)
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    """out[n] = float32(table[ids[n]]); ids must already be checked against the vocabulary."""
+    _dev(table, ids, out)
+    n, hidden = out.shape
+    if table.dim() != 2 or table.shape[1] != hidden or out.dtype != torch.float32:
+        raise KernelError("embed: table [V, H] and float32 out [N, H] expected")
+    _contig("table", table), _contig("out", out), _i32("ids", ids, n)
+    call("pyre_embed", table.data_ptr(), dtype_code(table), ids.data_ptr(), out.data_ptr(), n, hidden,
+         _stream())
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+    """resid += delta (all partials, then bias); out = rmsnorm(resid) * gain.
+
+    With ``rows`` only those rows are normed, into ``out[0:len(rows)]``, and
+    ``resid`` is left as it was.
+    """
+    _dev(resid, gain, out, rows)
+    hidden = resid.shape[-1]
+    if resid.dtype != torch.float32 or resid.dim() != 2:
+        raise KernelError("add_rmsnorm: the residual stream is float32 [N, H]")
+    n = resid.shape[0] if rows is None else rows.numel()
+    if out.shape[-1] != hidden or out.shape[0] < n or gain.numel() != hidden:
+        raise KernelError("add_rmsnorm: shapes of out / gain do not fit the residual")
+    _contig("resid", resid), _contig("out", out), _contig("gain", gain)
+    if rows is not None:
+        _i32("rows", rows)
+    if delta is not None:
+        if delta.rows < resid.shape[0]:
+            raise KernelError("add_rmsnorm: delta has fewer rows than the residual")
+        d = delta._args(hidden)
+    else:
+        d = (None, 0, 0, 0, None, 0)
+    call("pyre_add_rmsnorm", resid.data_ptr(), *d, gain.data_ptr(), dtype_code(gain), out.data_ptr(),
+         dtype_code(out), _ptr(rows), n, hidden, float(eps), _stream())
+
+
+def rope_kv_write(qkv: Partials, q_out: torch.Tensor, k_cache: torch.Tensor | None,
+                  v_cache: torch.Tensor | None, cos: torch.Tensor | None, sin: torch.Tensor | None,
+                  rotary_dim: int, positions: torch.Tensor, slots: torch.Tensor | None, n: int,
+                  nq: int, nkv: int, hd: int, page_size: int) -> None:
+    """Finish the q/k/v projection (partials + bias), rotate q and k by position,
+    store q in ``q_out [N, nq*hd]`` and, when a cache is given, k and v in their pages.
+
+    ``k_cache`` is one layer's ``[pages, nkv, page_size, hd]``; ``v_cache`` the same
+    layer's ``[pages, nkv, hd, page_size]``. ``slots[n] = page * page_size + offset``,
+    or -1 for a token that is not to be stored.
+    """
+    _dev(qkv.data, q_out, k_cache, v_cache, cos, sin, positions, slots)
+    width = (nq + 2 * nkv) * hd
+    q = qkv._args(width)
+    if qkv.rows < n or q_out.numel() < n * nq * hd:
+        raise KernelError("rope_kv_write: buffers are smaller than the batch")
+    _contig("q_out", q_out), _i32("positions", positions, n)
+    write = k_cache is not None
+    cache_dt = 0
+    if write:
+        if v_cache is None or slots is None:
+            raise KernelError("rope_kv_write: k cache without v cache or slots")
+        _i32("slots", slots, n), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        if tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
+            raise KernelError(f"rope_kv_write: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} "
+                              f"do not fit nkv={nkv} page={page_size} hd={hd}")
+        cache_dt = dtype_code(k_cache)
+    if rotary_dim:
+        if cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32:
+            raise KernelError("rope_kv_write: float32 cos/sin tables needed")
+        if cos.dim() != 2 or cos.shape[1] != rotary_dim // 2 or cos.shape != sin.shape:
+            raise KernelError("rope_kv_write: cos/sin tables must be [positions, rotary_dim/2]")
+        _contig("cos", cos), _contig("sin", sin)
+    call("pyre_rope_kv_write", *q, q_out.data_ptr(), dtype_code(q_out), _ptr(k_cache), _ptr(v_cache),
+         cache_dt, _ptr(cos), _ptr(sin), rotary_dim, positions.data_ptr(), _ptr(slots), n, nq, nkv, hd,
+         page_size, 1 if write else 0, _stream())
+
+
+def silu_mul(gu: Partials, out: torch.Tensor, n: int) -> None:
+    """out[n, i] = silu(gate[n, i]) * up[n, i] with gate = gu[:, :I], up = gu[:, I:]."""
+    _dev(gu.data, out)
+    inter = out.shape[-1]
+    if gu.width != 2 * inter or gu.rows < n or out.shape[0] < n:
+        raise KernelError("silu_mul: gate/up buffer does not fit the output")
+    if gu.bias is not None:
+        raise KernelError("silu_mul: a pending bias is not supported")
+    _contig("out", out)
+    call("pyre_silu_mul", gu.data.data_ptr(), dtype_code(gu.data), gu.count, gu.stride, out.data_ptr(),
+         dtype_code(out), n, inter, _stream())
+
+
+def reduce_partials(p: Partials, out: torch.Tensor, n: int) -> None:
+    _dev(p.data, out)
+    if out.shape[-1] != p.width or out.shape[0] < n or p.rows < n:
+        raise KernelError("reduce_partials: shapes do not fit")
+    _contig("out", out)
+    call("pyre_reduce_partials", *p._args(p.width), out.data_ptr(), dtype_code(out), n, p.width, _stream())
+
+
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
+                 m: int, a_rows: torch.Tensor | None = None) -> None:
+    """out[0:m] = a[0:m] (or a[a_rows]) @ w.T (+ bias), fp32 accumulation in ascending k."""
+    _dev(a, w, bias, out, a_rows)
+    n_out, k = w.shape
+    if a.dim() != 2 or a.shape[1] != k or out.dim() != 2 or out.shape[1] != n_out:
+        raise KernelError(f"gemm: a {tuple(a.shape)} @ w {tuple(w.shape)}.T -> out {tuple(out.shape)} do not fit")
+    if a.stride(1) != 1 or w.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: rows must be contiguous")
+    if out.shape[0] < m or (a_rows is None and a.shape[0] < m):
+        raise KernelError("gemm: fewer rows than m")
+    if a_rows is not None:
+        _i32("a_rows", a_rows, m)
+    if bias is not None and bias.numel() != n_out:
+        raise KernelError("gemm: bias length")
+    call("pyre_gemm_generic", a.data_ptr(), dtype_code(a), a.stride(0), _ptr(a_rows), w.data_ptr(),
+         dtype_code(w), w.stride(0), _ptr(bias), dtype_code(bias) if bias is not None else 0,
+         out.data_ptr(), dtype_code(out), out.stride(0), m, n_out, k, _stream())
+
+
+def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                 n: int, nq: int, nkv: int, hd: int, page_size: int, scale: float,
+                 window: int = 0) -> None:
+    """Causal attention of n tokens over the paged cache; see attention_generic.hip."""
+    _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table)
+    if q.dtype != out.dtype or q.numel() < n * nq * hd or out.numel() < n * nq * hd:
+        raise KernelError("attn: q/out buffers do not fit")
+    if tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
+        raise KernelError("attn: cache shapes do not fit the head geometry")
+    if k_cache.dtype != v_cache.dtype:
+        raise KernelError("attn: k and v caches differ in element type")
+    _contig("q", q), _contig("out", out), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+    _i32("positions", positions, n), _i32("seq_of_token", seq_of_token, n)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("attn: block table must be int32 [rows, pages]")
+    call("pyre_attn_generic", q.data_ptr(), out.data_ptr(), dtype_code(q), k_cache.data_ptr(),
+         v_cache.data_ptr(), dtype_code(k_cache), positions.data_ptr(), seq_of_token.data_ptr(),
+         block_table.data_ptr(), block_table.stride(0), n, nq, nkv, hd, page_size, float(scale),
+         int(window), _stream())
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    _dev(logits, out)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("argmax: float32 [M, V] logits expected")
+    _i32("out", out, logits.shape[0])
+    call("pyre_argmax", logits.data_ptr(), logits.stride(0), out.data_ptr(), logits.shape[0],
+         logits.shape[1], _stream())
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+           out: torch.Tensor) -> None:
+    """Rows with temperature > 0 get a token drawn by inverse CDF with their
+    uniform number; rows with temperature <= 0 keep what ``out`` holds."""
+    _dev(logits, temperature, uniform, out)
+    m = logits.shape[0]
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("sample: float32 [M, V] logits expected")
+    for name, t in (("temperature", temperature), ("uniform", uniform)):
+        if t.dtype != torch.float32 or t.numel() < m or not t.is_contiguous():
+            raise KernelError(f"sample: {name} must be contiguous float32 [M]")
+    _i32("out", out, m)
+    call("pyre_sample", logits.data_ptr(), logits.stride(0), temperature.data_ptr(), uniform.data_ptr(),
+         out.data_ptr(), m, logits.shape[1], _stream())

@@ -1,0 +1,65 @@
+"""Grouped-query attention over the paged cache (`pyre/model.py:75-125,251-342`)."""
+
+from __future__ import annotations
+
+import torch
+
+from pyre_amd.hip import ops
+from pyre_amd.parts import fast
+from pyre_amd.parts.base import AttentionSpec, KVCacheSpec, Mixer, TensorSpec, make_part
+from pyre_amd.parts.linear import Linear, linear_specs
+
+
+class Attention(Mixer):
+    """q, k, v = split(h Wqkv^T + b); rotate q, k; store k, v; out = softmax(q k^T scale) v; out Wo^T.
+
+    The three projections are one product over the row-wise concatenation
+    [Wq; Wk; Wv] (made at bind time). Query head i reads key/value head
+    i // (num_heads / num_kv_heads) (`pyre/model.py:66-72`).
+    """
+
+    def __init__(self, spec: AttentionSpec):
+        if spec.num_heads % spec.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        self.spec = spec
+        self.position = make_part("position", spec.position)
+        self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
+        self.q_dim = spec.num_heads * spec.head_dim
+        self.kv_dim = spec.num_kv_heads * spec.head_dim
+        self.qkv = Linear(spec.hidden_size, self.q_dim + 2 * self.kv_dim, "attn.qkv")
+        self.out = Linear(self.q_dim, spec.hidden_size, "attn.out")
+
+    def cache_spec(self):
+        s = self.spec
+        return KVCacheSpec(s.num_kv_heads, s.head_dim, s.window)
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s, p = self.spec, self.spec.prefix
+        return (linear_specs(f"{p}.q_proj", self.q_dim, s.hidden_size, s.qkv_bias)
+                + linear_specs(f"{p}.k_proj", self.kv_dim, s.hidden_size, s.qkv_bias)
+                + linear_specs(f"{p}.v_proj", self.kv_dim, s.hidden_size, s.qkv_bias)
+                + linear_specs(f"{p}.o_proj", s.hidden_size, self.q_dim, s.out_bias))
+
+    def bind(self, tensors, runtime) -> None:
+        p = self.spec.prefix
+        w = torch.cat([tensors[f"{p}.{n}_proj.weight"] for n in "qkv"], dim=0)
+        b = None
+        if self.spec.qkv_bias:
+            b = torch.cat([tensors[f"{p}.{n}_proj.bias"] for n in "qkv"], dim=0)
+        self.qkv.set(w, b)
+        self.out.set(tensors[f"{p}.o_proj.weight"], tensors.get(f"{p}.o_proj.bias") if self.spec.out_bias else None)
+
+    def forward(self, ctx, h, cache):
+        s, n, ws = self.spec, ctx.n_tokens, ctx.workspace
+        qkv = self.qkv.forward(ctx, h, n)
+        q = ws.get("attn.q", (n, self.q_dim), ctx.dtype)
+        cos, sin, rot = self.position.rotary(ctx.runtime)
+        ops.rope_kv_write(qkv, q, cache.k if cache.writes else None, cache.v if cache.writes else None,
+                          cos, sin, rot, ctx.positions, cache.slots, n, s.num_heads, s.num_kv_heads,
+                          s.head_dim, cache.page_size)
+        o = ws.get("attn.o", (n, self.q_dim), ctx.dtype)
+        if not fast.attention(self, ctx, q, o, cache):
+            ops.attn_generic(q, o, cache.k, cache.v, ctx.positions, ctx.seq_of_token, cache.table, n,
+                             s.num_heads, s.num_kv_heads, s.head_dim, cache.page_size, self.scale,
+                             cache.window)
+        return self.out.forward(ctx, o, n)

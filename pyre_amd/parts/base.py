@@ -1,0 +1,245 @@
+"""What a model is made of: the kinds of parts, what each must provide, and the
+table that maps a part's description to the class that runs it.
+
+A model is described by data (:class:`ModelSpec`): an embedding, a list of layer
+descriptions (each naming its mixer, feed-forward, norms and their arrangement),
+the order in which layers run, a final norm and an output head. Each description
+is a small dataclass with a ``kind``; ``register_part(role, kind, cls)`` says which
+class runs it. No part knows which model it is in: it sees its own description,
+its own tensors and the step's :class:`~pyre_amd.engine.context.StepContext`.
+
+Interfaces (duck-typed; the base classes document them):
+
+``Part``          ``tensor_specs()`` names the checkpoint tensors it needs;
+                  ``bind(tensors, runtime)`` takes them (already on the device).
+``Mixer``         ``cache_spec()`` says what it keeps per token (pages of keys and
+                  values, all or a window) or per request (fixed-size state), or
+                  nothing; ``forward(ctx, h, cache) -> Partials`` turns the normed
+                  hidden rows into the term to be added to the residual stream.
+``FeedForward``   ``forward(ctx, h) -> Partials``.
+``Norm``          ``forward(ctx, resid, delta, out, rows=None)``: adds ``delta`` to the
+                  fp32 residual stream and writes the normed rows to ``out``.
+``PositionEncoding``  ``rotary(runtime) -> (cos, sin, rotary_dim)`` tables indexed by
+                  absolute position for mixers that rotate queries and keys, or
+                  ``rotary_dim = 0`` for none.
+``Block``         ``forward(ctx, state, cache)`` arranges the four above around the
+                  residual stream.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, ClassVar
+
+# --------------------------------------------------------------------------- tensors
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """One checkpoint tensor a part needs.
+
+    ``init`` tells the random-weights mode how to draw it: ``"normal"`` (matrices,
+    embeddings, biases: N(0, std)), ``"gain"`` (norm gains: 1 + N(0, gain_std)),
+    ``"zeros"``, ``"int"`` (integer tables: zeros).
+    ``alias_of`` names a tensor that stands in when this one is absent from the
+    file (a tied output head).
+    """
+
+    name: str
+    shape: tuple[int, ...]
+    init: str = "normal"
+    alias_of: str | None = None
+
+
+# --------------------------------------------------------------------------- cache needs
+
+
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Keys and values per token, in pages. ``window`` = 0 keeps every key;
+    ``window`` = W keeps the last W (a query at position p sees p-W+1 .. p)."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+    kind: ClassVar[str] = "kv"
+
+
+@dataclass(frozen=True)
+class StateCacheSpec:
+    """A fixed-size state per request: ``shape`` elements of ``dtype`` ("float32" or
+    "model" for the engine's element type), zeroed when a request starts."""
+
+    shape: tuple[int, ...]
+    dtype: str = "float32"
+
+    kind: ClassVar[str] = "state"
+
+
+# --------------------------------------------------------------------------- part classes
+
+
+class Part:
+    """Base of everything that owns tensors."""
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return []
+
+    def bind(self, tensors: dict[str, Any], runtime: Any) -> None:
+        """Take the tensors named by ``tensor_specs`` out of ``tensors``."""
+
+
+class Mixer(Part):
+    def cache_spec(self) -> KVCacheSpec | StateCacheSpec | None:
+        return None
+
+    def forward(self, ctx, h, cache):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, h):
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, ctx, resid, delta, out, rows=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary(self, runtime):
+        return None, None, 0
+
+
+# --------------------------------------------------------------------------- registry of parts
+
+_PARTS: dict[tuple[str, str], type] = {}
+ROLES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+
+
+def register_part(role: str, kind: str, cls: type) -> None:
+    if role not in ROLES:
+        raise ValueError(f"unknown role {role!r}; roles are {ROLES}")
+    _PARTS[(role, kind)] = cls
+
+
+def make_part(role: str, spec: Any, **kw: Any):
+    """Build the part that ``spec`` (a dataclass with a ``kind``) describes."""
+    _load_builtin_parts()
+    kind = getattr(spec, "kind", None)
+    try:
+        cls = _PARTS[(role, kind)]
+    except KeyError:
+        known = sorted(k for r, k in _PARTS if r == role)
+        raise ValueError(f"no {role} of kind {kind!r} is registered; known: {known}") from None
+    return cls(spec, **kw)
+
+
+def _load_builtin_parts() -> None:
+    import pyre_amd.parts.builtin  # noqa: F401
+
+
+# --------------------------------------------------------------------------- descriptions
+
+
+@dataclass(frozen=True)
+class RMSNormSpec:
+    hidden_size: int
+    eps: float
+    prefix: str                      #: tensor name is ``prefix + ".weight"``
+    kind: ClassVar[str] = "rmsnorm"
+
+
+@dataclass(frozen=True)
+class RotarySpec:
+    """Half-split rotary positions: element j pairs with j + rotary_dim/2."""
+
+    head_dim: int
+    theta: float
+    max_positions: int
+    rotary_dim: int | None = None    #: None: the whole head
+    kind: ClassVar[str] = "rotary"
+
+
+@dataclass(frozen=True)
+class NoPositionSpec:
+    kind: ClassVar[str] = "none"
+
+
+@dataclass(frozen=True)
+class AttentionSpec:
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    position: Any                    #: a position-encoding description
+    prefix: str                      #: e.g. "model.layers.0.self_attn"
+    qkv_bias: bool = True
+    out_bias: bool = False
+    window: int = 0                  #: 0: every earlier key is visible
+    scale: float | None = None       #: None: head_dim ** -0.5
+    kind: ClassVar[str] = "attention"
+
+
+@dataclass(frozen=True)
+class SwiGLUSpec:
+    hidden_size: int
+    intermediate_size: int
+    prefix: str                      #: e.g. "model.layers.0.mlp"
+    kind: ClassVar[str] = "swiglu"
+
+
+@dataclass(frozen=True)
+class BlockSpec:
+    """x += mixer(norm(x)); x += feed_forward(norm(x))   (pre-norm residual block)."""
+
+    mixer: Any
+    mixer_norm: Any
+    feed_forward: Any
+    feed_forward_norm: Any
+    kind: ClassVar[str] = "pre_norm"
+
+
+@dataclass(frozen=True)
+class EmbeddingSpec:
+    vocab_size: int
+    hidden_size: int
+    name: str = "model.embed_tokens.weight"
+    kind: ClassVar[str] = "embedding"
+
+
+@dataclass(frozen=True)
+class LMHeadSpec:
+    vocab_size: int
+    hidden_size: int
+    name: str = "lm_head.weight"
+    tied_to: str | None = None       #: embedding tensor used when the head is tied
+    kind: ClassVar[str] = "lm_head"
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    """One entry of the order in which layers run.
+
+    ``layer`` indexes ``ModelSpec.layers`` (a layer may be named more than once).
+    ``cache_from`` = j lets this call's mixer read the cache that the j-th entry
+    of the order wrote, instead of keeping one of its own.
+    """
+
+    layer: int
+    cache_from: int | None = None
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    max_positions: int
+    embedding: Any
+    layers: tuple[Any, ...]
+    schedule: tuple[LayerCall, ...]
+    final_norm: Any
+    head: Any
+    extra: dict = field(default_factory=dict, compare=False)

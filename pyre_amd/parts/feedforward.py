@@ -1,0 +1,36 @@
+"""SwiGLU feed-forward: down(silu(gate(x)) * up(x)), no biases (`pyre/model.py:128-139`)."""
+
+from __future__ import annotations
+
+import torch
+
+from pyre_amd.hip import ops
+from pyre_amd.parts.base import FeedForward, SwiGLUSpec, TensorSpec
+from pyre_amd.parts.linear import Linear, linear_specs
+
+
+class SwiGLU(FeedForward):
+    """gate and up are one product over [Wgate; Wup]; the SiLU-gate reads its halves."""
+
+    def __init__(self, spec: SwiGLUSpec):
+        self.spec = spec
+        self.gate_up = Linear(spec.hidden_size, 2 * spec.intermediate_size, "ffn.gate_up")
+        self.down = Linear(spec.intermediate_size, spec.hidden_size, "ffn.down")
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s, p = self.spec, self.spec.prefix
+        return (linear_specs(f"{p}.gate_proj", s.intermediate_size, s.hidden_size, False)
+                + linear_specs(f"{p}.up_proj", s.intermediate_size, s.hidden_size, False)
+                + linear_specs(f"{p}.down_proj", s.hidden_size, s.intermediate_size, False))
+
+    def bind(self, tensors, runtime) -> None:
+        p = self.spec.prefix
+        self.gate_up.set(torch.cat([tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]], dim=0))
+        self.down.set(tensors[f"{p}.down_proj.weight"])
+
+    def forward(self, ctx, h):
+        n = ctx.n_tokens
+        gu = self.gate_up.forward(ctx, h, n)
+        act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)
+        ops.silu_mul(gu, act, n)
+        return self.down.forward(ctx, act, n)

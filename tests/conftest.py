@@ -1,0 +1,48 @@
+"""Shared fixtures: tiny model folders with random weights, made in a temporary folder."""
+
+from __future__ import annotations
+
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+for p in (str(ROOT), str(Path(__file__).resolve().parent)):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu); everything else runs on the CPU")
+
+
+#: The two tiny shapes differ in every size and option: layers, width, heads and
+#: groups, head size (16 / 12), feed-forward width, vocabulary, theta, eps, tied or
+#: untied head, gains of 1 or random.
+TINY = {
+    "tiny-a": dict(seed=0, std=0.02, gain_std=0.0),
+    "tiny-b": dict(seed=1, std=0.05, gain_std=0.1),
+}
+
+
+@pytest.fixture(scope="session")
+def model_dirs(tmp_path_factory):
+    """name -> folder with config.json + model.safetensors (bfloat16 weights)."""
+    from pyre_amd.config import preset
+    from pyre_amd.weights import write_random_model
+
+    out = {}
+    for name, kw in TINY.items():
+        d = tmp_path_factory.mktemp(name.replace("-", "_"))
+        write_random_model(d, preset(name), **kw)
+        out[name] = d
+    return out
+
+
+@pytest.fixture(scope="session")
+def plain_models(model_dirs):
+    """name -> (config dict, float64 weights) of the plain implementation."""
+    import plain_qwen2 as P
+
+    return {n: (P.read_config(d), P.read_weights(d)) for n, d in model_dirs.items()}

@@ -1,0 +1,134 @@
+"""The engine against the plain implementation: the same requests whole, with the
+last 32 tokens one by one, in portions of changing size, and mixed with other
+requests on so few pages that they are used again; in float32 and in bfloat16."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from helpers import TOL, cut, first_bad, make_engine, plain_logits, random_ids, replay
+
+pytestmark = pytest.mark.gpu
+
+CASES = [(m, d) for m in ("tiny-a", "tiny-b") for d in ("float32", "bfloat16")]
+LENGTHS = {"a": 97, "b": 64, "c": 33, "d": 150}
+
+
+def _requests(vocab):
+    return {r: random_ids(vocab, n, seed=ord(r) * 7 + n) for r, n in LENGTHS.items()}
+
+
+def _expected(plain, reqs, dtype):
+    rounding = torch.bfloat16 if dtype == "bfloat16" else None
+    return {r: plain_logits(plain, ids, rounding) for r, ids in reqs.items()}
+
+
+@pytest.fixture(scope="module")
+def engines(model_dirs):
+    cache = {}
+
+    def get(model, dtype, **kw):
+        key = (model, dtype, tuple(sorted(kw.items())))
+        if key not in cache:
+            cache[key] = make_engine(model_dirs[model], dtype, **kw)
+        return cache[key]
+
+    return get
+
+
+@pytest.mark.parametrize("model,dtype", CASES)
+def test_whole(model, dtype, engines, plain_models):
+    plain = plain_models[model]
+    reqs = _requests(plain[0]["vocab_size"])
+    eng = engines(model, dtype)
+    steps = [([(r, ids, list(range(len(ids))))], [r]) for r, ids in reqs.items()]
+    got = replay(eng, steps)
+    assert len(got) == sum(LENGTHS.values())
+    bad, worst = first_bad(got, _expected(plain, reqs, dtype), TOL[dtype])
+    assert bad is None, bad
+    eng.cache.check_invariants()
+    assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+@pytest.mark.parametrize("model,dtype", CASES)
+def test_tail_token_by_token(model, dtype, engines, plain_models):
+    plain = plain_models[model]
+    reqs = _requests(plain[0]["vocab_size"])
+    eng = engines(model, dtype)
+    steps = []
+    for r, ids in reqs.items():
+        head = len(ids) - 32
+        steps.append(([(r, ids[:head], [head - 1])], []))
+        for i in range(head, len(ids)):
+            steps.append(([(r, ids[i:i + 1], [0])], [r] if i == len(ids) - 1 else []))
+    got = replay(eng, steps)
+    bad, worst = first_bad(got, _expected(plain, reqs, dtype), TOL[dtype])
+    assert bad is None, bad
+    assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+@pytest.mark.parametrize("model,dtype", CASES)
+def test_ragged_portions(model, dtype, engines, plain_models):
+    plain = plain_models[model]
+    reqs = _requests(plain[0]["vocab_size"])
+    eng = engines(model, dtype)
+    steps = []
+    for r, ids in reqs.items():
+        pos = 0
+        portions = cut(len(ids), [17, 5, 2, 32, 3, 2, 21])
+        for k, n in enumerate(portions):
+            steps.append(([(r, ids[pos:pos + n], list(range(n)))], [r] if k == len(portions) - 1 else []))
+            pos += n
+    got = replay(eng, steps)
+    assert len(got) == sum(LENGTHS.values())
+    bad, worst = first_bad(got, _expected(plain, reqs, dtype), TOL[dtype])
+    assert bad is None, bad
+
+
+@pytest.mark.parametrize("model,dtype", CASES)
+def test_mixed_with_page_reuse(model, dtype, engines, plain_models):
+    """Up to four live requests; portions of some beside decoded tokens of others.
+    The pool holds 20 pages (320 tokens) while the requests need 24 in total, so
+    later requests get pages that earlier ones gave back."""
+    plain = plain_models[model]
+    vocab = plain[0]["vocab_size"]
+    lengths = {"p": 70, "q": 45, "r": 100, "s": 38, "t": 66, "u": 51}
+    reqs = {r: random_ids(vocab, n, seed=n) for r, n in lengths.items()}
+    eng = engines(model, dtype, max_cached_tokens=320)
+    order = list(reqs)
+    fed = {r: 0 for r in reqs}
+    prefill_until = {r: lengths[r] - 12 for r in reqs}   # then one token at a time
+    live, waiting, steps = [], order[:], []
+    k = 0
+    while live or waiting:
+        def pages(r, extra):
+            return -(-(fed[r] + extra) // 16)
+        while waiting and len(live) < 4:
+            # admit only if the whole request fits beside the live ones
+            need = sum(-(-lengths[r] // 16) for r in live) + -(-lengths[waiting[0]] // 16)
+            if need > 20:
+                break
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            ids = reqs[r]
+            if fed[r] < prefill_until[r]:
+                n = min([9, 23, 2, 14][k % 4], prefill_until[r] - fed[r])
+                if prefill_until[r] - fed[r] - n == 1:
+                    n += 1
+            else:
+                n = 1
+            k += 1
+            entries.append((r, ids[fed[r]:fed[r] + n], list(range(n))))
+            fed[r] += n
+            if fed[r] == lengths[r]:
+                end.append(r)
+        steps.append((entries, end))
+        live = [r for r in live if r not in end]
+    got = replay(eng, steps)
+    assert len(got) == sum(lengths.values())
+    bad, worst = first_bad(got, _expected(plain, reqs, dtype), TOL[dtype])
+    assert bad is None, bad
+    eng.cache.check_invariants()
+    assert eng.cache.page_groups[0].allocator.num_used == 0
