@@ -1,0 +1,38 @@
+"""Next tokens from logits on the device: argmax, or inverse-CDF sampling."""
+
+from __future__ import annotations
+
+import torch
+
+from pyre_amd.hip import ops
+
+
+class Sampler:
+    """One call per step: all rows at once, one small upload, one small download."""
+
+    def __init__(self, device: torch.device, max_rows: int):
+        self.device = device
+        self.max_rows = max_rows
+        self._host = torch.empty(2 * max_rows, dtype=torch.float32, pin_memory=True)
+        self._dev = torch.empty(2 * max_rows, dtype=torch.float32, device=device)
+        self._ids = torch.empty(max_rows, dtype=torch.int32, device=device)
+        self._ids_host = torch.empty(max_rows, dtype=torch.int32, pin_memory=True)
+
+    def sample(self, logits: torch.Tensor, temperatures: list[float], uniforms: list[float]) -> list[int]:
+        """logits: float32 [M, V] on the device. Row i: argmax if temperatures[i]
+        is 0, else the first token whose cumulative probability under
+        softmax(logits / T) exceeds uniforms[i]."""
+        m = logits.shape[0]
+        if m > self.max_rows or len(temperatures) != m or len(uniforms) != m:
+            raise ValueError("sampler: row counts do not fit")
+        with torch.cuda.device(self.device):
+            ids = self._ids[:m]
+            ops.argmax(logits, ids)
+            if any(t > 0 for t in temperatures):
+                self._host[:m] = torch.tensor(temperatures, dtype=torch.float32)
+                self._host[m:2 * m] = torch.tensor(uniforms, dtype=torch.float32)
+                self._dev[:2 * m].copy_(self._host[:2 * m], non_blocking=True)
+                ops.sample(logits, self._dev[:m], self._dev[m:2 * m], ids)
+            self._ids_host[:m].copy_(ids, non_blocking=True)
+            torch.cuda.current_stream().synchronize()
+        return self._ids_host[:m].tolist()
