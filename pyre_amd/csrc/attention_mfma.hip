@@ -1,0 +1,384 @@
+// bfloat16 attention over the paged cache on the matrix cores (MFMA 16x16x32),
+// for head sizes that are multiples of 32 up to 256 and page sizes that are
+// multiples of 16. Two kernels share one inner loop:
+//
+//   attn_decode_kernel   one new token per request; the keys of a request are
+//                        split over many waves, each writing a partial
+//                        (max, sum, unnormalised output) that attn_decode_reduce
+//                        merges. One wave serves up to 16 query heads that share
+//                        a key/value head, so K and V are read once per group.
+//   attn_prefill_kernel  portions of prompts: a wave takes 32 consecutive tokens
+//                        of one request and one query head; the four waves of a
+//                        block take four heads of one key/value head, so their
+//                        K/V reads hit the same cache lines.
+//
+// Both compute the transposed problem so that no operand needs a transpose:
+//   S^T[key, col]  = K[key, :] . Q[col, :]          A = K rows (cache, as stored)
+//   O^T[d, col]   += V^T[d, key] P^T[key, col]      A = V^T rows (cache stores V
+//                                                       transposed), B = P^T, which
+//                                                       is exactly the register
+//                                                       layout S^T comes out in.
+// A "column" is a query head (decode) or a token (prefill). Scores, softmax and
+// the output accumulators are fp32 (pyre/model.py:109-123; the reference's own
+// decode kernel is pyre/kernels/paged_attn.py:26-71).
+#include <type_traits>
+
+#include "pyre_api.h"
+#include "pyre_common.h"
+
+using namespace pyre;
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kChunk = 32;  // keys per iteration: two MFMA row tiles
+
+__device__ inline bf16x8 load_b128(const bf16* p) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ inline bf16x8 zero_b128() {
+  uint4 z = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8, z);
+}
+__device__ inline uint32_t pack2(float lo, float hi) {
+  return static_cast<uint32_t>(bf16_bits(lo)) | (static_cast<uint32_t>(bf16_bits(hi)) << 16);
+}
+
+// Addressing of one request's keys and values for one key/value head.
+struct KV {
+  const bf16* k;     // layer slab [pages, nkv, page_size, HD]
+  const bf16* v;     // layer slab [pages, nkv, HD, page_size]
+  const int* table;  // the request's block table
+  int nkv, kvh, page_size;
+};
+
+// Per-column causal window: column c sees keys in [lo[c], hi[c]].
+template <int CT>
+struct Bounds {
+  int lo[CT], hi[CT];
+};
+
+// One chunk of 32 keys starting at key0 for CT tiles of 16 columns.
+//   q[ct][c]   B operands of Q^T, c = 32-wide slice of the head
+//   o[dt][ct]  accumulators of O^T, dt = 16-wide slice of the head
+//   m, l       running max (in log2 units) and sum of each lane's column
+// `edge` says that some key of the chunk may be masked for some column or lie in
+// a page that is not there; interior chunks skip all masking.
+template <int HD, int CT>
+__device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bounds<CT>& bd,
+                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
+                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  int page[2], off[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int k0 = key0 + 16 * t;
+    page[t] = kv.table[k0 / kv.page_size];
+    off[t] = k0 % kv.page_size;
+  }
+
+  // S^T tiles: rows = keys key0 + 16 t + (4 g + j), columns = lane's column r.
+  f32x4 s[2][CT];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) s[t][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (page[t] < 0) continue;  // released or never allocated: every key of it is masked
+    const bf16* kp = kv.k + ((static_cast<size_t>(page[t]) * kv.nkv + kv.kvh) * kv.page_size + off[t] + r) * HD + 8 * g;
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c) {
+      const bf16x8 a = load_b128(kp + 32 * c);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        s[t][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[ct][c], s[t][ct], 0, 0, 0);
+    }
+  }
+
+  // Online softmax per column; P^T packed as the B operand of the second product:
+  // slots 0..3 of a lane are keys 4g..4g+3 of tile 0, slots 4..7 those of tile 1.
+  bf16x8 p[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    float x[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v = s[t][ct][j] * scale_log2;
+        if (edge) {
+          const int key = key0 + 16 * t + 4 * g + j;
+          if (page[t] < 0 || key < bd.lo[ct] || key > bd.hi[ct]) v = -INFINITY;
+        }
+        x[4 * t + j] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m[ct], mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // column without a visible key so far
+    const float alpha = __builtin_amdgcn_exp2f(m[ct] - m_use);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x[i] = __builtin_amdgcn_exp2f(x[i] - m_use);
+      sum += x[i];
+    }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    l[ct] = l[ct] * alpha + sum;
+    m[ct] = m_new;
+    uint4 u = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+    p[ct] = __builtin_bit_cast(bf16x8, u);
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) o[dt][ct] *= alpha;
+  }
+
+  // O^T += V^T P^T. Row of the A operand = output element d; its 8 slots are the
+  // same keys as P^T's: two runs of four keys, 8 bytes each in the transposed cache.
+  const bf16* vp[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+    vp[t] = page[t] < 0 ? nullptr
+                        : kv.v + ((static_cast<size_t>(page[t]) * kv.nkv + kv.kvh) * HD + r) * kv.page_size + off[t] + 4 * g;
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) {
+    uint2 h[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      h[t] = uint2{0u, 0u};
+      if (vp[t]) h[t] = *reinterpret_cast<const uint2*>(vp[t] + static_cast<size_t>(dt) * 16 * kv.page_size);
+    }
+    const uint4 u = {h[0].x, h[0].y, h[1].x, h[1].y};
+    const bf16x8 a = __builtin_bit_cast(bf16x8, u);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+      o[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p[ct], o[dt][ct], 0, 0, 0);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Decode: grid (ceil(nsplits / 4), nkv * qtiles, tokens), 4 waves = 4 splits.
+// ---------------------------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    const int* __restrict__ tokens, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int nq, int nkv, int page_size,
+    float scale_log2, int window, int nsplits) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int split = blockIdx.x * 4 + wave;
+  if (split >= nsplits) return;
+  const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
+  const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
+  const int head0 = kvh * n_rep + qt * 16, nheads = min(16, n_rep - qt * 16);
+  const int idx = blockIdx.z, tok = tokens[idx];
+  const int pos = positions[tok];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+
+  KV kv{k_cache, v_cache, block_table + static_cast<size_t>(seq_of_token[tok]) * table_stride, nkv, kvh, page_size};
+  Bounds<1> bd{{lo}, {pos}};
+
+  bf16x8 qr[1][HD / 32];
+#pragma unroll
+  for (int c = 0; c < HD / 32; ++c)
+    qr[0][c] = r < nheads ? load_b128(q + (static_cast<size_t>(tok) * nq + head0 + r) * HD + 32 * c + 8 * g) : zero_b128();
+
+  f32x4 o[HD / 16][1];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) o[dt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m[1] = {-INFINITY}, l[1] = {0.f};
+
+  const int first = lo / kChunk, last = pos / kChunk;
+  const int per = (last - first + 1 + nsplits - 1) / nsplits;
+  const int begin = first + split * per, end = min(last + 1, begin + per);
+  for (int c = begin; c < end; ++c)
+    attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
+
+  if (r < nheads) {
+    const size_t slot = (static_cast<size_t>(idx) * nq + head0 + r) * nsplits + split;
+    if (g == 0) {
+      part_ml[2 * slot] = m[0];
+      part_ml[2 * slot + 1] = l[0];
+    }
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt)
+      *reinterpret_cast<f32x4*>(part_acc + slot * HD + dt * 16 + 4 * g) = o[dt][0];
+  }
+}
+
+// out[token, head, :] = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s.
+template <int HD>
+__global__ void attn_decode_reduce(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                   const int* __restrict__ tokens, bf16* __restrict__ out, int nq,
+                                   int nsplits) {
+  const int idx = blockIdx.x, head = blockIdx.y;
+  const size_t base = (static_cast<size_t>(idx) * nq + head) * nsplits;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplits; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
+  float L = 0.f;
+  for (int s = 0; s < nsplits; ++s) {
+    const float ms = part_ml[2 * (base + s)];
+    if (ms != -INFINITY) L += part_ml[2 * (base + s) + 1] * __builtin_amdgcn_exp2f(ms - M);
+  }
+  const int tok = tokens[idx];
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < nsplits; ++s) {
+      const float ms = part_ml[2 * (base + s)];
+      if (ms != -INFINITY) acc += part_acc[(base + s) * HD + d] * __builtin_amdgcn_exp2f(ms - M);
+    }
+    out[(static_cast<size_t>(tok) * nq + head) * HD + d] = from_float<bf16>(acc / L);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Prefill: grid (tiles, nkv * head groups); wave w takes head group*4 + w.
+// tiles[i] = (first token of the tile in the flat batch, number of tokens <= 32).
+// ---------------------------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
+    int nq, int nkv, int page_size, float scale_log2, int window) {
+  constexpr int CT = 2;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
+  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int hin = hg * 4 + wave;
+  if (hin >= n_rep) return;
+  const int head = kvh * n_rep + hin;
+  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+  const int pos0 = positions[t0];
+
+  KV kv{k_cache, v_cache, block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride, nkv, kvh, page_size};
+  Bounds<CT> bd;
+  bf16x8 qr[CT][HD / 32];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = 16 * ct + r;
+    const bool live = col < ntok;
+    // A column past the tile's end computes on zeros over the first column's keys
+    // and is not stored.
+    bd.hi[ct] = live ? pos0 + col : pos0;
+    bd.lo[ct] = window > 0 ? max(0, bd.hi[ct] - window + 1) : 0;
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c)
+      qr[ct][c] = live ? load_b128(q + (static_cast<size_t>(t0 + col) * nq + head) * HD + 32 * c + 8 * g) : zero_b128();
+  }
+  f32x4 o[HD / 16][CT];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) o[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m[CT], l[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) { m[ct] = -INFINITY; l[ct] = 0.f; }
+
+  const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int hi_all = pos0 + ntok - 1;
+  const int first = lo_all / kChunk, last = hi_all / kChunk;
+  // A chunk is interior when every key of it is visible to every column: it ends
+  // at or before the first token's position and starts at or after the highest
+  // lower bound of the tile.
+  const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
+  for (int c = first; c <= last; ++c) {
+    const int key0 = c * kChunk;
+    const bool edge = key0 + kChunk - 1 > pos0 || key0 < lo_max;
+    attend_chunk<HD, CT>(kv, key0, edge, bd, scale_log2, qr, o, m, l);
+  }
+
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = 16 * ct + r;
+    if (col >= ntok) continue;
+    const float inv = 1.f / l[ct];
+    bf16* dst = out + (static_cast<size_t>(t0 + col) * nq + head) * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      const f32x4 v = o[dt][ct];
+      *reinterpret_cast<uint2*>(dst + dt * 16) = uint2{pack2(v[0] * inv, v[1] * inv), pack2(v[2] * inv, v[3] * inv)};
+    }
+  }
+}
+
+template <typename F>
+int dispatch_head(int hd, F&& f) {
+  switch (hd) {
+    case 32: f(std::integral_constant<int, 32>()); return 0;
+    case 64: f(std::integral_constant<int, 64>()); return 0;
+    case 96: f(std::integral_constant<int, 96>()); return 0;
+    case 128: f(std::integral_constant<int, 128>()); return 0;
+    case 160: f(std::integral_constant<int, 160>()); return 0;
+    case 192: f(std::integral_constant<int, 192>()); return 0;
+    case 224: f(std::integral_constant<int, 224>()); return 0;
+    case 256: f(std::integral_constant<int, 256>()); return 0;
+  }
+  return 1;
+}
+
+}  // namespace
+
+extern "C" int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv) {
+  return hd >= 32 && hd <= 256 && hd % 32 == 0 && page_size > 0 && page_size % 16 == 0 && nkv > 0 &&
+         nq % nkv == 0;
+}
+
+extern "C" int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache,
+                                     const void* v_cache, const int* tokens, int n_tokens,
+                                     const int* positions, const int* seq_of_token,
+                                     const int* block_table, int table_stride, float* part_acc,
+                                     float* part_ml, int nsplits, int nq, int nkv, int hd,
+                                     int page_size, float scale, int window, hipStream_t stream) {
+  PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
+               "attn_decode_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
+               "heads %d/%d are not supported", hd, page_size, nq, nkv);
+  PYRE_REQUIRE(nsplits >= 1 && table_stride > 0, "attn_decode_bf16: bad split count or table");
+  if (n_tokens <= 0) return 0;
+  const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
+  PYRE_REQUIRE(n_tokens <= 65535 && nkv * qtiles <= 65535, "attn_decode_bf16: grid too large");
+  const dim3 grid((nsplits + 3) / 4, nkv * qtiles, n_tokens);
+  const float scale_log2 = scale * kLog2e;
+  const int rc = dispatch_head(hd, [&](auto HDc) {
+    constexpr int HD = decltype(HDc)::value;
+    hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
+                       static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), tokens,
+                       positions, seq_of_token, block_table, table_stride, part_acc, part_ml, nq, nkv,
+                       page_size, scale_log2, window, nsplits);
+    hipLaunchKernelGGL(attn_decode_reduce<HD>, dim3(n_tokens, nq), dim3(HD <= 64 ? 64 : 128), 0, stream,
+                       part_acc, part_ml, tokens, static_cast<bf16*>(out), nq, nsplits);
+  });
+  PYRE_REQUIRE(rc == 0, "attn_decode_bf16: no kernel for head_dim %d", hd);
+  return check_launch("attn_decode_bf16");
+}
+
+extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache,
+                                      const void* v_cache, const int* tiles, int n_tiles,
+                                      const int* positions, const int* seq_of_token,
+                                      const int* block_table, int table_stride, int nq, int nkv,
+                                      int hd, int page_size, float scale, int window,
+                                      hipStream_t stream) {
+  PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
+               "attn_prefill_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
+               "heads %d/%d are not supported", hd, page_size, nq, nkv);
+  PYRE_REQUIRE(table_stride > 0, "attn_prefill_bf16: bad table");
+  if (n_tiles <= 0) return 0;
+  const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
+  PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
+  const dim3 grid(n_tiles, nkv * hgroups);
+  const float scale_log2 = scale * kLog2e;
+  const int rc = dispatch_head(hd, [&](auto HDc) {
+    constexpr int HD = decltype(HDc)::value;
+    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
+                       static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache),
+                       static_cast<bf16*>(out), tiles, positions, seq_of_token, block_table, table_stride,
+                       nq, nkv, page_size, scale_log2, window);
+  });
+  PYRE_REQUIRE(rc == 0, "attn_prefill_bf16: no kernel for head_dim %d", hd);
+  return check_launch("attn_prefill_bf16");
+}

@@ -42,6 +42,25 @@ int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                       int nq, int nkv, int hd, int page_size, float scale, int window,
                       hipStream_t stream);
 
+// 1 if the MFMA attention kernels take this geometry (else use pyre_attn_generic).
+int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv);
+
+// One new token per request. tokens[i] indexes the flat batch; part_acc is
+// [n_tokens, nq, nsplits, hd] floats and part_ml [n_tokens, nq, nsplits, 2] of scratch.
+int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                          const int* tokens, int n_tokens, const int* positions,
+                          const int* seq_of_token, const int* block_table, int table_stride,
+                          float* part_acc, float* part_ml, int nsplits, int nq, int nkv, int hd,
+                          int page_size, float scale, int window, hipStream_t stream);
+
+// Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
+// all tokens of a tile from one request at consecutive positions.
+int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                           const int* tiles, int n_tiles, const int* positions,
+                           const int* seq_of_token, const int* block_table, int table_stride,
+                           int nq, int nkv, int hd, int page_size, float scale, int window,
+                           hipStream_t stream);
+
 int pyre_argmax(const float* logits, long row_stride, int* out, int m, int vocab,
                 hipStream_t stream);
 

@@ -15,6 +15,9 @@ from dataclasses import dataclass, field
 import numpy as np
 
 
+TILE = 32  #: tokens of one request that the prompt-portion attention kernel takes at a time
+
+
 @dataclass
 class Entry:
     rid: object
@@ -39,6 +42,9 @@ class HostBatch:
     slots: list[np.ndarray]     #: per page group [N]: cache slot of each token
     tables: list[np.ndarray]    #: per page group [S, P]: block tables (-1: released or unused)
     max_q_len: int = 0
+    decode_tokens: np.ndarray = None   #: token indices of requests that bring one token
+    prefill_tiles: np.ndarray = None   #: [T, 2] (first token, count <= TILE) of the others, longest context first
+    max_decode_ctx: int = 0            #: longest context among the single-token requests
 
     @property
     def decode_only(self) -> bool:
@@ -94,7 +100,18 @@ def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: 
             tables[g][s, :len(tbl)] = tbl
         max_q = max(max_q, n)
     i32 = lambda x: np.asarray(x, dtype=np.int32)  # noqa: E731
+    decode_tokens, tiles, max_decode_ctx = [], [], 0
+    for s in range(len(entries)):
+        a, b = q_start[s], q_start[s + 1]
+        if b - a == 1:
+            decode_tokens.append(a)
+            max_decode_ctx = max(max_decode_ctx, ctx_len[s])
+        else:
+            tiles.extend((positions[t0] + min(TILE, b - t0), t0, min(TILE, b - t0)) for t0 in range(a, b, TILE))
+    tiles.sort(key=lambda t: -t[0])  # the tiles with the most keys start first
     return HostBatch(
+        decode_tokens=i32(decode_tokens), prefill_tiles=i32([t[1:] for t in tiles]).reshape(-1, 2),
+        max_decode_ctx=max_decode_ctx,
         n_tokens=len(tokens), n_seqs=len(entries), rids=[e.rid for e in entries], tokens=i32(tokens),
         positions=i32(positions), seq_of_token=i32(seq_of_token), q_start=i32(q_start),
         ctx_len=i32(ctx_len), state_slots=i32(state_slots), logit_rows=i32(logit_rows),

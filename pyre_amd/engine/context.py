@@ -67,8 +67,9 @@ def meta_layout(n_cap: int, s_cap: int, table_widths: list[int]) -> tuple[dict, 
         lay[name] = (off, n)
         off += (n + 3) // 4 * 4
 
-    for name in ("tokens", "positions", "seq_of_token", "logit_rows"):
+    for name in ("tokens", "positions", "seq_of_token", "logit_rows", "decode_tokens"):
         put(name, n_cap)
+    put("prefill_tiles", 2 * (n_cap // 32 + s_cap))
     put("q_start", s_cap + 1)
     put("ctx_len", s_cap)
     put("state_slots", s_cap)
@@ -111,6 +112,7 @@ class MetaBuffers:
         fill("tokens", hb.tokens), fill("positions", hb.positions), fill("seq_of_token", hb.seq_of_token)
         fill("logit_rows", hb.logit_rows), fill("q_start", hb.q_start), fill("ctx_len", hb.ctx_len)
         fill("state_slots", hb.state_slots)
+        fill("decode_tokens", hb.decode_tokens), fill("prefill_tiles", hb.prefill_tiles)
         for g, w in enumerate(widths):
             fill(f"slots{g}", hb.slots[g])
             o, _ = lay[f"table{g}"]
@@ -164,6 +166,8 @@ class StepContext:
     q_start: torch.Tensor
     ctx_len: torch.Tensor
     state_slots: torch.Tensor
+    decode_tokens: torch.Tensor = None   #: flat indices of the single-token requests' tokens
+    prefill_tiles: torch.Tensor = None   #: (first token, count) of the other requests' tiles
 
     @property
     def workspace(self) -> Workspace:

@@ -128,7 +128,8 @@ class Engine:
                 runtime=self.runtime, host=hb, n_tokens=hb.n_tokens, n_seqs=hb.n_seqs,
                 n_logits=len(hb.logit_rows), tokens=views["tokens"], positions=views["positions"],
                 seq_of_token=views["seq_of_token"], logit_rows=views["logit_rows"][:len(hb.logit_rows)],
-                q_start=views["q_start"], ctx_len=views["ctx_len"], state_slots=views["state_slots"])
+                q_start=views["q_start"], ctx_len=views["ctx_len"], state_slots=views["state_slots"],
+                decode_tokens=views["decode_tokens"], prefill_tiles=views["prefill_tiles"])
             logits = self.model.forward(ctx, self._layer_views(views))
         for e in entries:
             cache.commit(e.rid, len(e.tokens))

@@ -28,6 +28,9 @@ _SIGNATURES = {
     "pyre_reduce_partials": [P, I, I, L, P, I, P, I, I, I, P],
     "pyre_gemm_generic": [P, I, L, P, P, I, L, P, I, P, I, L, I, I, I, P],
     "pyre_attn_generic": [P, P, I, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+    "pyre_attn_mfma_supports": [I, I, I, I],
+    "pyre_attn_decode_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
+    "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_argmax": [P, L, P, I, I, P],
     "pyre_sample": [P, L, P, P, P, I, I, P],
 }

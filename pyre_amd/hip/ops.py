@@ -252,3 +252,48 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
     _i32("out", out, m)
     call("pyre_sample", logits.data_ptr(), logits.stride(0), temperature.data_ptr(), uniform.data_ptr(),
          out.data_ptr(), m, logits.shape[1], _stream())
+
+
+def attn_mfma_supports(hd: int, page_size: int, nq: int, nkv: int) -> bool:
+    from pyre_amd.hip.lib import lib
+
+    return bool(lib().pyre_attn_mfma_supports(hd, page_size, nq, nkv))
+
+
+def _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size):
+    _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table)
+    for name, t in (("q", q), ("out", out), ("k_cache", k_cache), ("v_cache", v_cache)):
+        if t.dtype != torch.bfloat16:
+            raise KernelError(f"attn (MFMA): {name} must be bfloat16")
+        _contig(name, t)
+    if tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
+        raise KernelError("attn (MFMA): cache shapes do not fit the head geometry")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("attn (MFMA): block table must be int32 [rows, pages]")
+    _i32("positions", positions), _i32("seq_of_token", seq_of_token)
+
+
+def attn_decode_bf16(q, out, k_cache, v_cache, tokens, n_tokens, positions, seq_of_token, block_table,
+                     part_acc, part_ml, nsplits, nq, nkv, hd, page_size, scale, window=0) -> None:
+    """Attention of ``n_tokens`` single new tokens (``tokens`` indexes the flat
+    batch) over the paged cache, keys split ``nsplits`` ways."""
+    _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
+    _i32("tokens", tokens, n_tokens)
+    if part_acc.dtype != torch.float32 or part_acc.numel() < n_tokens * nq * nsplits * hd:
+        raise KernelError("attn_decode: partial accumulators too small")
+    if part_ml.dtype != torch.float32 or part_ml.numel() < n_tokens * nq * nsplits * 2:
+        raise KernelError("attn_decode: partial max/sum buffer too small")
+    call("pyre_attn_decode_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         tokens.data_ptr(), n_tokens, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+         block_table.stride(0), part_acc.data_ptr(), part_ml.data_ptr(), nsplits, nq, nkv, hd, page_size,
+         float(scale), int(window), _stream())
+
+
+def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,
+                      nq, nkv, hd, page_size, scale, window=0) -> None:
+    """Attention of prompt portions; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32)."""
+    _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
+    _i32("tiles", tiles, 2 * n_tiles)
+    call("pyre_attn_prefill_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         tiles.data_ptr(), n_tiles, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+         block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), _stream())

@@ -23,19 +23,35 @@ def pytest_configure(config):
 TINY = {
     "tiny-a": dict(seed=0, std=0.02, gain_std=0.0),
     "tiny-b": dict(seed=1, std=0.05, gain_std=0.1),
+    "tiny-c": dict(seed=2, std=0.04, gain_std=0.05),
 }
+
+#: A third shape whose head size (32) and 16-token pages are taken by the MFMA
+#: attention kernels in bfloat16; three query heads per key/value head.
+TINY_C = {
+    "architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 80,
+    "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 32, "intermediate_size": 144,
+    "vocab_size": 777, "rope_theta": 5e4, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+    "max_position_embeddings": 1024,
+}
+
+
+def tiny_config(name):
+    from pyre_amd.config import preset
+    from pyre_amd.registry import config_from_dict
+
+    return config_from_dict(TINY_C) if name == "tiny-c" else preset(name)
 
 
 @pytest.fixture(scope="session")
 def model_dirs(tmp_path_factory):
     """name -> folder with config.json + model.safetensors (bfloat16 weights)."""
-    from pyre_amd.config import preset
     from pyre_amd.weights import write_random_model
 
     out = {}
     for name, kw in TINY.items():
         d = tmp_path_factory.mktemp(name.replace("-", "_"))
-        write_random_model(d, preset(name), **kw)
+        write_random_model(d, tiny_config(name), **kw)
         out[name] = d
     return out
 

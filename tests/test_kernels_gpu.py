@@ -1,0 +1,357 @@
+"""Each kernel alone against a plain torch reference of the same formula, at sizes
+other than the engine's tiny models (odd widths, many heads, long contexts,
+scrambled pages)."""
+
+from __future__ import annotations
+
+import math
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def _ops():
+    from pyre_amd.hip import ops
+
+    return ops
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+# ----------------------------------------------------------------------------- small kernels
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    ops = _ops()
+    table = rnd(301, 70, dtype=DT[dtype])
+    ids = i32([5, 300, 0, 17, 5])
+    out = torch.empty(5, 70, device=DEV)
+    ops.embed(table, ids, out)
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [70, 1000, 3584])
+def test_add_rmsnorm(dtype, hidden):
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+
+    n, eps = 7, 1e-5
+    resid = rnd(n, hidden, seed=1)
+    delta = rnd(3, n, hidden, seed=2)                      # three partial sums
+    bias = rnd(hidden, seed=3)
+    gain = rnd(hidden, seed=4, dtype=DT[dtype]) + 1
+    out = torch.empty(n, hidden, device=DEV, dtype=DT[dtype])
+    want_resid = resid.double() + delta.double().sum(0) + bias.double()
+    want = want_resid * torch.rsqrt(want_resid.pow(2).mean(-1, keepdim=True) + eps) * gain.double()
+    r = resid.clone()
+    ops.add_rmsnorm(r, Partials(delta, bias), gain, eps, out)
+    assert torch.allclose(r.double(), want_resid, atol=1e-5)
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert torch.allclose(out.double(), want, atol=tol, rtol=tol)
+    # library special case: no delta, unit gain -> torch's rms_norm
+    ones = torch.ones(hidden, device=DEV)
+    o32 = torch.empty(n, hidden, device=DEV)
+    ops.add_rmsnorm(resid.clone(), None, ones, eps, o32)
+    assert torch.allclose(o32, torch.nn.functional.rms_norm(resid, (hidden,), eps=eps), atol=1e-5)
+    # rows: only the listed rows, resid untouched
+    rows = i32([6, 2])
+    r2 = resid.clone()
+    o2 = torch.empty(2, hidden, device=DEV, dtype=DT[dtype])
+    ops.add_rmsnorm(r2, Partials(delta, bias), gain, eps, o2, rows=rows)
+    assert torch.equal(r2, resid)
+    assert torch.allclose(o2.double(), want[[6, 2]], atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("adt,wdt", [("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")])
+@pytest.mark.parametrize("m,n,k", [(1, 37, 50), (5, 130, 257), (77, 200, 64), (130, 65, 1000)])
+def test_gemm_generic(adt, wdt, m, n, k):
+    ops = _ops()
+    a = rnd(m, k, dtype=DT[adt], seed=1)
+    w = rnd(n, k, dtype=DT[wdt], seed=2)
+    bias = rnd(n, seed=3)
+    out = torch.empty(m, n, device=DEV)
+    ops.gemm_generic(a, w, bias, out, m)
+    want = a.double() @ w.double().T + bias.double()
+    assert torch.allclose(out.double(), want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
+    # linearity in the input, and bias alone for a zero input
+    out0 = torch.empty(m, n, device=DEV)
+    ops.gemm_generic(torch.zeros_like(a), w, bias, out0, m)
+    assert torch.allclose(out0, bias.expand(m, n))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_silu_mul(dtype):
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+
+    n, inter = 5, 176
+    gu = rnd(2, n, 2 * inter, seed=5, scale=3.0)
+    out = torch.empty(n, inter, device=DEV, dtype=DT[dtype])
+    ops.silu_mul(Partials(gu), out, n)
+    s = gu.double().sum(0)
+    want = torch.nn.functional.silu(s[:, :inter]) * s[:, inter:]
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert torch.allclose(out.double(), want, atol=tol, rtol=tol)
+
+
+# ----------------------------------------------------------------------------- rotary + cache write
+
+def rope_plain(x, pos, theta, rot):
+    """x [n, heads, hd]; half-split rotation of the first `rot` elements (pyre/model.py:41-63)."""
+    inv = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+    ang = torch.outer(pos.float(), inv)
+    cos, sin = ang.cos().double()[:, None, :], ang.sin().double()[:, None, :]
+    x = x.double().clone()
+    a, b = x[..., :rot // 2].clone(), x[..., rot // 2:rot].clone()
+    x[..., :rot // 2] = a * cos - b * sin
+    x[..., rot // 2:rot] = b * cos + a * sin
+    return x
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,hd,rot,page", [(4, 2, 16, 16, 16), (6, 3, 12, 12, 8), (5, 1, 40, 24, 4), (28, 4, 128, 128, 16)])
+def test_rope_kv_write(dtype, nq, nkv, hd, rot, page):
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+    from pyre_amd.parts.rotary import rotary_tables
+
+    n, theta, npages = 9, 1e4, 12
+    width = (nq + 2 * nkv) * hd
+    qkv = rnd(2, n, width, seed=7)
+    bias = rnd(width, seed=8)
+    pos = torch.tensor([0, 1, 2, 40, 41, 7, 100, 3, 64])
+    cos, sin = rotary_tables(rot, theta, 128)
+    slots = torch.tensor(random.Random(1).sample(range(npages * page), n))
+    slots[4] = -1                                           # this token is not stored
+    q = torch.empty(n, nq * hd, device=DEV, dtype=DT[dtype])
+    kc = torch.zeros(npages, nkv, page, hd, device=DEV, dtype=DT[dtype])
+    vc = torch.zeros(npages, nkv, hd, page, device=DEV, dtype=DT[dtype])
+    ops.rope_kv_write(Partials(qkv, bias), q, kc, vc, cos.to(DEV), sin.to(DEV), rot, i32(pos.tolist()),
+                      i32(slots.tolist()), n, nq, nkv, hd, page)
+    full = (qkv.double().sum(0) + bias.double()).cpu()
+    wq = rope_plain(full[:, :nq * hd].view(n, nq, hd), pos, theta, rot)
+    wk = rope_plain(full[:, nq * hd:(nq + nkv) * hd].view(n, nkv, hd), pos, theta, rot)
+    wv = full[:, (nq + nkv) * hd:].view(n, nkv, hd)
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert torch.allclose(q.double().cpu().view(n, nq, hd), wq, atol=tol, rtol=tol)
+    for t in range(n):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        p, o = divmod(s, page)
+        assert torch.allclose(kc[p, :, o, :].double().cpu(), wk[t], atol=tol, rtol=tol)
+        assert torch.allclose(vc[p, :, :, o].double().cpu(), wv[t], atol=tol, rtol=tol)
+    # nothing else was written: everything outside the used slots is still zero
+    used = {int(s) for s in slots if s >= 0}
+    for s in range(npages * page):
+        if s not in used:
+            p, o = divmod(s, page)
+            assert not kc[p, :, o, :].any() and not vc[p, :, :, o].any()
+    # position 0 is the identity
+    assert torch.allclose(q.double().cpu().view(n, nq, hd)[0], full[0, :nq * hd].view(nq, hd), atol=tol, rtol=tol)
+
+
+# ----------------------------------------------------------------------------- attention
+
+def paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dtype, seed=0, table_extra=2):
+    """Random requests whose keys and values lie in scrambled pages.
+    Returns the kernel's inputs and, per request, dense K/V and queries."""
+    rng = random.Random(seed)
+    S = len(ctx_lens)
+    npages_each = [-(-c // page) for c in ctx_lens]
+    total = sum(npages_each) + 5
+    order = list(range(total))
+    rng.shuffle(order)
+    width = max(8, -(-max(npages_each) // 8) * 8) + table_extra
+    table = torch.full((S, width), -1, dtype=torch.int32)
+
+    def cpu(*shape, seed):
+        return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)).to(dtype)
+
+    kc = cpu(total, nkv, page, hd, seed=seed + 1)                 # stale values everywhere
+    vc = cpu(total, nkv, hd, page, seed=seed + 2)
+    dense, qs, positions, seq_of = [], [], [], []
+    it = iter(order)
+    for s in range(S):
+        pages = [next(it) for _ in range(npages_each[s])]
+        table[s, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        K = cpu(ctx_lens[s], nkv, hd, seed=seed + 10 + s)
+        V = cpu(ctx_lens[s], nkv, hd, seed=seed + 50 + s)
+        for t in range(ctx_lens[s]):
+            kc[pages[t // page], :, t % page, :] = K[t]
+            vc[pages[t // page], :, :, t % page] = V[t]
+        dense.append((K, V))
+        ql = q_lens[s]
+        qs.append(cpu(ql, nq, hd, seed=seed + 90 + s))
+        positions += list(range(ctx_lens[s] - ql, ctx_lens[s]))
+        seq_of += [s] * ql
+    q = torch.cat(qs).contiguous().to(DEV)
+    return q, kc.to(DEV), vc.to(DEV), table.to(DEV), i32(positions), i32(seq_of), dense, qs
+
+
+def attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window=0):
+    """softmax(q k^T scale) v per request and head in float64 (pyre/model.py:109-123)."""
+    outs = []
+    for s, (K, V) in enumerate(dense):
+        ql, T = q_lens[s], ctx_lens[s]
+        q = qs[s].double().transpose(0, 1)                        # nq, ql, hd
+        k = K.double().transpose(0, 1).repeat_interleave(nq // nkv, 0)
+        v = V.double().transpose(0, 1).repeat_interleave(nq // nkv, 0)
+        sc = q @ k.transpose(-1, -2) * scale
+        qpos = torch.arange(T - ql, T, device=sc.device)[:, None]
+        kpos = torch.arange(T, device=sc.device)[None, :]
+        hide = kpos > qpos
+        if window:
+            hide = hide | (kpos < qpos - window + 1)
+        sc = sc.masked_fill(hide, -math.inf)
+        outs.append((torch.softmax(sc, -1) @ v).transpose(0, 1))   # ql, nq, hd
+    return torch.cat(outs)
+
+
+GENERIC_SHAPES = [(4, 2, 16, 16), (8, 2, 12, 8), (6, 6, 40, 4), (28, 4, 128, 16), (5, 1, 256, 32)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,hd,page", GENERIC_SHAPES)
+@pytest.mark.parametrize("window", [0, 37])
+def test_attn_generic(dtype, nq, nkv, hd, page, window):
+    ops = _ops()
+    ctx_lens, q_lens = [1, 33, 300, 1500, 64], [1, 5, 1, 40, 64]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, DT[dtype])
+    out = torch.empty_like(q)
+    scale = hd ** -0.5
+    ops.attn_generic(q, out, kc, vc, pos, seq_of, table, q.shape[0], nq, nkv, hd, page, scale, window)
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    assert torch.allclose(out.double().cpu(), want, atol=tol, rtol=tol)
+    if window == 0:
+        # one visible key: the output is exactly that key's value (request 0)
+        assert torch.allclose(out[0].double().cpu(), dense[0][1][0].double().repeat_interleave(nq // nkv, 0), atol=tol)
+
+
+MFMA_SHAPES = [(28, 4, 128, 16), (8, 8, 64, 16), (6, 1, 32, 32), (40, 2, 96, 16), (3, 1, 256, 48)]
+
+
+@pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 50])
+@pytest.mark.parametrize("nsplits", [1, 3, 16])
+def test_attn_decode_mfma(nq, nkv, hd, page, window, nsplits):
+    ops = _ops()
+    assert ops.attn_mfma_supports(hd, page, nq, nkv)
+    ctx_lens = [1, 31, 32, 33, 700, 2049]
+    q_lens = [1] * len(ctx_lens)
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=3)
+    n = q.shape[0]
+    out = torch.full_like(q, float("nan"))
+    acc = torch.empty(n * nq * nsplits * hd, device=DEV)
+    ml = torch.empty(n * nq * nsplits * 2, device=DEV)
+    toks = i32(list(range(n)))
+    scale = hd ** -0.5
+    ops.attn_decode_bf16(q, out, kc, vc, toks, n, pos, seq_of, table, acc, ml, nsplits, nq, nkv, hd, page, scale, window)
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 50])
+def test_attn_prefill_mfma(nq, nkv, hd, page, window):
+    ops = _ops()
+    from pyre_amd.engine.batch import TILE
+
+    ctx_lens, q_lens = [2, 40, 97, 700, 1100], [2, 40, 33, 3, 600]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=4)
+    out = torch.full_like(q, float("nan"))
+    tiles, base = [], 0
+    for ql in q_lens:
+        tiles += [(t0, min(TILE, base + ql - t0)) for t0 in range(base, base + ql, TILE)]
+        base += ql
+    scale = hd ** -0.5
+    ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), len(tiles), pos, seq_of, table, nq, nkv, hd, page, scale, window)
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("kernel", ["generic32", "generic16", "decode", "prefill"])
+def test_attention_finds_a_far_key(kernel):
+    """Random scores would hide a key that is skipped or misplaced: make one far
+    key (at a page's first slot, deep in a long context) dominate and check that
+    the output is its value."""
+    ops = _ops()
+    nq, nkv, hd, page = 8, 2, 64, 16
+    dt = torch.float32 if kernel == "generic32" else torch.bfloat16
+    ctx_lens, q_lens = [900], [1 if kernel != "prefill" else 34]
+    for target in (0, 16 * 20, 16 * 20 + 15, 899 - 34):
+        q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=9)
+        K, V = dense[0]
+        # all queries point along e0; the target key has a large e0 component
+        q.zero_()
+        q[:, :, 0] = 8.0
+        pages = table[0].tolist()
+        kc[pages[target // page], :, target % page, :] = 0
+        kc[pages[target // page], :, target % page, 0] = 60.0
+        out = torch.empty_like(q)
+        n = q.shape[0]
+        scale = hd ** -0.5
+        if kernel.startswith("generic"):
+            ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, 0)
+        elif kernel == "decode":
+            acc, ml = torch.empty(n * nq * 8 * hd, device=DEV), torch.empty(n * nq * 16, device=DEV)
+            ops.attn_decode_bf16(q, out, kc, vc, i32([0]), 1, pos, seq_of, table, acc, ml, 8, nq, nkv, hd, page, scale, 0)
+        else:
+            tiles = [(0, 32), (32, 2)]
+            ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), 2, pos, seq_of, table, nq, nkv, hd, page, scale, 0)
+        want = V[target].double().repeat_interleave(nq // nkv, 0)      # nq, hd
+        assert torch.allclose(out.double().cpu(), want.expand(n, nq, hd), atol=3e-2), (kernel, target)
+
+
+# ----------------------------------------------------------------------------- sampling
+
+def test_argmax_first_of_equals():
+    ops = _ops()
+    logits = rnd(6, 1001, seed=11)
+    logits[2, 700] = 50.0
+    logits[2, 30] = 50.0        # tie: the lower index wins, as torch.argmax
+    logits[3, 1000] = 99.0
+    out = torch.zeros(6, dtype=torch.int32, device=DEV)
+    ops.argmax(logits, out)
+    assert out.tolist() == logits.argmax(-1).tolist()
+    assert out[2] == 30 and out[3] == 1000
+
+
+def test_sample_inverse_cdf():
+    ops = _ops()
+    m, v = 64, 1537
+    logits = rnd(m, v, seed=12, scale=2.0)
+    temps = [0.0 if i % 8 == 0 else 0.5 + 0.01 * i for i in range(m)]
+    us = [random.Random(i).random() for i in range(m)]
+    out = torch.full((m,), -1, dtype=torch.int32, device=DEV)
+    ops.argmax(logits, out)
+    ops.sample(logits, torch.tensor(temps, device=DEV), torch.tensor(us, device=DEV), out)
+    got = out.tolist()
+    for i in range(m):
+        if temps[i] == 0:
+            assert got[i] == int(logits[i].argmax())
+            continue
+        c = torch.cumsum(torch.softmax(logits[i].double() / temps[i], -1), -1).cpu()
+        lo = c[got[i] - 1].item() if got[i] > 0 else 0.0
+        # the drawn number lies in the chosen token's interval (up to float32 rounding of the sums)
+        assert lo - 1e-5 <= us[i] <= c[got[i]].item() + 1e-5, (i, got[i], us[i])
+    # u = 0 picks the first token with non-zero probability; large T is near uniform: u maps linearly
+    out2 = torch.zeros(1, dtype=torch.int32, device=DEV)
+    flat = torch.zeros(1, v, device=DEV)
+    ops.sample(flat, torch.tensor([1.0], device=DEV), torch.tensor([0.5], device=DEV), out2)
+    assert abs(int(out2[0]) - v // 2) <= 1
