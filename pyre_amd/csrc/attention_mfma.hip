@@ -212,26 +212,33 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 }
 
 // out[token, head, :] = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s.
+// One block per (token, head); the weights of the splits are formed once in LDS.
+constexpr int kMaxSplits = 128;
+
 template <int HD>
-__global__ void attn_decode_reduce(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                   const int* __restrict__ tokens, bf16* __restrict__ out, int nq,
-                                   int nsplits) {
-  const int idx = blockIdx.x, head = blockIdx.y;
+__global__ __launch_bounds__(128) void attn_decode_reduce(const float* __restrict__ part_acc,
+                                                          const float* __restrict__ part_ml,
+                                                          const int* __restrict__ tokens,
+                                                          bf16* __restrict__ out, int nq, int nsplits) {
+  __shared__ float w[kMaxSplits];
+  __shared__ float scratch[16];
+  const int idx = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   const size_t base = (static_cast<size_t>(idx) * nq + head) * nsplits;
-  float M = -INFINITY;
-  for (int s = 0; s < nsplits; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
-  float L = 0.f;
-  for (int s = 0; s < nsplits; ++s) {
-    const float ms = part_ml[2 * (base + s)];
-    if (ms != -INFINITY) L += part_ml[2 * (base + s) + 1] * __builtin_amdgcn_exp2f(ms - M);
+  float ms = -INFINITY, ls = 0.f;
+  if (tid < nsplits) {
+    const float2 v = *reinterpret_cast<const float2*>(part_ml + 2 * (base + tid));
+    ms = v.x;
+    ls = v.y;
   }
+  const float M = block_max(ms, scratch);
+  const float ws = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
+  if (tid < nsplits) w[tid] = ws;
+  const float L = block_sum(ls * ws, scratch);  // its barriers publish w[]
   const int tok = tokens[idx];
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+  for (int d = tid; d < HD; d += 128) {
     float acc = 0.f;
-    for (int s = 0; s < nsplits; ++s) {
-      const float ms = part_ml[2 * (base + s)];
-      if (ms != -INFINITY) acc += part_acc[(base + s) * HD + d] * __builtin_amdgcn_exp2f(ms - M);
-    }
+#pragma unroll 8
+    for (int s = 0; s < nsplits; ++s) acc += part_acc[(base + s) * HD + d] * w[s];
     out[(static_cast<size_t>(tok) * nq + head) * HD + d] = from_float<bf16>(acc / L);
   }
 }
@@ -338,7 +345,8 @@ extern "C" int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cac
   PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
                "attn_decode_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
-  PYRE_REQUIRE(nsplits >= 1 && table_stride > 0, "attn_decode_bf16: bad split count or table");
+  PYRE_REQUIRE(nsplits >= 1 && nsplits <= kMaxSplits && table_stride > 0,
+               "attn_decode_bf16: split count %d is outside 1..%d, or bad table", nsplits, kMaxSplits);
   if (n_tokens <= 0) return 0;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
   PYRE_REQUIRE(n_tokens <= 65535 && nkv * qtiles <= 65535, "attn_decode_bf16: grid too large");
@@ -350,7 +358,7 @@ extern "C" int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cac
                        static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), tokens,
                        positions, seq_of_token, block_table, table_stride, part_acc, part_ml, nq, nkv,
                        page_size, scale_log2, window, nsplits);
-    hipLaunchKernelGGL(attn_decode_reduce<HD>, dim3(n_tokens, nq), dim3(HD <= 64 ? 64 : 128), 0, stream,
+    hipLaunchKernelGGL(attn_decode_reduce<HD>, dim3(n_tokens, nq), dim3(128), 0, stream,
                        part_acc, part_ml, tokens, static_cast<bf16*>(out), nq, nsplits);
   });
   PYRE_REQUIRE(rc == 0, "attn_decode_bf16: no kernel for head_dim %d", hd);

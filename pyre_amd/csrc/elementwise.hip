@@ -3,6 +3,7 @@
 // only roundings are the stores to a 16-bit output.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec.h"
 
 using namespace pyre;
 
@@ -86,6 +87,9 @@ extern "C" int pyre_add_rmsnorm(float* resid, const void* delta, int delta_dt, i
   PYRE_REQUIRE(!bias || known_dtype(bias_dt), "add_rmsnorm: unknown bias dtype");
   PYRE_REQUIRE(n >= 0 && hidden > 0 && eps > 0.f, "add_rmsnorm: bad sizes n=%d hidden=%d", n, hidden);
   if (n == 0) return 0;
+  if (!bias && add_rmsnorm_vec(resid, delta, delta_dt, delta ? n_partials : 0, partial_stride, gain, gain_dt,
+                               out, out_dt, rows, n, hidden, eps, stream))
+    return check_launch("add_rmsnorm");
   hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(256), 0, stream, resid, delta, delta_dt,
                      n_partials, static_cast<size_t>(partial_stride), bias, bias_dt, gain, gain_dt,
                      out, out_dt, rows, hidden, eps);
@@ -181,6 +185,10 @@ extern "C" int pyre_rope_kv_write(const void* qkv, int qkv_dt, int n_partials, l
                "rope_kv_write: rotary_dim %d must be even and at most head_dim %d", rotary_dim, hd);
   PYRE_REQUIRE(rotary_dim == 0 || (cos_t && sin_t), "rope_kv_write: rotary tables missing");
   if (n <= 0) return 0;
+  if (rope_kv_write_vec(qkv, qkv_dt, n_partials, partial_stride, bias, bias_dt, q_out, q_dt, k_cache, v_cache,
+                        write_kv ? cache_dt : q_dt, cos_t, sin_t, rotary_dim, positions, slots, n, nq, nkv, hd,
+                        page_size, write_kv, stream))
+    return check_launch("rope_kv_write");
   PYRE_DISPATCH(cache_dt, TC,
                 hipLaunchKernelGGL(rope_kv_write_kernel<TC>, dim3(n), dim3(256), 0, stream, qkv,
                                    qkv_dt, n_partials, static_cast<size_t>(partial_stride), bias,
@@ -214,6 +222,8 @@ extern "C" int pyre_silu_mul(const void* gu, int gu_dt, int n_partials, long par
   PYRE_REQUIRE(known_dtype(gu_dt) && known_dtype(out_dt), "silu_mul: unknown dtype");
   PYRE_REQUIRE(n_partials >= 1 && inter > 0, "silu_mul: bad sizes");
   if (n <= 0) return 0;
+  if (silu_mul_vec(gu, gu_dt, n_partials, partial_stride, out, out_dt, n, inter, stream))
+    return check_launch("silu_mul");
   const size_t total = static_cast<size_t>(n) * inter;
   hipLaunchKernelGGL(silu_mul_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, gu, gu_dt,
                      n_partials, static_cast<size_t>(partial_stride), out, out_dt, total, inter);

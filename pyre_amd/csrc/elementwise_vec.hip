@@ -1,0 +1,202 @@
+// Vectorised forms of the row kernels for the common case (widths that are
+// multiples of 4, no pending bias in the norm, full-head rotary): same formulas and
+// the same order of additions as elementwise.hip, 16 bytes per load where the
+// general kernels load one element. The entry points in elementwise.hip try these
+// first and fall back to the general kernels.
+#include "pyre_common.h"
+#include "pyre_vec.h"
+
+using namespace pyre;
+
+namespace {
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ inline float4 load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+  static __device__ inline void store(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <> struct Vec4<bf16> {
+  static __device__ inline float4 load(const bf16* p) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    float4 v;
+    v.x = __uint_as_float(u.x << 16);
+    v.y = __uint_as_float(u.x & 0xffff0000u);
+    v.z = __uint_as_float(u.y << 16);
+    v.w = __uint_as_float(u.y & 0xffff0000u);
+    return v;
+  }
+  static __device__ inline void store(bf16* p, float4 v) {
+    uint2 u;
+    u.x = static_cast<uint32_t>(bf16_bits(v.x)) | (static_cast<uint32_t>(bf16_bits(v.y)) << 16);
+    u.y = static_cast<uint32_t>(bf16_bits(v.z)) | (static_cast<uint32_t>(bf16_bits(v.w)) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+  }
+};
+
+__device__ inline float4 add4(float4 a, float4 b) { return float4{a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w}; }
+
+// ---------------------------------------------------------------------------
+// add + RMSNorm, one block per row, the row kept in registers between the passes.
+// ---------------------------------------------------------------------------
+constexpr int kNormThreads = 256;
+constexpr int kNormMaxVec = 8;  // float4 per thread: rows of up to 8192 elements
+
+template <typename TD, typename TG, typename TO>
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_vec_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, int n_partials, size_t partial_stride,
+    const TG* __restrict__ gain, TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int r_out = blockIdx.x, r_in = rows ? rows[r_out] : r_out;
+  const size_t in_off = static_cast<size_t>(r_in) * hidden;
+  const int nvec = hidden / 4;
+  float4 v[kNormMaxVec];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kNormMaxVec; ++i) {
+    const int c = threadIdx.x + i * kNormThreads;
+    if (c >= nvec) break;
+    float4 x = Vec4<float>::load(resid + in_off + 4 * c);
+    if (delta) {
+      float4 d = Vec4<TD>::load(delta + in_off + 4 * c);
+      for (int p = 1; p < n_partials; ++p) d = add4(d, Vec4<TD>::load(delta + p * partial_stride + in_off + 4 * c));
+      x = add4(x, d);
+      if (!rows) Vec4<float>::store(resid + in_off + 4 * c, x);
+    }
+    v[i] = x;
+    ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+  const size_t out_off = static_cast<size_t>(r_out) * hidden;
+#pragma unroll
+  for (int i = 0; i < kNormMaxVec; ++i) {
+    const int c = threadIdx.x + i * kNormThreads;
+    if (c >= nvec) break;
+    const float4 gn = Vec4<TG>::load(gain + 4 * c);
+    const float4 x = v[i];
+    Vec4<TO>::store(out + out_off + 4 * c, float4{x.x * inv * gn.x, x.y * inv * gn.y, x.z * inv * gn.z, x.w * inv * gn.w});
+  }
+}
+
+// ---------------------------------------------------------------------------
+// rotary + cache write, four pairs per item; grid (tokens, ceil(items / 256)).
+// ---------------------------------------------------------------------------
+template <typename TI, typename TC>
+__global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
+    const TI* __restrict__ qkv, int n_partials, size_t partial_stride, const void* __restrict__ bias,
+    int bias_dt, TC* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ positions,
+    const int* __restrict__ slots, int nq, int nkv, int hd, int page_size, int write_kv) {
+  const int n = blockIdx.x;
+  const int half = hd / 2, hv = half / 4;            // vec4 pairs per head
+  const int n_rot = (nq + nkv) * hv, n_items = n_rot + nkv * (hd / 4);
+  const int it = blockIdx.y * 256 + threadIdx.x;
+  if (it >= n_items) return;
+  const int width = (nq + 2 * nkv) * hd;
+  const size_t in_row = static_cast<size_t>(n) * width;
+  const int slot = write_kv ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+
+  auto value4 = [&](int col) {
+    float4 v = Vec4<TI>::load(qkv + in_row + col);
+    for (int p = 1; p < n_partials; ++p) v = add4(v, Vec4<TI>::load(qkv + p * partial_stride + in_row + col));
+    if (bias) {
+      v.x += load_as_float(bias, bias_dt, col);
+      v.y += load_as_float(bias, bias_dt, col + 1);
+      v.z += load_as_float(bias, bias_dt, col + 2);
+      v.w += load_as_float(bias, bias_dt, col + 3);
+    }
+    return v;
+  };
+
+  if (it < n_rot) {
+    const int head = it / hv, j = 4 * (it % hv);
+    if (head >= nq && slot < 0) return;
+    const int base = head * hd;
+    const float4 x1 = value4(base + j), x2 = value4(base + j + half);
+    const size_t t = static_cast<size_t>(positions[n]) * half + j;
+    const float4 c = Vec4<float>::load(cos_t + t), s = Vec4<float>::load(sin_t + t);
+    const float4 a{x1.x * c.x - x2.x * s.x, x1.y * c.y - x2.y * s.y, x1.z * c.z - x2.z * s.z, x1.w * c.w - x2.w * s.w};
+    const float4 b{x2.x * c.x + x1.x * s.x, x2.y * c.y + x1.y * s.y, x2.z * c.z + x1.z * s.z, x2.w * c.w + x1.w * s.w};
+    TC* dst = head < nq ? q_out + static_cast<size_t>(n) * nq * hd + base
+                        : k_cache + ((static_cast<size_t>(page) * nkv + (head - nq)) * page_size + off) * hd;
+    Vec4<TC>::store(dst + j, a);
+    Vec4<TC>::store(dst + j + half, b);
+  } else if (slot >= 0) {
+    const int e = 4 * (it - n_rot);
+    const int kvh = e / hd, d = e % hd;
+    const float4 v = value4((nq + nkv) * hd + e);
+    TC* dst = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off;
+    dst[0] = from_float<TC>(v.x);
+    dst[page_size] = from_float<TC>(v.y);
+    dst[2 * static_cast<size_t>(page_size)] = from_float<TC>(v.z);
+    dst[3 * static_cast<size_t>(page_size)] = from_float<TC>(v.w);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// SiLU-gate, four features per thread.
+// ---------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict__ gu, int n_partials,
+                                                           size_t partial_stride, TO* __restrict__ out,
+                                                           size_t total4, int inter) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const int per_row = inter / 4;
+  const size_t n = i / per_row, c = 4 * (i % per_row);
+  const size_t gi = n * 2 * inter + c, ui = gi + inter;
+  float4 g = Vec4<TI>::load(gu + gi), u = Vec4<TI>::load(gu + ui);
+  for (int p = 1; p < n_partials; ++p) {
+    g = add4(g, Vec4<TI>::load(gu + p * partial_stride + gi));
+    u = add4(u, Vec4<TI>::load(gu + p * partial_stride + ui));
+  }
+  Vec4<TO>::store(out + n * inter + c, float4{g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
+                                              g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w});
+}
+
+}  // namespace
+
+namespace pyre {
+
+bool add_rmsnorm_vec(float* resid, const void* delta, int delta_dt, int n_partials, long partial_stride,
+                     const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
+                     int hidden, float eps, hipStream_t stream) {
+  if (hidden % 4 || hidden > 4 * kNormThreads * kNormMaxVec || (delta && partial_stride % 4)) return false;
+  PYRE_DISPATCH(delta_dt, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO,
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO>), dim3(n), dim3(kNormThreads), 0, stream, resid,
+                         static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),
+                         static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps))));
+  return true;
+}
+
+bool rope_kv_write_vec(const void* qkv, int qkv_dt, int n_partials, long partial_stride, const void* bias,
+                       int bias_dt, void* q_out, int q_dt, void* k_cache, void* v_cache, int cache_dt,
+                       const float* cos_t, const float* sin_t, int rotary_dim, const int* positions,
+                       const int* slots, int n, int nq, int nkv, int hd, int page_size, int write_kv,
+                       hipStream_t stream) {
+  if (rotary_dim != hd || hd % 8 || partial_stride % 4 || (write_kv && q_dt != cache_dt)) return false;
+  const int items = (nq + nkv) * (hd / 8) + nkv * (hd / 4);
+  const dim3 grid(n, (items + 255) / 256);
+  if (grid.y > 65535) return false;
+  PYRE_DISPATCH(qkv_dt, TI, PYRE_DISPATCH(q_dt, TC,
+      hipLaunchKernelGGL((rope_kv_write_vec_kernel<TI, TC>), grid, dim3(256), 0, stream,
+                         static_cast<const TI*>(qkv), n_partials, static_cast<size_t>(partial_stride), bias,
+                         bias_dt, static_cast<TC*>(q_out), static_cast<TC*>(k_cache),
+                         static_cast<TC*>(v_cache), cos_t, sin_t, positions, slots, nq, nkv, hd, page_size,
+                         write_kv)));
+  return true;
+}
+
+bool silu_mul_vec(const void* gu, int gu_dt, int n_partials, long partial_stride, void* out, int out_dt,
+                  int n, int inter, hipStream_t stream) {
+  if (inter % 4 || partial_stride % 4) return false;
+  const size_t total4 = static_cast<size_t>(n) * (inter / 4);
+  PYRE_DISPATCH(gu_dt, TI, PYRE_DISPATCH(out_dt, TO,
+      hipLaunchKernelGGL((silu_mul_vec_kernel<TI, TO>), dim3((total4 + 255) / 256), dim3(256), 0, stream,
+                         static_cast<const TI*>(gu), n_partials, static_cast<size_t>(partial_stride),
+                         static_cast<TO*>(out), total4, inter)));
+  return true;
+}
+
+}  // namespace pyre

@@ -36,6 +36,17 @@ int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, cons
                       int w_dt, long ldw, const void* bias, int bias_dt, void* out, int out_dt,
                       long ldo, int M, int N, int K, hipStream_t stream);
 
+// bfloat16 products with 1..64 rows (decode): 1 if the kernel takes the shape.
+int pyre_gemm_skinny_supports(int M, int N, int K, long ldx, long ldw);
+
+// out: float32 [ksplit][M][N] partial sums of X[M, K] W[N, K]^T.
+int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N,
+                          int K, int ksplit, hipStream_t stream);
+
+// W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
+int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
+                               int two_i, int K, hipStream_t stream);
+
 int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                       const void* v_cache, int cache_dt, const int* positions,
                       const int* seq_of_token, const int* block_table, int table_stride, int n,
@@ -61,7 +72,8 @@ int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const 
                            int nq, int nkv, int hd, int page_size, float scale, int window,
                            hipStream_t stream);
 
-int pyre_argmax(const float* logits, long row_stride, int* out, int m, int vocab,
+// scratch: m * 64 floats followed by m * 64 ints of device memory.
+int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,
                 hipStream_t stream);
 
 int pyre_sample(const float* logits, long row_stride, const float* temperature,

@@ -11,31 +11,51 @@ namespace {
 constexpr int kThreads = 1024;
 
 // Largest value; among equal values the lowest index (torch.argmax's choice).
-__global__ __launch_bounds__(kThreads) void argmax_kernel(const float* __restrict__ logits,
-                                                          size_t row_stride, int* __restrict__ out,
-                                                          int vocab) {
-  __shared__ float best_v[kThreads / kWave];
-  __shared__ int best_i[kThreads / kWave];
+// Two stages so that a few rows still fill the chip: kSlices blocks per row each
+// reduce a slice of the vocabulary, then one block per row reduces the slices.
+constexpr int kSlices = 64;
+constexpr int kArgThreads = 256;
+
+__device__ inline void better(float& bv, int& bi, float ov, int oi) {
+  if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+}
+
+__device__ inline void block_argmax(float& bv, int& bi, float* sv, int* si) {
+  for (int o = kWave / 2; o > 0; o >>= 1) better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
+  const int w = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) { sv[w] = bv; si[w] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int i = 1; i < kArgThreads / kWave; ++i) better(bv, bi, sv[i], si[i]);
+}
+
+__global__ __launch_bounds__(kArgThreads) void argmax_slices_kernel(const float* __restrict__ logits,
+                                                                    size_t row_stride, float* __restrict__ pv,
+                                                                    int* __restrict__ pi, int vocab) {
+  __shared__ float sv[kArgThreads / kWave];
+  __shared__ int si[kArgThreads / kWave];
   const float* row = logits + blockIdx.x * row_stride;
+  const int per = (vocab + kSlices - 1) / kSlices;
+  const int begin = min(vocab, static_cast<int>(blockIdx.y) * per), end = min(vocab, begin + per);
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += kThreads) {
+  for (int i = begin + threadIdx.x; i < end; i += kArgThreads) {
     const float v = row[i];
-    if (v > bv || (v == bv && i < bi) || bi == 0x7fffffff) { bv = v; bi = i; }
+    if (bi == 0x7fffffff) { bv = v; bi = i; } else better(bv, bi, v, i);
   }
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(bv, o, kWave);
-    const int oi = __shfl_xor(bi, o, kWave);
-    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-  }
-  const int w = threadIdx.x / kWave;
-  if ((threadIdx.x & (kWave - 1)) == 0) { best_v[w] = bv; best_i[w] = bi; }
-  __syncthreads();
+  block_argmax(bv, bi, sv, si);
   if (threadIdx.x == 0) {
-    for (int i = 1; i < kThreads / kWave; ++i)
-      if (best_v[i] > bv || (best_v[i] == bv && best_i[i] < bi)) { bv = best_v[i]; bi = best_i[i]; }
-    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    pv[blockIdx.x * kSlices + blockIdx.y] = bv;
+    pi[blockIdx.x * kSlices + blockIdx.y] = bi;
   }
+}
+
+__global__ __launch_bounds__(kWave) void argmax_final_kernel(const float* __restrict__ pv,
+                                                             const int* __restrict__ pi, int* __restrict__ out) {
+  float bv = pv[blockIdx.x * kSlices + threadIdx.x];
+  int bi = pi[blockIdx.x * kSlices + threadIdx.x];
+  for (int o = kWave / 2; o > 0; o >>= 1) better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
 }
 
 // p_i = exp((x_i - max) / T) / sum;  token = first i with cumsum(p)_i > u, u in [0, 1).
@@ -96,12 +116,18 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(const float* __restric
 
 }  // namespace
 
-extern "C" int pyre_argmax(const float* logits, long row_stride, int* out, int m, int vocab,
+// scratch: m * 64 floats followed by m * 64 ints.
+extern "C" int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,
                            hipStream_t stream) {
   PYRE_REQUIRE(vocab > 0 && row_stride >= vocab, "argmax: bad sizes");
+  PYRE_REQUIRE(m <= 65535, "argmax: too many rows");
   if (m <= 0) return 0;
-  hipLaunchKernelGGL(argmax_kernel, dim3(m), dim3(kThreads), 0, stream, logits,
-                     static_cast<size_t>(row_stride), out, vocab);
+  static_assert(kSlices == kWave, "the final stage reduces one slice per lane");
+  float* pv = static_cast<float*>(scratch);
+  int* pi = reinterpret_cast<int*>(pv + static_cast<size_t>(m) * kSlices);
+  hipLaunchKernelGGL(argmax_slices_kernel, dim3(m, kSlices), dim3(kArgThreads), 0, stream, logits,
+                     static_cast<size_t>(row_stride), pv, pi, vocab);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(m), dim3(kWave), 0, stream, pv, pi, out);
   return check_launch("argmax");
 }
 

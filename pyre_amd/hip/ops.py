@@ -229,12 +229,22 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_ca
          int(window), _stream())
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
-    _dev(logits, out)
+ARGMAX_SCRATCH_PER_ROW = 128  #: 4-byte words of scratch per row of logits
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor | None = None) -> None:
+    """out[i] = index of the largest logit of row i (the lowest index among equals).
+    ``scratch``: int32 or float32 device memory of 128 words per row (allocated if absent)."""
+    _dev(logits, out, scratch)
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("argmax: float32 [M, V] logits expected")
-    _i32("out", out, logits.shape[0])
-    call("pyre_argmax", logits.data_ptr(), logits.stride(0), out.data_ptr(), logits.shape[0],
+    m = logits.shape[0]
+    _i32("out", out, m)
+    if scratch is None:
+        scratch = torch.empty(m * ARGMAX_SCRATCH_PER_ROW, dtype=torch.int32, device=logits.device)
+    if scratch.element_size() != 4 or scratch.numel() < m * ARGMAX_SCRATCH_PER_ROW or not scratch.is_contiguous():
+        raise KernelError("argmax: scratch must hold 128 four-byte words per row")
+    call("pyre_argmax", logits.data_ptr(), logits.stride(0), out.data_ptr(), scratch.data_ptr(), m,
          logits.shape[1], _stream())
 
 
@@ -297,3 +307,40 @@ def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_o
     call("pyre_attn_prefill_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
          tiles.data_ptr(), n_tiles, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
          block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), _stream())
+
+
+def gemm_skinny_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
+    from pyre_amd.hip.lib import lib
+
+    return bool(lib().pyre_gemm_skinny_supports(m, n, k, ldx, ldw))
+
+
+def _skinny_common(x, w, m):
+    _dev(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("gemm_skinny: bfloat16 operands expected")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.shape[0] < m:
+        raise KernelError(f"gemm_skinny: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit {m} rows")
+    if x.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError("gemm_skinny: rows must be contiguous")
+
+
+def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int) -> None:
+    """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 64."""
+    _skinny_common(x, w, m)
+    n = w.shape[0]
+    if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() < ksplit * m * n or not out.is_cuda:
+        raise KernelError("gemm_skinny: out must be contiguous float32 [ksplit, m, N] on the GPU")
+    call("pyre_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), m, n,
+         w.shape[1], ksplit, _stream())
+
+
+def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int) -> None:
+    """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up]."""
+    _skinny_common(x, w_gate_up, m)
+    two_i = w_gate_up.shape[0]
+    if (out.dtype != torch.bfloat16 or not out.is_contiguous() or not out.is_cuda or out.dim() != 2
+            or out.shape[1] * 2 != two_i or out.shape[0] < m):
+        raise KernelError("gemm_skinny_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
+    call("pyre_gemm_skinny_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+         out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())

@@ -14,21 +14,63 @@ import torch
 
 from pyre_amd.hip.ops import Partials
 
-#: rows from which a 16-bit product goes to the BLAS library
-LIBRARY_GEMM_MIN_ROWS = 1
+#: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the BLAS library
+SKINNY_MAX_ROWS = 64
+#: blocks (of four waves) a weight-streaming product is spread over at least
+SKINNY_TARGET_BLOCKS = 512
+
+
+def skinny_ksplit(n_out: int, k: int) -> int:
+    """Blocks per output tile, so that a product with few columns still fills the chip."""
+    tiles = -(-n_out // 16)
+    blocks = -(-tiles // 2) if tiles >= 4096 else tiles
+    return max(1, min(-(-SKINNY_TARGET_BLOCKS // blocks), k // 512, 64))
+
+
+def _is_bf16(ctx, lin, x) -> bool:
+    return (ctx.runtime.dtype == torch.bfloat16 and lin.weight.dtype == torch.bfloat16
+            and x.dtype == torch.bfloat16)
 
 
 def linear(lin, ctx, x, n, out):
+    from pyre_amd.hip import ops
+
     rt = ctx.runtime
-    if rt.dtype != torch.bfloat16 or lin.weight.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+    if not _is_bf16(ctx, lin, x):
         return None
-    if not rt.options.get("library_gemm", True) or n < LIBRARY_GEMM_MIN_ROWS:
+    k, n_out = lin.in_features, lin.out_features
+    skinny = rt.options.get("skinny_gemm", True) and ops.gemm_skinny_supports(
+        min(n, SKINNY_MAX_ROWS), n_out, k, x.stride(0), lin.weight.stride(0))
+    if skinny and (n <= SKINNY_MAX_ROWS or out is not None):
+        if out is not None:
+            # float32 results wanted in place (the head's logits): no split, 64 rows at a time
+            for r0 in range(0, n, SKINNY_MAX_ROWS):
+                rows = min(SKINNY_MAX_ROWS, n - r0)
+                ops.gemm_skinny_bf16(x[r0:r0 + rows], lin.weight, out[r0:r0 + rows], rows, 1)
+            return Partials(out.view(1, n, n_out), lin.bias)
+        ks = skinny_ksplit(n_out, k)
+        buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
+        ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
+        return Partials(buf, lin.bias)
+    if out is not None or not rt.options.get("library_gemm", True):
         return None
-    if out is not None:
-        return None  # float32 results (the head's logits) stay with the engine's own kernels for now
-    buf = ctx.workspace.get(f"linear16.{lin.role}", (n, lin.out_features), torch.bfloat16)
+    buf = ctx.workspace.get(f"linear16.{lin.role}", (n, n_out), torch.bfloat16)
     torch.mm(x[:n], lin.weight.t(), out=buf)
-    return Partials(buf.view(1, n, lin.out_features), lin.bias)
+    return Partials(buf.view(1, n, n_out), lin.bias)
+
+
+def gate_up_silu(lin, ctx, x, n, act) -> bool:
+    """silu(x gate^T) * (x up^T) in one kernel for a decode step's few rows."""
+    from pyre_amd.hip import ops
+
+    if not _is_bf16(ctx, lin, x) or n > SKINNY_MAX_ROWS or lin.bias is not None:
+        return False
+    if not ctx.runtime.options.get("skinny_gemm", True):
+        return False
+    if not ops.gemm_skinny_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):
+        return False
+    ops.gemm_skinny_silu_bf16(x, lin.weight, act, n)
+    return True
 
 
 #: waves the split of decode attention aims at (256 CUs x 8)

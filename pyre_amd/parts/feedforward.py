@@ -5,6 +5,7 @@ from __future__ import annotations
 import torch
 
 from pyre_amd.hip import ops
+from pyre_amd.parts import fast
 from pyre_amd.parts.base import FeedForward, SwiGLUSpec, TensorSpec
 from pyre_amd.parts.linear import Linear, linear_specs
 
@@ -30,7 +31,8 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx, h):
         n = ctx.n_tokens
-        gu = self.gate_up.forward(ctx, h, n)
         act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)
-        ops.silu_mul(gu, act, n)
+        if not fast.gate_up_silu(self.gate_up, ctx, h, n, act):
+            gu = self.gate_up.forward(ctx, h, n)
+            ops.silu_mul(gu, act, n)
         return self.down.forward(ctx, act, n)

@@ -17,6 +17,7 @@ class Sampler:
         self._dev = torch.empty(2 * max_rows, dtype=torch.float32, device=device)
         self._ids = torch.empty(max_rows, dtype=torch.int32, device=device)
         self._ids_host = torch.empty(max_rows, dtype=torch.int32, pin_memory=True)
+        self._scratch = torch.empty(max_rows * ops.ARGMAX_SCRATCH_PER_ROW, dtype=torch.int32, device=device)
 
     def sample(self, logits: torch.Tensor, temperatures: list[float], uniforms: list[float]) -> list[int]:
         """logits: float32 [M, V] on the device. Row i: argmax if temperatures[i]
@@ -27,7 +28,7 @@ class Sampler:
             raise ValueError("sampler: row counts do not fit")
         with torch.cuda.device(self.device):
             ids = self._ids[:m]
-            ops.argmax(logits, ids)
+            ops.argmax(logits, ids, self._scratch)
             if any(t > 0 for t in temperatures):
                 self._host[:m] = torch.tensor(temperatures, dtype=torch.float32)
                 self._host[m:2 * m] = torch.tensor(uniforms, dtype=torch.float32)
