@@ -112,7 +112,8 @@ class CacheManager:
             g.v = torch.zeros((n, g.num_pages, s.num_kv_heads, s.head_dim, g.page_size), device=device, dtype=dtype)
         for g in self.state_groups:
             dt = torch.float32 if g.spec.dtype == "float32" else dtype
-            g.tensor = torch.zeros((len(g.entries), self.max_num_seqs, *g.spec.shape), device=device, dtype=dt)
+            # one slot more than requests: padding rows of a captured step write there
+            g.tensor = torch.zeros((len(g.entries), self.max_num_seqs + 1, *g.spec.shape), device=device, dtype=dt)
 
     def bytes_per_page(self, dtype_bytes: int) -> int:
         return sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * g.page_size * dtype_bytes

@@ -58,18 +58,22 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
     for (int j = tid; j < cnt; j += kThreads) {
       const int key = base + j;
       const int page = table[key / page_size], off = key % page_size;
-      const TC* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * hd;
-      float s = 0.f;
-      for (int e = 0; e < hd; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
-      s *= scale;
+      float s = -INFINITY;  // a page that is not there (padding rows of a captured step) hides its keys
+      if (page >= 0) {
+        const TC* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * hd;
+        s = 0.f;
+        for (int e = 0; e < hd; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+        s *= scale;
+      }
       sc[j] = s;
       lmax = fmaxf(lmax, s);
     }
     const float m_new = fmaxf(m, block_max(lmax, scratch));
-    const float alpha = expf(m - m_new);  // 0 on the first chunk (m = -inf)
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = expf(m - m_use);  // 0 on the first chunk (m = -inf)
     float lsum = 0.f;
     for (int j = tid; j < cnt; j += kThreads) {
-      const float p = expf(sc[j] - m_new);
+      const float p = expf(sc[j] - m_use);
       sc[j] = p;
       lsum += p;
     }
@@ -79,6 +83,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
       for (int j = g; j < cnt; j += groups) {
         const int key = base + j;
         const int page = table[key / page_size], off = key % page_size;
+        if (page < 0) continue;
         const TC* vp = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off;
         acc = fmaf(sc[j], to_float(*vp), acc);
       }
@@ -92,7 +97,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
   if (tid < hd) {
     float total = 0.f;
     for (int gg = 0; gg < groups; ++gg) total += accs[gg * hd + tid];
-    out[(static_cast<size_t>(n) * nq + h) * hd + tid] = from_float<TQ>(total / l);
+    out[(static_cast<size_t>(n) * nq + h) * hd + tid] = from_float<TQ>(l > 0.f ? total / l : 0.f);
   }
 }
 

@@ -239,7 +239,8 @@ __global__ __launch_bounds__(128) void attn_decode_reduce(const float* __restric
     float acc = 0.f;
 #pragma unroll 8
     for (int s = 0; s < nsplits; ++s) acc += part_acc[(base + s) * HD + d] * w[s];
-    out[(static_cast<size_t>(tok) * nq + head) * HD + d] = from_float<bf16>(acc / L);
+    // L is 0 only for a row that sees no key at all (padding of a captured step).
+    out[(static_cast<size_t>(tok) * nq + head) * HD + d] = from_float<bf16>(L > 0.f ? acc / L : 0.f);
   }
 }
 

@@ -39,13 +39,14 @@ int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, cons
 // bfloat16 products with 1..64 rows (decode): 1 if the kernel takes the shape.
 int pyre_gemm_skinny_supports(int M, int N, int K, long ldx, long ldw);
 
-// out: float32 [ksplit][M][N] partial sums of X[M, K] W[N, K]^T.
+// out: float32 [ksplit][M][N] partial sums of X[M, K] W[N, K]^T. form 0: the waves
+// of a block split k (fewest rows); form 1: X staged through LDS (more rows).
 int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N,
-                          int K, int ksplit, hipStream_t stream);
+                          int K, int ksplit, int form, hipStream_t stream);
 
 // W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
 int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
-                               int two_i, int K, hipStream_t stream);
+                               int two_i, int K, int form, hipStream_t stream);
 
 int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                       const void* v_cache, int cache_dt, const int* positions,

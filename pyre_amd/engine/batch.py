@@ -116,3 +116,28 @@ def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: 
         positions=i32(positions), seq_of_token=i32(seq_of_token), q_start=i32(q_start),
         ctx_len=i32(ctx_len), state_slots=i32(state_slots), logit_rows=i32(logit_rows),
         slots=[i32(x) for x in slots], tables=tables, max_q_len=max_q)
+
+
+def pad_decode_batch(hb: HostBatch, n_rows: int, scratch_slot: int, max_ctx: int) -> HostBatch:
+    """A decode-only batch widened to ``n_rows`` requests with rows that do nothing:
+    token 0 at position 0, no cache slot to write to, an empty block table (every key
+    hidden), the scratch state slot. A captured step is replayed at a fixed size;
+    the rows beyond the live requests are these. ``max_ctx`` (the longest context
+    the step's table can hold) fixes how the keys are split."""
+    pad = n_rows - hb.n_seqs
+    if pad < 0 or not hb.decode_only:
+        raise ValueError("only decode batches can be padded, and only upwards")
+    i32 = lambda x: np.asarray(x, dtype=np.int32)  # noqa: E731
+    cat = lambda a, b: np.concatenate([a, i32(b)])  # noqa: E731
+    n = hb.n_tokens
+    return HostBatch(
+        n_tokens=n_rows, n_seqs=n_rows, rids=hb.rids + [None] * pad,
+        tokens=cat(hb.tokens, [0] * pad), positions=cat(hb.positions, [0] * pad),
+        seq_of_token=cat(hb.seq_of_token, range(hb.n_seqs, n_rows)),
+        q_start=i32(range(n_rows + 1)), ctx_len=cat(hb.ctx_len, [1] * pad),
+        state_slots=cat(hb.state_slots, [scratch_slot] * pad),
+        logit_rows=i32(range(n_rows)),
+        slots=[cat(s, [-1] * pad) for s in hb.slots],
+        tables=[np.concatenate([t, np.full((pad, t.shape[1]), -1, dtype=np.int32)]) for t in hb.tables],
+        max_q_len=1, decode_tokens=i32(range(n_rows)), prefill_tiles=i32([]).reshape(-1, 2),
+        max_decode_ctx=max_ctx)

@@ -16,12 +16,17 @@ import torch
 from pyre_amd.cache import CacheManager
 from pyre_amd.config.engine import EngineConfig
 from pyre_amd.config.model import ModelConfig
-from pyre_amd.engine.batch import Entry, build_host_batch
+from pyre_amd.engine.batch import Entry, build_host_batch, pad_decode_batch
 from pyre_amd.engine.context import (TORCH_DTYPES, KVLayerView, MetaBuffers, Runtime, StateLayerView,
                                      StepContext)
 from pyre_amd.parts.model import LayeredModel
 from pyre_amd.registry import get_architecture, load_config
 from pyre_amd.weights.loader import adopt_state, load_weights
+
+
+#: decode steps of up to this many requests are captured in HIP graphs, at these sizes
+GRAPH_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64)
+GRAPH_MAX_ROWS = GRAPH_ROW_BUCKETS[-1]
 
 
 class Engine:
@@ -44,9 +49,13 @@ class Engine:
         num_pages = self._choose_num_pages(probe)
         self.cache = CacheManager(specs, ec.page_size, num_pages, ec.max_num_seqs, self.max_model_len)
         self.cache.materialize(self.device, self.dtype)
-        widths = [self.cache.max_pages_per_seq for _ in self.cache.page_groups]
-        self.meta = MetaBuffers(self.device, ec.max_num_batched_tokens, ec.max_num_seqs, widths)
+        # captured steps round their tables up to a power of two of pages
+        widths = [max(8, 1 << (self.cache.max_pages_per_seq - 1).bit_length()) for _ in self.cache.page_groups]
+        self.meta = MetaBuffers(self.device, max(ec.max_num_batched_tokens, ec.max_num_seqs), ec.max_num_seqs, widths)
         self.steps_run = 0
+        #: captured decode steps: (rows, table width) -> "warm" (ran eagerly once) or (graph, logits)
+        self._graphs: dict[tuple[int, int], object] = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ construction
 
@@ -120,21 +129,70 @@ class Engine:
         for e in entries:
             cache.reserve(e.rid, len(e.tokens))
         pages = max((len(cache.block_table(e.rid, 0)) for e in entries), default=0) if cache.page_groups else 0
-        width = max(8, -(-pages // 8) * 8)
+        graphable = (ec.use_graphs and n_tokens == len(entries) and n_tokens <= GRAPH_MAX_ROWS
+                     and all(len(e.want) == 1 for e in entries))
+        if graphable:
+            # Fixed sizes, so that the step can be captured once and replayed:
+            # the table as wide as a power of two of pages, the rows up to a bucket.
+            width = max(8, 1 << (pages - 1).bit_length())
+            rows = next(b for b in GRAPH_ROW_BUCKETS if b >= n_tokens)
+        else:
+            width = max(8, -(-pages // 8) * 8)
         hb = build_host_batch(entries, cache, self.vocab_size, table_width=width)
         with torch.cuda.device(self.device):
-            views = self.meta.upload(hb)
-            ctx = StepContext(
-                runtime=self.runtime, host=hb, n_tokens=hb.n_tokens, n_seqs=hb.n_seqs,
-                n_logits=len(hb.logit_rows), tokens=views["tokens"], positions=views["positions"],
-                seq_of_token=views["seq_of_token"], logit_rows=views["logit_rows"][:len(hb.logit_rows)],
-                q_start=views["q_start"], ctx_len=views["ctx_len"], state_slots=views["state_slots"],
-                decode_tokens=views["decode_tokens"], prefill_tiles=views["prefill_tiles"])
-            logits = self.model.forward(ctx, self._layer_views(views))
+            if graphable:
+                logits = self._step_captured(hb, rows, width)
+            else:
+                logits = self._run(hb)
         for e in entries:
             cache.commit(e.rid, len(e.tokens))
         self.steps_run += 1
         return logits
+
+    def _context(self, hb, n_cap=None, s_cap=None):
+        views = self.meta.upload(hb, n_cap, s_cap)
+        ctx = StepContext(
+            runtime=self.runtime, host=hb, n_tokens=hb.n_tokens, n_seqs=hb.n_seqs,
+            n_logits=len(hb.logit_rows), tokens=views["tokens"], positions=views["positions"],
+            seq_of_token=views["seq_of_token"], logit_rows=views["logit_rows"][:len(hb.logit_rows)],
+            q_start=views["q_start"], ctx_len=views["ctx_len"], state_slots=views["state_slots"],
+            decode_tokens=views["decode_tokens"], prefill_tiles=views["prefill_tiles"])
+        return ctx, self._layer_views(views)
+
+    def _run(self, hb):
+        ctx, caches = self._context(hb)
+        return self.model.forward(ctx, caches)
+
+    def _step_captured(self, hb, rows: int, width: int):
+        """A decode step at a fixed size (``rows`` requests, tables ``width`` pages
+        wide): run eagerly the first time, captured in a HIP graph the second,
+        replayed from then on. Only the metadata upload happens outside the graph."""
+        live = hb.n_seqs
+        key = (rows, width)
+        padded = pad_decode_batch(hb, rows, self.cache.max_num_seqs, width * self.cache.page_size)
+        state = self._graphs.get(key)
+        if state is None:
+            ctx, caches = self._context(padded)
+            logits = self.model.forward(ctx, caches)
+            self._graphs[key] = "warm"
+            return logits[:live]
+        if state == "warm":
+            ctx, caches = self._context(padded)
+            ws = self.runtime.workspace
+            graph = torch.cuda.CUDAGraph()
+            ws.frozen = True
+            try:
+                with torch.cuda.graph(graph):
+                    logits = self.model.forward(ctx, caches)
+            finally:
+                ws.frozen = False
+            state = self._graphs[key] = (graph, logits)
+        else:
+            self.meta.upload(padded)
+        graph, logits = state
+        graph.replay()
+        self.graph_replays += 1
+        return logits[:live]
 
     def _layer_views(self, views) -> list:
         cache = self.cache

@@ -16,15 +16,25 @@ from pyre_amd.hip.ops import Partials
 
 #: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the BLAS library
 SKINNY_MAX_ROWS = 64
-#: blocks (of four waves) a weight-streaming product is spread over at least
-SKINNY_TARGET_BLOCKS = 512
+#: blocks a weight-streaming product is spread over at least, by form of the kernel
+SKINNY_TARGET_BLOCKS = {0: 2048, 1: 600}
+#: up to this many rows the gate/up product and the SiLU-gate are one kernel
+FUSED_SILU_MAX_ROWS = 8
 
 
-def skinny_ksplit(n_out: int, k: int) -> int:
-    """Blocks per output tile, so that a product with few columns still fills the chip."""
+def skinny_ksplit(m: int, n_out: int, k: int) -> int:
+    """Blocks per output tile, so that a product with few columns still fills the chip
+    (measured on the 7B shapes: more than ~2,000 blocks of form 0 or ~600 of form 1
+    bring nothing, fewer leave bandwidth unused)."""
+    from pyre_amd.hip.ops import skinny_form
+
+    form = skinny_form(m)
     tiles = -(-n_out // 16)
-    blocks = -(-tiles // 2) if tiles >= 4096 else tiles
-    return max(1, min(-(-SKINNY_TARGET_BLOCKS // blocks), k // 512, 64))
+    if form == 0:
+        blocks = -(-tiles // 2) if tiles >= 4096 else tiles
+    else:
+        blocks = -(-tiles // (8 if tiles >= 2048 else 4))
+    return max(1, min(-(-SKINNY_TARGET_BLOCKS[form] // blocks), k // 512, 64))
 
 
 def _is_bf16(ctx, lin, x) -> bool:
@@ -48,7 +58,7 @@ def linear(lin, ctx, x, n, out):
                 rows = min(SKINNY_MAX_ROWS, n - r0)
                 ops.gemm_skinny_bf16(x[r0:r0 + rows], lin.weight, out[r0:r0 + rows], rows, 1)
             return Partials(out.view(1, n, n_out), lin.bias)
-        ks = skinny_ksplit(n_out, k)
+        ks = skinny_ksplit(n, n_out, k)
         buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
         ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
         return Partials(buf, lin.bias)
@@ -63,13 +73,13 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
     """silu(x gate^T) * (x up^T) in one kernel for a decode step's few rows."""
     from pyre_amd.hip import ops
 
-    if not _is_bf16(ctx, lin, x) or n > SKINNY_MAX_ROWS or lin.bias is not None:
+    if not _is_bf16(ctx, lin, x) or n > FUSED_SILU_MAX_ROWS or lin.bias is not None:
         return False
     if not ctx.runtime.options.get("skinny_gemm", True):
         return False
     if not ops.gemm_skinny_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):
         return False
-    ops.gemm_skinny_silu_bf16(x, lin.weight, act, n)
+    ops.gemm_skinny_silu_bf16(x, lin.weight, act, n, 0)
     return True
 
 

@@ -359,27 +359,29 @@ def test_sample_inverse_cdf():
 
 # ----------------------------------------------------------------------------- weight-streaming products
 
+@pytest.mark.parametrize("form", [0, 1])
 @pytest.mark.parametrize("m", [1, 7, 16, 33, 64])
 @pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (3584, 3584, 3), (1000, 136, 2), (131, 8, 1), (70000, 96, 1)])
-def test_gemm_skinny(m, n, k, ksplit):
+def test_gemm_skinny(m, n, k, ksplit, form):
     ops = _ops()
     assert ops.gemm_skinny_supports(m, n, k, k, k)
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
     w = rnd(n, k, dtype=torch.bfloat16, seed=2)
     out = torch.full((ksplit, m, n), float("nan"), device=DEV)
-    ops.gemm_skinny_bf16(x, w, out, m, ksplit)
+    ops.gemm_skinny_bf16(x, w, out, m, ksplit, form)
     want = x.double() @ w.double().T
     assert torch.allclose(out.double().sum(0), want, atol=1e-3 * math.sqrt(k), rtol=1e-4)
 
 
+@pytest.mark.parametrize("form", [0, 1])
 @pytest.mark.parametrize("m", [1, 8, 40])
 @pytest.mark.parametrize("inter,k", [(176, 64), (18944, 3584), (250, 96)])
-def test_gemm_skinny_silu(m, inter, k):
+def test_gemm_skinny_silu(m, inter, k, form):
     ops = _ops()
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
     w = rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.1)
     out = torch.full((m, inter), float("nan"), device=DEV, dtype=torch.bfloat16)
-    ops.gemm_skinny_silu_bf16(x, w, out, m)
+    ops.gemm_skinny_silu_bf16(x, w, out, m, form)
     gu = x.double() @ w.double().T
     want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
     assert torch.allclose(out.double(), want, atol=2e-2, rtol=2e-2)
