@@ -57,6 +57,8 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--opt", action="append", default=[], metavar="KEY=VALUE",
+                    help="engine runtime option (kernel choice ablations), e.g. skinny_gemm=0")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -84,6 +86,9 @@ def main() -> int:
     state = random_state(model_tensor_specs(cfg), 0, 0.02, 0.0, TORCH_DTYPES[ec.dtype], device=dev)
     engine = Engine.from_state(cfg, state, ec)
     del state
+    for kv in args.opt:
+        k, v = kv.split("=", 1)
+        engine.runtime.options[k] = int(v)
     print(f"[bench] engine ready in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
     dtype_bytes = 2 if args.dtype == "bfloat16" else 4
     weight_bytes, kv_per_token, prefill_flops = model_numbers(cfg, n_layers, dtype_bytes)

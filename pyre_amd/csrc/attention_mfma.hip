@@ -65,32 +65,29 @@ struct Bounds {
 //   q[ct][c]   B operands of Q^T, c = 32-wide slice of the head
 //   o[dt][ct]  accumulators of O^T, dt = 16-wide slice of the head
 //   m, l       running max (in log2 units) and sum of each lane's column
-// `edge` says that some key of the chunk may be masked for some column or lie in
-// a page that is not there; interior chunks skip all masking.
-template <int HD, int CT>
-__device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bounds<CT>& bd,
-                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
-                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
-  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
-  int page[2], off[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int k0 = key0 + 16 * t;
-    page[t] = kv.table[k0 / kv.page_size];
-    off[t] = k0 % kv.page_size;
-  }
-
+//   load_k(t, c)  A operand of key tile t (16 keys), head slice c: lane (r, g) gets
+//                 K[key0 + 16 t + r][32 c + 8 g .. + 8]
+//   load_v(dt)    A operand of V^T rows 16 dt + r: slots 0..3 = keys 4g..4g+3 of
+//                 tile 0, slots 4..7 = the same keys of tile 1
+//   tile_ok[t]    false for a tile whose page is not there: all its keys are hidden
+// `edge` says that some key of the chunk may be hidden from some column;
+// interior chunks skip all masking.
+template <int HD, int CT, typename LoadK, typename LoadV>
+__device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2], const Bounds<CT>& bd,
+                                   float scale_log2, const bf16x8 (&q)[CT][HD / 32],
+                                   f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT],
+                                   LoadK&& load_k, LoadV&& load_v) {
+  const int g = (threadIdx.x & 63) >> 4;
   // S^T tiles: rows = keys key0 + 16 t + (4 g + j), columns = lane's column r.
   f32x4 s[2][CT];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) s[t][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (page[t] < 0) continue;  // released or never allocated: every key of it is masked
-    const bf16* kp = kv.k + ((static_cast<size_t>(page[t]) * kv.nkv + kv.kvh) * kv.page_size + off[t] + r) * HD + 8 * g;
+    if (!tile_ok[t]) continue;
 #pragma unroll
     for (int c = 0; c < HD / 32; ++c) {
-      const bf16x8 a = load_b128(kp + 32 * c);
+      const bf16x8 a = load_k(t, c);
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
         s[t][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[ct][c], s[t][ct], 0, 0, 0);
@@ -111,7 +108,7 @@ __device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bou
         float v = s[t][ct][j] * scale_log2;
         if (edge) {
           const int key = key0 + 16 * t + 4 * g + j;
-          if (page[t] < 0 || key < bd.lo[ct] || key > bd.hi[ct]) v = -INFINITY;
+          if (!tile_ok[t] || key < bd.lo[ct] || key > bd.hi[ct]) v = -INFINITY;
         }
         x[4 * t + j] = v;
         mx = fmaxf(mx, v);
@@ -137,27 +134,48 @@ __device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bou
     for (int dt = 0; dt < HD / 16; ++dt) o[dt][ct] *= alpha;
   }
 
-  // O^T += V^T P^T. Row of the A operand = output element d; its 8 slots are the
-  // same keys as P^T's: two runs of four keys, 8 bytes each in the transposed cache.
-  const bf16* vp[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-    vp[t] = page[t] < 0 ? nullptr
-                        : kv.v + ((static_cast<size_t>(page[t]) * kv.nkv + kv.kvh) * HD + r) * kv.page_size + off[t] + 4 * g;
+  // O^T += V^T P^T.
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
-    uint2 h[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      h[t] = uint2{0u, 0u};
-      if (vp[t]) h[t] = *reinterpret_cast<const uint2*>(vp[t] + static_cast<size_t>(dt) * 16 * kv.page_size);
-    }
-    const uint4 u = {h[0].x, h[0].y, h[1].x, h[1].y};
-    const bf16x8 a = __builtin_bit_cast(bf16x8, u);
+    const bf16x8 a = load_v(dt);
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
       o[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p[ct], o[dt][ct], 0, 0, 0);
   }
+}
+
+// The chunk's operands straight from the paged cache (no LDS): K rows as stored,
+// V^T as two runs of four keys, 8 bytes each in the transposed cache.
+template <int HD, int CT>
+__device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bounds<CT>& bd,
+                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
+                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const bf16* kp[2];
+  const bf16* vp[2];
+  bool ok[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int k0 = key0 + 16 * t;
+    const int page = kv.table[k0 / kv.page_size], off = k0 % kv.page_size;
+    ok[t] = page >= 0;  // released or never allocated: every key of it is hidden
+    const size_t base = static_cast<size_t>(ok[t] ? page : 0) * kv.nkv + kv.kvh;
+    kp[t] = kv.k + (base * kv.page_size + off + r) * HD + 8 * g;
+    vp[t] = kv.v + (base * HD + r) * kv.page_size + off + 4 * g;
+  }
+  attend_core<HD, CT>(
+      key0, edge, ok, bd, scale_log2, q, o, m, l,
+      [&](int t, int c) { return load_b128(kp[t] + 32 * c); },
+      [&](int dt) {
+        uint2 h[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          h[t] = uint2{0u, 0u};
+          if (ok[t]) h[t] = *reinterpret_cast<const uint2*>(vp[t] + static_cast<size_t>(dt) * 16 * kv.page_size);
+        }
+        const uint4 u = {h[0].x, h[0].y, h[1].x, h[1].y};
+        return __builtin_bit_cast(bf16x8, u);
+      });
 }
 
 // ---------------------------------------------------------------------------
@@ -315,6 +333,129 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Prefill with K and V staged through LDS: the NW waves of a block take NW query
+// heads of one key/value head over the same 32 tokens, so each chunk of keys is
+// read from memory once per block, double-buffered: the next chunk's loads are in
+// flight while the current one is multiplied.
+//   ks[stage][key][HD + 8]     rows padded so that 16 rows fall on different banks
+//   vs[stage][d][32 + 8]       V^T: 32 keys of the chunk per output element
+// ---------------------------------------------------------------------------
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_prefill_lds_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
+    int nq, int nkv, int page_size, float scale_log2, int window) {
+  constexpr int CT = 2, KS = HD + 8, VS = kChunk + 8, T = NW * 64;
+  constexpr int NPK = kChunk * HD / 8, NP = 2 * NPK;   // 16-byte pieces of K and of V per chunk
+  constexpr int PER = (NP + T - 1) / T;
+  __shared__ __attribute__((aligned(16))) bf16 ks[2][kChunk][KS];
+  __shared__ __attribute__((aligned(16))) bf16 vs[2][HD][VS];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+  const int n_rep = nq / nkv, hgroups = (n_rep + NW - 1) / NW;
+  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int hin = hg * NW + wave;
+  const bool active = hin < n_rep;           // a wave without a head still helps loading
+  const int head = kvh * n_rep + (active ? hin : 0);
+  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+  const int pos0 = positions[t0];
+  const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
+
+  Bounds<CT> bd;
+  bf16x8 qr[CT][HD / 32];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = 16 * ct + r;
+    const bool live = active && col < ntok;
+    bd.hi[ct] = col < ntok ? pos0 + col : pos0;
+    bd.lo[ct] = window > 0 ? max(0, bd.hi[ct] - window + 1) : 0;
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c)
+      qr[ct][c] = live ? load_b128(q + (static_cast<size_t>(t0 + col) * nq + head) * HD + 32 * c + 8 * g) : zero_b128();
+  }
+  f32x4 o[HD / 16][CT];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) o[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m[CT], l[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) { m[ct] = -INFINITY; l[ct] = 0.f; }
+
+  const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int hi_all = pos0 + ntok - 1;
+  const int first = lo_all / kChunk, last = hi_all / kChunk;
+  const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
+
+  // Piece p < NPK: K[key p / (HD/8)][8 (p % (HD/8)) ..]; else V^T[d][8 part ..] with
+  // d = (p - NPK) / 4, part = (p - NPK) % 4 (eight keys, always within one page).
+  auto fetch = [&](int key0, uint4 (&regs)[PER]) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = tid + i * T;
+      regs[i] = uint4{0u, 0u, 0u, 0u};
+      if (p >= NP) continue;
+      const bool is_k = p < NPK;
+      const int key = is_k ? key0 + p / (HD / 8) : key0 + 8 * ((p - NPK) % 4);
+      const int page = table[key / page_size], slot = key % page_size;
+      if (page < 0) continue;
+      const size_t base = static_cast<size_t>(page) * nkv + kvh;
+      const bf16* src = is_k ? k_cache + (base * page_size + slot) * HD + 8 * (p % (HD / 8))
+                             : v_cache + (base * HD + (p - NPK) / 4) * page_size + slot;
+      regs[i] = *reinterpret_cast<const uint4*>(src);
+    }
+  };
+  auto stash = [&](int stage, const uint4 (&regs)[PER]) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = tid + i * T;
+      if (p >= NP) continue;
+      if (p < NPK) *reinterpret_cast<uint4*>(&ks[stage][p / (HD / 8)][8 * (p % (HD / 8))]) = regs[i];
+      else *reinterpret_cast<uint4*>(&vs[stage][(p - NPK) / 4][8 * ((p - NPK) % 4)]) = regs[i];
+    }
+  };
+
+  uint4 regs[PER];
+  fetch(first * kChunk, regs);
+  stash(0, regs);
+  for (int c = first; c <= last; ++c) {
+    const int st = (c - first) & 1;
+    __syncthreads();  // chunk c is in stage st; nobody reads stage st ^ 1 any more
+    if (c < last) fetch((c + 1) * kChunk, regs);
+    const int key0 = c * kChunk;
+    if (active) {
+      const bool edge = key0 + kChunk - 1 > pos0 || key0 < lo_max;
+      const bool ok[2] = {true, true};  // a missing page holds zeros and its keys lie outside every column's bounds
+      attend_core<HD, CT>(
+          key0, edge, ok, bd, scale_log2, qr, o, m, l,
+          [&](int t, int cc) { return *reinterpret_cast<const bf16x8*>(&ks[st][16 * t + r][32 * cc + 8 * g]); },
+          [&](int dt) {
+            const uint2 lo = *reinterpret_cast<const uint2*>(&vs[st][16 * dt + r][4 * g]);
+            const uint2 hi = *reinterpret_cast<const uint2*>(&vs[st][16 * dt + r][16 + 4 * g]);
+            const uint4 u = {lo.x, lo.y, hi.x, hi.y};
+            return __builtin_bit_cast(bf16x8, u);
+          });
+    }
+    if (c < last) stash(st ^ 1, regs);
+  }
+
+  if (!active) return;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = 16 * ct + r;
+    if (col >= ntok) continue;
+    const float inv = 1.f / l[ct];
+    bf16* dst = out + (static_cast<size_t>(t0 + col) * nq + head) * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      const f32x4 v = o[dt][ct];
+      *reinterpret_cast<uint2*>(dst + dt * 16) = uint2{pack2(v[0] * inv, v[1] * inv), pack2(v[2] * inv, v[3] * inv)};
+    }
+  }
+}
+
 template <typename F>
 int dispatch_head(int hd, F&& f) {
   switch (hd) {
@@ -370,23 +511,42 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
                                       const void* v_cache, const int* tiles, int n_tiles,
                                       const int* positions, const int* seq_of_token,
                                       const int* block_table, int table_stride, int nq, int nkv,
-                                      int hd, int page_size, float scale, int window,
+                                      int hd, int page_size, float scale, int window, int form,
                                       hipStream_t stream) {
   PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
                "attn_prefill_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
   PYRE_REQUIRE(table_stride > 0, "attn_prefill_bf16: bad table");
   if (n_tiles <= 0) return 0;
-  const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
+  const int n_rep = nq / nkv;
+  const float scale_log2 = scale * kLog2e;
+  const bf16* qp = static_cast<const bf16*>(q);
+  const bf16* kp = static_cast<const bf16*>(k_cache);
+  const bf16* vp = static_cast<const bf16*>(v_cache);
+  bf16* op = static_cast<bf16*>(out);
+  // Up to 128 elements per head, K and V go through LDS (two stages fit in 64 KB);
+  // larger heads read the cache directly in every wave.
+  const bool staged = hd <= 128 && form != 0;
+  const int nw = staged ? (n_rep > 4 ? 8 : 4) : 4;
+  const int hgroups = (n_rep + nw - 1) / nw;
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
   const dim3 grid(n_tiles, nkv * hgroups);
-  const float scale_log2 = scale * kLog2e;
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
-    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
-                       static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache),
-                       static_cast<bf16*>(out), tiles, positions, seq_of_token, block_table, table_stride,
-                       nq, nkv, page_size, scale_log2, window);
+    if constexpr (HD <= 128) {
+      if (staged && nw == 8) {
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 8>), grid, dim3(512), 0, stream, qp, kp, vp, op, tiles,
+                           positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window);
+        return;
+      }
+      if (staged) {
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 4>), grid, dim3(256), 0, stream, qp, kp, vp, op, tiles,
+                           positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window);
+        return;
+      }
+    }
+    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, qp, kp, vp, op, tiles, positions,
+                       seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window);
   });
   PYRE_REQUIRE(rc == 0, "attn_prefill_bf16: no kernel for head_dim %d", hd);
   return check_launch("attn_prefill_bf16");

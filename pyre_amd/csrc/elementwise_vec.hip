@@ -38,11 +38,13 @@ __device__ inline float4 add4(float4 a, float4 b) { return float4{a.x + b.x, a.y
 // ---------------------------------------------------------------------------
 // add + RMSNorm, one block per row, the row kept in registers between the passes.
 // ---------------------------------------------------------------------------
-constexpr int kNormThreads = 256;
-constexpr int kNormMaxVec = 8;  // float4 per thread: rows of up to 8192 elements
+constexpr int kNormMaxVec = 8;  // float4 per thread
 
-template <typename TD, typename TG, typename TO>
-__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_vec_kernel(
+// THREADS = 256 keeps up to 8192 elements of a row in registers and suits many rows;
+// THREADS = 1024 gives a short row one float4 per thread, so that all loads of a
+// decode step's few rows are in flight at once.
+template <typename TD, typename TG, typename TO, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, int n_partials, size_t partial_stride,
     const TG* __restrict__ gain, TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
   __shared__ float scratch[16];
@@ -53,12 +55,21 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_vec_kernel(
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < kNormMaxVec; ++i) {
-    const int c = threadIdx.x + i * kNormThreads;
+    const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) break;
     float4 x = Vec4<float>::load(resid + in_off + 4 * c);
     if (delta) {
-      float4 d = Vec4<TD>::load(delta + in_off + 4 * c);
-      for (int p = 1; p < n_partials; ++p) d = add4(d, Vec4<TD>::load(delta + p * partial_stride + in_off + 4 * c));
+      const TD* dp = delta + in_off + 4 * c;
+      float4 d = Vec4<TD>::load(dp);
+      int p = 1;
+      for (; p + 3 < n_partials; p += 4) {  // four loads in flight, added in the order p, p+1, ...
+        const float4 d0 = Vec4<TD>::load(dp + p * partial_stride);
+        const float4 d1 = Vec4<TD>::load(dp + (p + 1) * partial_stride);
+        const float4 d2 = Vec4<TD>::load(dp + (p + 2) * partial_stride);
+        const float4 d3 = Vec4<TD>::load(dp + (p + 3) * partial_stride);
+        d = add4(add4(add4(add4(d, d0), d1), d2), d3);
+      }
+      for (; p < n_partials; ++p) d = add4(d, Vec4<TD>::load(dp + p * partial_stride));
       x = add4(x, d);
       if (!rows) Vec4<float>::store(resid + in_off + 4 * c, x);
     }
@@ -70,7 +81,7 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_vec_kernel(
   const size_t out_off = static_cast<size_t>(r_out) * hidden;
 #pragma unroll
   for (int i = 0; i < kNormMaxVec; ++i) {
-    const int c = threadIdx.x + i * kNormThreads;
+    const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) break;
     const float4 gn = Vec4<TG>::load(gain + 4 * c);
     const float4 x = v[i];
@@ -162,11 +173,18 @@ namespace pyre {
 bool add_rmsnorm_vec(float* resid, const void* delta, int delta_dt, int n_partials, long partial_stride,
                      const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
                      int hidden, float eps, hipStream_t stream) {
-  if (hidden % 4 || hidden > 4 * kNormThreads * kNormMaxVec || (delta && partial_stride % 4)) return false;
-  PYRE_DISPATCH(delta_dt, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO,
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO>), dim3(n), dim3(kNormThreads), 0, stream, resid,
+  if (hidden % 4 || hidden > 4 * 256 * kNormMaxVec || (delta && partial_stride % 4)) return false;
+  const bool few = n <= 128 && hidden > 1024;  // a decode step: spread each row over more threads
+  PYRE_DISPATCH(delta_dt, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO, {
+    if (few)
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, 1024>), dim3(n), dim3(1024), 0, stream, resid,
                          static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),
-                         static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps))));
+                         static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps);
+    else
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, 256>), dim3(n), dim3(256), 0, stream, resid,
+                         static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),
+                         static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps);
+  })));
   return true;
 }
 

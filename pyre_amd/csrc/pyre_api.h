@@ -11,6 +11,10 @@ extern "C" {
 const char* pyre_last_error();
 int pyre_abi_version();
 
+// Streams `bytes` of device memory through the chip and writes (almost) nothing:
+// a measurement of achievable read bandwidth.
+int pyre_read_probe(const void* p, size_t bytes, int blocks, unsigned* sink, hipStream_t stream);
+
 int pyre_embed(const void* table, int table_dt, const int* ids, float* out, int n, int hidden,
                hipStream_t stream);
 
@@ -66,11 +70,12 @@ int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache, const v
                           int page_size, float scale, int window, hipStream_t stream);
 
 // Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
-// all tokens of a tile from one request at consecutive positions.
+// all tokens of a tile from one request at consecutive positions. form 1 stages
+// K and V through LDS (heads of up to 128 elements), form 0 never does.
 int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
                            const int* tiles, int n_tiles, const int* positions,
                            const int* seq_of_token, const int* block_table, int table_stride,
-                           int nq, int nkv, int hd, int page_size, float scale, int window,
+                           int nq, int nkv, int hd, int page_size, float scale, int window, int form,
                            hipStream_t stream);
 
 // scratch: m * 64 floats followed by m * 64 ints of device memory.

@@ -21,6 +21,7 @@ class KernelError(RuntimeError):
 P, I, L, F = c_void_p, c_int, c_long, c_float
 
 _SIGNATURES = {
+    "pyre_read_probe": [P, ctypes.c_size_t, I, P, P],
     "pyre_embed": [P, I, P, P, I, I, P],
     "pyre_add_rmsnorm": [P, P, I, I, L, P, I, P, I, P, I, P, I, I, F, P],
     "pyre_rope_kv_write": [P, I, I, L, P, I, P, I, P, P, I, P, P, I, P, P, I, I, I, I, I, I, P],
@@ -30,7 +31,7 @@ _SIGNATURES = {
     "pyre_attn_generic": [P, P, I, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     "pyre_attn_mfma_supports": [I, I, I, I],
     "pyre_attn_decode_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
-    "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
+    "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
     "pyre_gemm_skinny_supports": [I, I, I, L, L],
     "pyre_gemm_skinny_bf16": [P, L, P, L, P, I, I, I, I, I, P],

@@ -300,13 +300,13 @@ def attn_decode_bf16(q, out, k_cache, v_cache, tokens, n_tokens, positions, seq_
 
 
 def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,
-                      nq, nkv, hd, page_size, scale, window=0) -> None:
+                      nq, nkv, hd, page_size, scale, window=0, form=1) -> None:
     """Attention of prompt portions; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32)."""
     _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
     _i32("tiles", tiles, 2 * n_tiles)
     call("pyre_attn_prefill_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
          tiles.data_ptr(), n_tiles, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
-         block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), _stream())
+         block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), int(form), _stream())
 
 
 def gemm_skinny_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
@@ -352,3 +352,22 @@ def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.T
         raise KernelError("gemm_skinny_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
     call("pyre_gemm_skinny_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
          out.data_ptr(), m, two_i, w_gate_up.shape[1], skinny_form(m) if form is None else form, _stream())
+
+
+def read_bandwidth(device: str = "cuda:0", gib: float = 2.0, blocks: int = 4096, repeats: int = 10) -> float:
+    """Measured streaming-read bandwidth in GB/s (a buffer larger than every cache)."""
+    import time
+
+    n = int(gib * (1 << 30)) // 16 * 16
+    buf = torch.empty(n, dtype=torch.uint8, device=device)
+    buf.zero_()
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+    with torch.cuda.device(buf.device):
+        for _ in range(2):
+            call("pyre_read_probe", buf.data_ptr(), n, blocks, sink.data_ptr(), _stream())
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(repeats):
+            call("pyre_read_probe", buf.data_ptr(), n, blocks, sink.data_ptr(), _stream())
+        torch.cuda.synchronize()
+    return n * repeats / (time.perf_counter() - t) / 1e9

@@ -19,7 +19,7 @@ SKINNY_MAX_ROWS = 64
 #: blocks a weight-streaming product is spread over at least, by form of the kernel
 SKINNY_TARGET_BLOCKS = {0: 2048, 1: 600}
 #: up to this many rows the gate/up product and the SiLU-gate are one kernel
-FUSED_SILU_MAX_ROWS = 8
+FUSED_SILU_MAX_ROWS = 4
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
@@ -84,16 +84,17 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
 
 
 #: waves the split of decode attention aims at (256 CUs x 8)
-DECODE_TARGET_WAVES = 2048
+DECODE_TARGET_WAVES = 4096
 DECODE_MAX_SPLITS = 128
 
 
-def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int) -> int:
+def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
+                  target_waves: int = DECODE_TARGET_WAVES) -> int:
     """How many ways to split each request's keys so that the chip is full."""
     span = min(max_ctx, window + 32) if window > 0 else max_ctx
     chunks = max(1, -(-span // 32))
     items = n_tokens * nkv * -(-(nq // nkv) // 16)
-    return max(1, min(chunks, DECODE_MAX_SPLITS, -(-DECODE_TARGET_WAVES // items)))
+    return max(1, min(chunks, DECODE_MAX_SPLITS, -(-target_waves // items)))
 
 
 def attention(mixer, ctx, q, o, cache) -> bool:
@@ -110,7 +111,8 @@ def attention(mixer, ctx, q, o, cache) -> bool:
     n_dec, n_tiles = len(hb.decode_tokens), len(hb.prefill_tiles)
     if n_dec:
         nsplits = ctx.runtime.options.get("decode_splits") or decode_splits(
-            n_dec, s.num_heads, s.num_kv_heads, hb.max_decode_ctx, cache.window)
+            n_dec, s.num_heads, s.num_kv_heads, hb.max_decode_ctx, cache.window,
+            ctx.runtime.options.get("decode_target_waves", DECODE_TARGET_WAVES))
         acc = ctx.workspace.get("attn.part_acc", (n_dec, s.num_heads, nsplits, s.head_dim), torch.float32)
         ml = ctx.workspace.get("attn.part_ml", (n_dec, s.num_heads, nsplits, 2), torch.float32)
         ops.attn_decode_bf16(q, o, cache.k, cache.v, ctx.decode_tokens, n_dec, ctx.positions,

@@ -266,9 +266,10 @@ def test_attn_decode_mfma(nq, nkv, hd, page, window, nsplits):
     assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("form", [0, 1])
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 50])
-def test_attn_prefill_mfma(nq, nkv, hd, page, window):
+def test_attn_prefill_mfma(nq, nkv, hd, page, window, form):
     ops = _ops()
     from pyre_amd.engine.batch import TILE
 
@@ -280,7 +281,7 @@ def test_attn_prefill_mfma(nq, nkv, hd, page, window):
         tiles += [(t0, min(TILE, base + ql - t0)) for t0 in range(base, base + ql, TILE)]
         base += ql
     scale = hd ** -0.5
-    ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), len(tiles), pos, seq_of, table, nq, nkv, hd, page, scale, window)
+    ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), len(tiles), pos, seq_of, table, nq, nkv, hd, page, scale, window, form)
     want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
     assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
 
