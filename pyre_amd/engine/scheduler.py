@@ -7,8 +7,10 @@ whole prompt alone at admission and then decodes all running requests
 (`pyre/scheduler.py:46-97`); here portions of prompts ride in the same step as the
 decoded tokens of the others.
 
-When pages run out: a request is admitted only if pages for its first portion are
-free; if a running request needs a page and none is free, the request admitted
+When pages run out: a request is admitted only if the pages for all the tokens it
+has so far (its prompt, and what it generated before a preemption) are free beside
+those that running prompts are still going to take, with one page to spare for
+every running request; if a running request needs a page and none is free, the request admitted
 last is preempted: its pages and slot are given back and it re-enters the front
 of the waiting queue to be recomputed from its prompt and the tokens it has
 generated so far (which it keeps). A request that could not fit the pool even
@@ -156,21 +158,28 @@ class Scheduler:
             i += 1
 
         # 2. admit waiting requests, first come first served (pyre/scheduler.py:49-50)
+        # Pages that running prompts will still take in later steps are spoken for.
+        planned = {e.request.seq_id: e.count for e in entries}
+        promised = sum(
+            self.cache.pages_needed(r.seq_id, r.cur_len - r.num_computed)
+            - self.cache.pages_needed(r.seq_id, planned.get(r.seq_id, 0)) for r in self.running)
         while (self.waiting and not preempted and budget > 0 and len(self.running) < self.max_batch
                and self.cache.has_free_slot()):
             r = self.waiting[0]
             n = portion(r, budget)
-            need = self.cache.pages_needed(None, n)
+            need_now = self.cache.pages_needed(None, n)
+            need_all = self.cache.pages_needed(None, r.cur_len)
             # One page of headroom for every running request, so that an admission
             # is not undone by the very next decoded token.
-            if need + len(self.running) > free:
+            if need_all + promised + len(self.running) > free:
                 break
             self.waiting.pop(0)
             self.running.append(r)
             self.cache.add_request(r.seq_id)
             admitted.append(r)
             entries.append(PlannedEntry(r, 0, n, n == r.cur_len))
-            free -= need
+            free -= need_now
+            promised += need_all - need_now
             budget -= n
         return StepPlan(entries, preempted, admitted)
 

@@ -112,8 +112,11 @@ def causal_attention(q, k, v, scale: float, window: int = 0) -> torch.Tensor:
     return torch.matmul(torch.softmax(scores, dim=-1), v)
 
 
-def attention_block(h, w: dict, prefix: str, cfg: dict, cos, sin, rnd) -> torch.Tensor:
-    """pyre/model.py:89-125 for one sequence at start_pos = 0. h: (S, H)."""
+def attention_block(h, w: dict, prefix: str, cfg: dict, cos, sin, rnd, window: int = 0, kv=None, keep=None) -> torch.Tensor:
+    """pyre/model.py:89-125 for one sequence at start_pos = 0. h: (S, H).
+    Not in the reference: ``window``; ``kv`` = rotated keys and values of another
+    layer to attend over instead of this layer's own; ``keep`` = a list that
+    receives this layer's (keys, values)."""
     S = h.shape[0]
     nq, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     q = (h @ w[f"{prefix}.q_proj.weight"].T + w[f"{prefix}.q_proj.bias"]).view(S, nq, hd).transpose(0, 1)
@@ -121,8 +124,12 @@ def attention_block(h, w: dict, prefix: str, cfg: dict, cos, sin, rnd) -> torch.
     v = (h @ w[f"{prefix}.v_proj.weight"].T + w[f"{prefix}.v_proj.bias"]).view(S, nkv, hd).transpose(0, 1)
     q, k = apply_rope(q, k, cos[:S], sin[:S])
     q, k, v = rnd(q), rnd(k), rnd(v)
+    if keep is not None:
+        keep.append((k, v))
+    if kv is not None:
+        k, v = kv
     k, v = repeat_kv(k, nq // nkv), repeat_kv(v, nq // nkv)
-    out = causal_attention(q, k, v, hd ** -0.5)
+    out = causal_attention(q, k, v, hd ** -0.5, window)
     out = rnd(out.transpose(0, 1).reshape(S, nq * hd))
     return out @ w[f"{prefix}.o_proj.weight"].T
 

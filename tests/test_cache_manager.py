@@ -1,0 +1,219 @@
+"""The cache manager's bookkeeping (CPU): allocator vectors of the reference's tests,
+block tables, groups, windows, slots, and invariants under random orders."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+
+from pyre_amd.cache import RELEASED, CacheManager, OutOfPages, PageAllocator
+from pyre_amd.parts.base import KVCacheSpec, StateCacheSpec
+
+FULL = KVCacheSpec(2, 16)
+WIN = KVCacheSpec(2, 16, window=40)
+
+
+# --- the reference's allocator tests (tests/test_paged_cache.py:23-66) ------------
+
+def test_allocate_and_free_roundtrip():
+    a = PageAllocator(4)
+    pages = [a.allocate() for _ in range(4)]
+    assert a.num_free == 0 and len(set(pages)) == 4
+    for p in pages:
+        a.free(p)
+    assert a.num_free == 4 and a.num_used == 0
+
+
+def test_exhaustion_raises():
+    a = PageAllocator(2)
+    a.allocate(), a.allocate()
+    with pytest.raises(MemoryError, match="exhausted"):
+        a.allocate()
+    with pytest.raises(OutOfPages):
+        a.allocate_many(1)
+
+
+def test_freed_pages_are_reused_at_once():
+    a = PageAllocator(2)
+    p0 = a.allocate()
+    a.allocate()
+    a.free(p0)
+    assert a.allocate() == p0
+
+
+def test_double_free_raises():
+    a = PageAllocator(2)
+    p = a.allocate()
+    a.free(p)
+    with pytest.raises(ValueError, match="double free"):
+        a.free(p)
+    with pytest.raises(ValueError):
+        a.free(1)            # never allocated
+
+
+def test_allocate_many_is_all_or_nothing():
+    a = PageAllocator(3)
+    a.allocate()
+    with pytest.raises(OutOfPages):
+        a.allocate_many(3)
+    assert a.num_free == 2
+
+
+# --- block tables (tests/test_paged_cache.py:69-102) -----------------------------
+
+def manager(specs=(FULL, FULL), pages=8, seqs=4, page_size=16, max_len=256):
+    return CacheManager(list(specs), page_size, pages, seqs, max_len)
+
+
+def test_seventeen_tokens_take_two_pages():
+    m = manager()
+    m.add_request("a")
+    m.reserve("a", 17)
+    assert len(m.block_table("a", 0)) == 2 and m.page_groups[0].allocator.num_used == 2
+    m.commit("a", 17)
+    m.reserve("a", 15)                                   # 32 tokens still fit two pages
+    assert len(m.block_table("a", 0)) == 2
+    m.commit("a", 15)
+    m.reserve("a", 1)
+    assert len(m.block_table("a", 0)) == 3
+
+
+def test_free_returns_everything_and_requests_are_disjoint():
+    m = manager()
+    m.add_request("a"), m.add_request("b")
+    m.reserve("a", 48), m.reserve("b", 16)
+    assert set(m.block_table("a", 0)).isdisjoint(m.block_table("b", 0))
+    assert m.slot("a") != m.slot("b")
+    m.check_invariants()
+    m.free_request("a")
+    assert "a" not in m and m.page_groups[0].allocator.num_used == 1
+    m.free_request("b")
+    assert m.page_groups[0].allocator.num_used == 0 and m.slots.num_used == 0
+    with pytest.raises(ValueError, match="already exists"):
+        m.add_request("c"), m.add_request("c")
+
+
+def test_slot_mapping_follows_the_table():
+    m = manager(page_size=8)
+    m.add_request("a")
+    m.reserve("a", 20)
+    t = m.block_table("a", 0)
+    got = m.slot_mapping("a", 0, 5, 6)                   # positions 5..10 cross a page edge
+    assert got == [t[0] * 8 + 5, t[0] * 8 + 6, t[0] * 8 + 7, t[1] * 8 + 0, t[1] * 8 + 1, t[1] * 8 + 2]
+
+
+def test_reserve_takes_all_pages_or_none():
+    m = manager(pages=3)
+    m.add_request("a"), m.add_request("b")
+    m.reserve("a", 32)
+    with pytest.raises(OutOfPages):
+        m.reserve("b", 33)                               # needs 3, 1 free
+    assert m.block_table("b", 0) == [] and m.page_groups[0].allocator.num_free == 1
+    m.check_invariants()
+    with pytest.raises(ValueError, match="limit"):
+        m.reserve("a", 1000)
+    with pytest.raises(RuntimeError, match="reservation"):
+        m.commit("b", 5)
+
+
+def test_slots_run_out_separately():
+    m = manager(seqs=2)
+    m.add_request(1), m.add_request(2)
+    assert not m.has_free_slot()
+    with pytest.raises(OutOfPages, match="slot"):
+        m.add_request(3)
+
+
+# --- groups -----------------------------------------------------------------------
+
+def test_layers_with_the_same_needs_share_a_group():
+    specs = [FULL, WIN, FULL, None, StateCacheSpec((4, 8)), WIN, StateCacheSpec((4, 8))]
+    m = CacheManager(specs, 16, 10, 4, 512)
+    assert [g.entries for g in m.page_groups] == [[0, 2], [1, 5]]
+    assert [g.entries for g in m.state_groups] == [[4, 6]]
+    assert m.group_of_entry == {0: ("kv", 0), 2: ("kv", 0), 1: ("kv", 1), 5: ("kv", 1), 4: ("state", 0), 6: ("state", 0)}
+    assert m.page_groups[1].layer_index(5) == 1
+    assert m.bytes_per_page(2) == 2 * (2 * 2 * 16 * 16 * 2) * 2
+
+
+def test_a_window_gives_pages_back_once_passed():
+    m = CacheManager([FULL, WIN], 16, 12, 2, 512)
+    m.add_request("a")
+    m.reserve("a", 100)
+    m.commit("a", 100)
+    full, win = m.block_table("a", 0), m.block_table("a", 1)
+    # next query at 100 sees keys 61..100: keys <= 60 are dead: pages 0..2 (keys 0..47) go, page 3 (48..63) stays
+    assert win[:3] == [RELEASED] * 3 and all(p != RELEASED for p in win[3:]) and RELEASED not in full
+    assert m.page_groups[1].allocator.num_used == 4 and m.page_groups[0].allocator.num_used == 7
+    with pytest.raises(RuntimeError, match="released"):
+        m.slot_mapping("a", 1, 40, 1)
+    for _ in range(30):                                   # decoding on: the window slides, pages keep coming back
+        m.reserve("a", 1)
+        m.commit("a", 1)
+    m.check_invariants()
+    assert m.page_groups[1].allocator.num_used <= 4
+    m.free_request("a")
+    assert all(g.allocator.num_used == 0 for g in m.page_groups)
+
+
+def test_window_release_never_hides_a_visible_key():
+    """For every way of cutting a request into portions, each query's window
+    [p - w + 1, p] lies in pages that are still held when the portion runs."""
+    rng = random.Random(4)
+    for _ in range(50):
+        w, ps = rng.choice([1, 5, 16, 33]), rng.choice([4, 16])
+        m = CacheManager([KVCacheSpec(1, 8, window=w)], ps, 64, 1, 400)
+        m.add_request(0)
+        total = 0
+        while total < 300:
+            n = rng.choice([1, 1, 2, 7, 40])
+            m.reserve(0, n)
+            table = m.block_table(0, 0)
+            first_query = total
+            for key in range(max(0, first_query - w + 1), total + n):
+                assert table[key // ps] != RELEASED
+            m.commit(0, n)
+            total += n
+        m.free_request(0)
+        assert m.page_groups[0].allocator.num_used == 0
+
+
+# --- random orders -----------------------------------------------------------------
+
+@pytest.mark.parametrize("seed", range(8))
+def test_no_page_lost_held_twice_or_freed_twice(seed):
+    rng = random.Random(seed)
+    m = CacheManager([FULL, WIN, StateCacheSpec((3,))], rng.choice([4, 16]), 40, 6, 300)
+    live, next_id = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and m.has_free_slot():
+            m.add_request(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 3, 17, 50])
+            try:
+                m.reserve(rid, n)
+            except OutOfPages:
+                victim = rng.choice(list(live))            # what a scheduler would do: give one up
+                m.free_request(victim)
+                del live[victim]
+            except ValueError:
+                m.free_request(rid)                        # reached the longest length
+                del live[rid]
+            else:
+                m.commit(rid, n)
+                live[rid] += n
+                assert m.length(rid) == live[rid]
+        elif live:
+            rid = rng.choice(list(live))
+            m.free_request(rid)
+            del live[rid]
+        m.check_invariants()
+        assert set(m.live_requests) == set(live)
+    for rid in list(live):
+        m.free_request(rid)
+    assert all(g.allocator.num_used == 0 for g in m.page_groups) and m.slots.num_used == 0

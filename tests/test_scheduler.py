@@ -1,0 +1,189 @@
+"""The scheduler's decisions (CPU), with a stand-in engine: admission, token budget,
+portions, finishing, and what happens when pages run out."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import pytest
+
+from pyre_amd.cache import CacheManager
+from pyre_amd.engine.scheduler import Scheduler
+from pyre_amd.parts.base import KVCacheSpec
+
+
+@dataclass
+class FakeConfig:
+    max_num_seqs: int = 4
+    max_num_batched_tokens: int = 64
+    prefill_chunk: int = 32
+
+
+class FakeEngine:
+    """Keeps the real cache bookkeeping; its "logits" are the entries themselves."""
+
+    vocab_size = 100
+
+    def __init__(self, pages=64, page_size=16, max_len=512, **cfg):
+        self.engine_config = FakeConfig(**cfg)
+        self.cache = CacheManager([KVCacheSpec(1, 8)], page_size, pages, self.engine_config.max_num_seqs, max_len)
+        self.max_model_len = max_len
+        self.steps = []
+
+    def step(self, entries):
+        for e in entries:
+            if e.rid not in self.cache:
+                self.cache.add_request(e.rid)
+        for e in entries:
+            self.cache.reserve(e.rid, len(e.tokens))
+        for e in entries:
+            self.cache.commit(e.rid, len(e.tokens))
+        self.cache.check_invariants()
+        self.steps.append([(e.rid, len(e.tokens), list(e.want)) for e in entries])
+        return [e for e in entries if e.want]
+
+    def finish(self, rid):
+        self.cache.free_request(rid)
+
+
+class FakeSampler:
+    """Next token = (sum of the request's tokens so far) mod vocabulary: a function of
+    the request alone, like a real model's greedy choice."""
+
+    def __init__(self, sched):
+        self.sched = sched
+
+    def sample(self, rows, temps, us):
+        out = []
+        for e in rows:
+            r = next(x for x in self.sched.running if x.seq_id == e.rid)
+            out.append(sum(r.tokens) % 100)
+        return out
+
+
+def make(**kw):
+    eng = FakeEngine(**kw)
+    s = Scheduler(eng)
+    s.sampler = FakeSampler(s)
+    return eng, s
+
+
+def expected(prompt, n, eos=None):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = sum(toks) % 100
+        toks.append(t)
+        out.append(t)
+        if eos is not None and t == eos:
+            break
+    return out
+
+
+def test_portions_under_the_budget_and_decodes_first():
+    eng, s = make()
+    a = s.add_request(list(range(1, 71)), 5)                 # 70 tokens: 32 + 32 + 6
+    s.step()
+    assert eng.steps[-1] == [(a, 32, [])]
+    b = s.add_request([7] * 10, 5)
+    s.step()                                                 # a's second portion, then b whole
+    assert eng.steps[-1] == [(a, 32, []), (b, 10, [9])]
+    s.step()                                                 # oldest first: a's last portion, then b's decoded token
+    assert eng.steps[-1] == [(a, 6, [5]), (b, 1, [0])]
+    s.step()
+    assert eng.steps[-1] == [(a, 1, [0]), (b, 1, [0])]
+    out = s.run()
+    assert out[a] == expected(range(1, 71), 5) and out[b] == expected([7] * 10, 5)
+    assert eng.cache.page_groups[0].allocator.num_used == 0 and not s.has_work
+
+
+def test_budget_caps_a_step():
+    eng, s = make(max_num_batched_tokens=40)
+    for _ in range(3):
+        s.add_request([1] * 30, 2)
+    s.step()
+    assert [n for _, n, _ in eng.steps[-1]] == [30, 10]       # the second prompt is cut by the budget
+    s.step()
+    assert sum(n for _, n, _ in eng.steps[-1]) <= 40
+    s.run()
+
+
+def test_max_batch_and_first_come_first_served():
+    eng, s = make(max_num_seqs=2)
+    ids = [s.add_request([i + 1] * 4, 3) for i in range(4)]
+    s.step()
+    assert [r for r, _, _ in eng.steps[-1]] == ids[:2]
+    out = s.run()
+    assert list(out) == ids and all(len(v) == 3 for v in out.values())
+    assert max(len(st) for st in eng.steps) == 2
+
+
+def test_finishing_by_length_and_by_eos():
+    eng, s = make()
+    p = [3, 4]
+    toks = expected(p, 6)
+    a = s.add_request(p, 6, eos_id=toks[2])
+    b = s.add_request(p, 6, eos_id=toks[2], ignore_eos=True)
+    c = s.add_request(p, 1)                                   # one new token means one (pyre/scheduler.py:84 gives two)
+    out = s.run()
+    assert out[a] == toks[:3] and s.finished[a].finish_reason == "eos"
+    assert out[b] == toks and s.finished[b].finish_reason == "length"
+    assert out[c] == toks[:1]
+    assert [n for st in eng.steps for r, n, _ in st if r == c] == [2]   # a finished request never enters a step again
+
+
+def test_requests_that_can_never_run_are_refused():
+    eng, s = make(pages=4, max_len=512)
+    with pytest.raises(ValueError, match="could never run"):
+        s.add_request([1] * 60, 10)                           # 69 cached tokens = 5 pages > 4
+    s.add_request([1] * 55, 10)                               # 64 cached tokens = 4 pages: fits alone
+    with pytest.raises(ValueError, match="longest request"):
+        s.add_request([1] * 500, 20)
+    with pytest.raises(ValueError, match="vocabulary"):
+        s.add_request([100], 2)
+    with pytest.raises(ValueError, match="at least one"):
+        s.add_request([], 2)
+    assert len(s.run()) == 1
+
+
+def test_no_admission_without_pages():
+    eng, s = make(pages=6)
+    a = s.add_request([1] * 60, 4)                            # 4 pages
+    b = s.add_request([2] * 40, 4)                            # 3 pages: does not fit beside a
+    while s.running or not s.finished:
+        s.step()
+        if a in s.finished:
+            break
+        assert all(r == a for r, _, _ in eng.steps[-1])
+    out = s.run()
+    assert out[a] == expected([1] * 60, 4) and out[b] == expected([2] * 40, 4)
+    assert s.finished[b].preemptions == 0
+
+
+def test_preemption_takes_the_latest_and_recomputes():
+    """Two requests fit at admission but not when both grow: the one admitted last
+    goes back to the front of the queue, keeps its tokens, and is recomputed."""
+    eng, s = make(pages=5, max_num_seqs=4)
+    a = s.add_request([1] * 30, 40)                           # grows to 69 cached tokens: 5 pages alone
+    b = s.add_request([2] * 14, 40)
+    c = s.add_request([3] * 5, 3)
+    out = s.run()
+    assert out[a] == expected([1] * 30, 40) and out[b] == expected([2] * 14, 40) and out[c] == expected([3] * 5, 3)
+    assert s.finished[a].preemptions == 0 and s.finished[b].preemptions >= 1
+    # after a preemption the victim's next entry starts from position 0 again and covers prompt + generated
+    first_again = [st for st in eng.steps if any(r == b and n > 1 for r, n, _ in st)]
+    assert len(first_again) >= 2
+    assert eng.cache.page_groups[0].allocator.num_used == 0 and eng.cache.slots.num_used == 0
+
+
+def test_batched_equals_alone():
+    """tests/test_scheduler.py:20-64 of the reference: caps 24/16/32, different prompts."""
+    prompts = {0: [5] * 9, 1: [8, 1, 4], 2: list(range(20))}
+    caps = {0: 24, 1: 16, 2: 32}
+    eng, s = make(pages=32)
+    ids = {s.add_request(prompts[i], caps[i]): i for i in prompts}
+    together = {ids[k]: v for k, v in s.run().items()}
+    for i in prompts:
+        e2, s2 = make(pages=32)
+        sid = s2.add_request(prompts[i], caps[i])
+        assert s2.run()[sid] == together[i]
+    assert not s.running and not s.waiting
