@@ -1,0 +1,46 @@
+"""Per-kernel totals of a rocprofv3 kernel trace.
+
+    python -m pyre_amd.profile_summary RESULTS.db [TOP] [--match TEXT]
+
+reads the ``kernels`` view of the rocpd SQLite file that
+``rocprofv3 --kernel-trace --stats -d DIR -o NAME -- <program>`` writes
+(``DIR/NAME_results.db``) and prints calls, total, share, mean, min and max time per
+kernel name, longest total first.
+"""
+
+from __future__ import annotations
+
+import sqlite3
+import sys
+
+
+def summarise(path: str, top: int = 25, match: str | None = None) -> str:
+    con = sqlite3.connect(path)
+    rows = con.execute("select name, count(*), sum(end - start), min(end - start), max(end - start) "
+                       "from kernels group by name order by 3 desc").fetchall()
+    if match:
+        rows = [r for r in rows if match in r[0]]
+    total = sum(r[2] for r in rows) or 1
+    out = [f"total kernel time {total / 1e6:.3f} ms over {sum(r[1] for r in rows)} launches",
+           f"{'kernel':72s} {'calls':>7s} {'total ms':>10s} {'%':>6s} {'avg us':>9s} {'min us':>9s} {'max us':>9s}"]
+    for name, calls, t, mn, mx in rows[:top]:
+        out.append(f"{name[:72]:72s} {calls:7d} {t / 1e6:10.3f} {100 * t / total:6.2f} {t / calls / 1e3:9.1f} "
+                   f"{mn / 1e3:9.1f} {mx / 1e3:9.1f}")
+    return "\n".join(out)
+
+
+def main(argv: list[str]) -> int:
+    if not argv:
+        print(__doc__)
+        return 2
+    match = None
+    if "--match" in argv:
+        i = argv.index("--match")
+        match = argv[i + 1]
+        del argv[i:i + 2]
+    print(summarise(argv[0], int(argv[1]) if len(argv) > 1 else 25, match))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))
