@@ -362,7 +362,7 @@ extern "C" int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, lon
   PYRE_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_skinny_bf16: ksplit=%d", ksplit);
   const int mt = (M + 15) / 16;
   const int tiles = (N + 15) / 16;
-  if (form == 1) {  // waves on different tiles, X through LDS
+  if ((form & 15) == 1) {  // waves on different tiles, X through LDS
     const int rt = tiles >= 2048 ? 2 : 1;
     const int kper = ((K + ksplit - 1) / ksplit + kRun - 1) / kRun * kRun;
     const dim3 grid((tiles + 4 * rt - 1) / (4 * rt), ksplit);
@@ -373,15 +373,21 @@ extern "C" int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, lon
     PYRE_REQUIRE(rc == 0, "gemm_skinny_bf16: no kernel for %d rows", M);
     return check_launch("gemm_skinny_bf16");
   }
-  const int rt = tiles >= 4096 ? 2 : 1;  // wide products: two tiles per block halve the reads of X
+  // Form 0: tiles per block. More tiles per block mean fewer reads of X (each block
+  // reads all of X's k range once) but fewer blocks; `form` may carry a choice in
+  // its upper bits (form = 0 + 16 * tiles), else it is made from the sizes.
+  int rt = form >> 4;
+  if (rt == 0) rt = tiles >= 4096 ? 2 : 1;  // measured: more tiles per block only pay for very wide products
   // k per block, a multiple of what its four waves take in one round
   const int kper = ((K + ksplit - 1) / ksplit + 4 * kRun - 1) / (4 * kRun) * (4 * kRun);
   const dim3 grid((tiles + rt - 1) / rt, ksplit);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
-  int rc = rt == 2 ? launch<2, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper)
-                   : launch<1, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
-  PYRE_REQUIRE(rc == 0, "gemm_skinny_bf16: no kernel for %d rows", M);
+  int rc = 1;
+  if (rt == 4) rc = launch<4, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
+  else if (rt == 2) rc = launch<2, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
+  else if (rt == 1) rc = launch<1, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
+  PYRE_REQUIRE(rc == 0, "gemm_skinny_bf16: no kernel for %d rows, %d tiles per block", M, rt);
   return check_launch("gemm_skinny_bf16");
 }
 

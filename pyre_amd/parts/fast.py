@@ -17,15 +17,16 @@ from pyre_amd.hip.ops import Partials
 #: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the BLAS library
 SKINNY_MAX_ROWS = 64
 #: blocks a weight-streaming product is spread over at least, by form of the kernel
-SKINNY_TARGET_BLOCKS = {0: 2048, 1: 600}
+SKINNY_TARGET_BLOCKS = {0: 6000, 1: 900}
+SKINNY_MAX_KSPLIT = 12
 #: up to this many rows the gate/up product and the SiLU-gate are one kernel
 FUSED_SILU_MAX_ROWS = 4
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
     """Blocks per output tile, so that a product with few columns still fills the chip
-    (measured on the 7B shapes: more than ~2,000 blocks of form 0 or ~600 of form 1
-    bring nothing, fewer leave bandwidth unused)."""
+    (measured on the 7B shapes with weights that are not in cache: about 6,000
+    blocks of form 0 or 900 of form 1, and never more than 12 partial sums)."""
     from pyre_amd.hip.ops import skinny_form
 
     form = skinny_form(m)
@@ -34,7 +35,7 @@ def skinny_ksplit(m: int, n_out: int, k: int) -> int:
         blocks = -(-tiles // 2) if tiles >= 4096 else tiles
     else:
         blocks = -(-tiles // (8 if tiles >= 2048 else 4))
-    return max(1, min(-(-SKINNY_TARGET_BLOCKS[form] // blocks), k // 512, 64))
+    return max(1, min(-(-SKINNY_TARGET_BLOCKS[form] // blocks), k // 512, SKINNY_MAX_KSPLIT))
 
 
 def _is_bf16(ctx, lin, x) -> bool:
