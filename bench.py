@@ -57,6 +57,7 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-tune", action="store_true", help="keep the BLAS library's default kernels for prefill")
     ap.add_argument("--opt", action="append", default=[], metavar="KEY=VALUE",
                     help="engine runtime option (kernel choice ablations), e.g. skinny_gemm=0")
     args = ap.parse_args()
@@ -82,7 +83,7 @@ def main() -> int:
     ec = EngineConfig(dtype=args.dtype, device=dev, page_size=16, max_num_seqs=max_batch,
                       max_cached_tokens=max_batch * args.context + 64 * 16, max_model_len=args.context,
                       max_num_batched_tokens=PREFILL_TOKENS, prefill_chunk=PREFILL_TOKENS,
-                      use_graphs=not args.no_graphs)
+                      use_graphs=not args.no_graphs, tune_gemm_rows=() if args.no_tune else (PREFILL_TOKENS,))
     state = random_state(model_tensor_specs(cfg), 0, 0.02, 0.0, TORCH_DTYPES[ec.dtype], device=dev)
     engine = Engine.from_state(cfg, state, ec)
     del state
@@ -165,7 +166,8 @@ def main() -> int:
                    "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
                    "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "page_size": 16,
-                   "prefill_tokens": PREFILL_TOKENS, "graphs": bool(ec.use_graphs)},
+                   "prefill_tokens": PREFILL_TOKENS, "graphs": bool(ec.use_graphs),
+                   "blas_tuned_rows": PREFILL_TOKENS if ec.tune_gemm_rows else 0},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

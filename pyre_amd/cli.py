@@ -35,6 +35,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
     ap.add_argument("--prefill-chunk", type=int, default=512)
     ap.add_argument("--max-model-len", type=int, default=None)
+    ap.add_argument("--tune-gemm-rows", type=int, nargs="*", default=[],
+                    help="step sizes for which the BLAS library's kernels are timed at start-up")
     ap.add_argument("--out", default=None, help="write a JSON result file")
     return ap
 
@@ -47,7 +49,7 @@ def main(argv: list[str] | None = None) -> int:
         args.model, device=args.device, dtype=args.dtype, random_seed=args.random_seed,
         num_blocks=args.num_blocks, page_size=args.page_size, max_num_seqs=args.max_batch,
         max_num_batched_tokens=args.max_num_batched_tokens, prefill_chunk=args.prefill_chunk,
-        max_model_len=args.max_model_len)
+        max_model_len=args.max_model_len, tune_gemm_rows=tuple(args.tune_gemm_rows))
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     if args.prompt_len is not None:
         rng = random.Random(args.seed)

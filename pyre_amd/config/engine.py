@@ -27,6 +27,9 @@ class EngineConfig:
     prefill_chunk: int = 512         #: largest portion of one prompt in a step
     max_model_len: int | None = None  #: longest request; None: the model's max positions
     use_graphs: bool = True          #: capture decode-only steps in HIP graphs
+    #: row counts (tokens in a step) for which the BLAS library is asked, once at start-up,
+    #: to time its kernels for this model's many-row 16-bit products and keep the fastest
+    tune_gemm_rows: tuple = ()
 
     def __post_init__(self) -> None:
         if self.dtype not in DTYPE_NAMES:

@@ -56,6 +56,8 @@ class Engine:
         #: captured decode steps: (rows, table width) -> "warm" (ran eagerly once) or (graph, logits)
         self._graphs: dict[tuple[int, int], object] = {}
         self.graph_replays = 0
+        if ec.tune_gemm_rows and self.dtype == torch.bfloat16:
+            self.tune_library_gemms(ec.tune_gemm_rows)
 
     # ------------------------------------------------------------------ construction
 
@@ -99,6 +101,57 @@ class Engine:
             model.bind(tensors, rt)
             tensors.clear()
             return cls(model, config, ec)
+
+    def tune_library_gemms(self, rows) -> int:
+        """For steps of exactly ``rows`` tokens (any of them), let the BLAS front end
+        time the vendor libraries' kernels for each distinct many-row 16-bit product of
+        this model and remember the fastest (torch's TunableOp). Other row counts keep
+        the libraries' own choice. Returns the number of products tuned."""
+        import os
+        import tempfile
+
+        import torch.cuda.tunable as tunable
+
+        from pyre_amd.parts.fast import SKINNY_MAX_ROWS
+        from pyre_amd.parts.linear import Linear
+
+        shapes = {}
+
+        def walk(obj, depth=0):
+            if isinstance(obj, Linear):
+                if obj.weight is not None and obj.weight.dtype == torch.bfloat16:
+                    shapes.setdefault((obj.out_features, obj.in_features), obj)
+                return
+            if depth > 4 or not hasattr(obj, "__dict__"):
+                return
+            for v in vars(obj).values():
+                for item in (v if isinstance(v, (list, tuple)) else [v]):
+                    if hasattr(item, "__dict__") and type(item).__module__.startswith(("pyre_amd", "test", "tests")):
+                        walk(item, depth + 1)
+
+        walk(self.model)
+        tunable.enable(True)
+        if hasattr(tunable, "write_file_on_exit"):
+            tunable.write_file_on_exit(False)
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), f"pyre_amd_tunable_{os.getpid()}.csv"))
+        tunable.set_max_tuning_duration(30)
+        tunable.set_max_tuning_iterations(20)
+        tunable.tuning_enable(True)
+        tuned = 0
+        try:
+            with torch.cuda.device(self.device):
+                for m in sorted({int(r) for r in rows if int(r) > SKINNY_MAX_ROWS}):
+                    for (n_out, k), lin in shapes.items():
+                        if n_out == self.vocab_size:
+                            continue  # the head's float32 logits do not go through the library
+                        x = torch.zeros(m, k, device=self.device, dtype=torch.bfloat16)
+                        out = torch.empty(m, n_out, device=self.device, dtype=torch.bfloat16)
+                        torch.mm(x, lin.weight.t(), out=out)
+                        tuned += 1
+                torch.cuda.synchronize()
+        finally:
+            tunable.tuning_enable(False)
+        return tuned
 
     # ------------------------------------------------------------------ the step
 
