@@ -43,9 +43,7 @@ __device__ inline bf16x8 zero_b128() {
   uint4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, z);
 }
-__device__ inline uint32_t pack2(float lo, float hi) {
-  return static_cast<uint32_t>(bf16_bits(lo)) | (static_cast<uint32_t>(bf16_bits(hi)) << 16);
-}
+__device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
 // Addressing of one request's keys and values for one key/value head.
 struct KV {
@@ -130,8 +128,12 @@ __device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2]
     m[ct] = m_new;
     uint4 u = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
     p[ct] = __builtin_bit_cast(bf16x8, u);
+    // Once the running maxima have settled alpha is exactly 1 in every lane: skip
+    // the rescaling of the accumulators then.
+    if (__any(alpha != 1.f)) {
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) o[dt][ct] *= alpha;
+      for (int dt = 0; dt < HD / 16; ++dt) o[dt][ct] *= alpha;
+    }
   }
 
   // O^T += V^T P^T.
@@ -527,7 +529,7 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
   // Up to 128 elements per head, K and V go through LDS (two stages fit in 64 KB);
   // larger heads read the cache directly in every wave.
   const bool staged = hd <= 128 && form != 0;
-  const int nw = staged ? (n_rep > 4 ? 8 : 4) : 4;
+  const int nw = staged ? (n_rep > 4 && form != 2 ? 8 : 4) : 4;  // form 2: four heads per block even for larger groups
   const int hgroups = (n_rep + nw - 1) / nw;
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
   const dim3 grid(n_tiles, nkv * hgroups);

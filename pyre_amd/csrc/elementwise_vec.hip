@@ -27,8 +27,8 @@ template <> struct Vec4<bf16> {
   }
   static __device__ inline void store(bf16* p, float4 v) {
     uint2 u;
-    u.x = static_cast<uint32_t>(bf16_bits(v.x)) | (static_cast<uint32_t>(bf16_bits(v.y)) << 16);
-    u.y = static_cast<uint32_t>(bf16_bits(v.z)) | (static_cast<uint32_t>(bf16_bits(v.w)) << 16);
+    u.x = pack_bf16x2(v.x, v.y);
+    u.y = pack_bf16x2(v.z, v.w);
     *reinterpret_cast<uint2*>(p) = u;
   }
 };

@@ -38,9 +38,7 @@ __device__ inline bf16x8 zero128() {
   uint4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, z);
 }
-__device__ inline uint32_t pack2(float lo, float hi) {
-  return static_cast<uint32_t>(bf16_bits(lo)) | (static_cast<uint32_t>(bf16_bits(hi)) << 16);
-}
+__device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
 template <int RT, int MT, int EPI>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ X, size_t ldx,

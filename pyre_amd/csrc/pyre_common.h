@@ -28,8 +28,21 @@ __host__ __device__ inline float to_float(bf16 v) {
   return x.f;
 }
 
+typedef __bf16 hw_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float hw_f32x2 __attribute__((ext_vector_type(2)));
+
+// Two floats to two bfloat16 in one word (low half first), round to nearest even:
+// one v_cvt_pk_bf16_f32 on the device.
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+  const hw_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, hw_bf16x2));
+}
+
 // Round to nearest, ties to even; NaN stays NaN.
 __host__ __device__ inline uint16_t bf16_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return static_cast<uint16_t>(pack_bf16x2(f, 0.f) & 0xffffu);
+#endif
   union { uint32_t u; float f; } x;
   x.f = f;
   if ((x.u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((x.u >> 16) | 0x40u);

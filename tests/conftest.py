@@ -24,6 +24,7 @@ TINY = {
     "tiny-a": dict(seed=0, std=0.02, gain_std=0.0),
     "tiny-b": dict(seed=1, std=0.05, gain_std=0.1),
     "tiny-c": dict(seed=2, std=0.04, gain_std=0.05),
+    "tiny-d": dict(seed=3, std=0.1, gain_std=0.2),
 }
 
 #: A third shape whose head size (32) and 16-token pages are taken by the MFMA
@@ -36,11 +37,22 @@ TINY_C = {
 }
 
 
+#: Awkward sizes: nothing is a multiple of 8, heads * head_dim is not the width, one
+#: key/value head for three query heads, a single layer.
+TINY_D = {
+    "architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 1, "hidden_size": 70,
+    "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 10, "intermediate_size": 50,
+    "vocab_size": 131, "rope_theta": 300.0, "rms_norm_eps": 1e-3, "tie_word_embeddings": True,
+    "max_position_embeddings": 300,
+}
+
+
 def tiny_config(name):
     from pyre_amd.config import preset
     from pyre_amd.registry import config_from_dict
 
-    return config_from_dict(TINY_C) if name == "tiny-c" else preset(name)
+    custom = {"tiny-c": TINY_C, "tiny-d": TINY_D}
+    return config_from_dict(custom[name]) if name in custom else preset(name)
 
 
 @pytest.fixture(scope="session")

@@ -11,7 +11,7 @@ from helpers import TOL, cut, first_bad, make_engine, plain_logits, random_ids, 
 
 pytestmark = pytest.mark.gpu
 
-CASES = [(m, d) for m in ("tiny-a", "tiny-b", "tiny-c") for d in ("float32", "bfloat16")]
+CASES = [(m, d) for m in ("tiny-a", "tiny-b", "tiny-c", "tiny-d") for d in ("float32", "bfloat16")]
 LENGTHS = {"a": 97, "b": 64, "c": 33, "d": 150}
 
 
