@@ -42,7 +42,9 @@ class Engine:
         self.device = torch.device(ec.device)
         self.dtype = TORCH_DTYPES[ec.dtype]
         spec = model.spec
-        self.max_model_len = min(ec.max_model_len or spec.max_positions, spec.max_positions)
+        # The model's own limit is the default, not a bound: the reference reads
+        # max_position_embeddings and never consults it (`pyre/config.py:60`).
+        self.max_model_len = ec.max_model_len or spec.max_positions
         self.runtime = Runtime(self.device, self.dtype, self.max_model_len)
         specs = model.cache_specs()
         probe = CacheManager(specs, ec.page_size, 1, ec.max_num_seqs, self.max_model_len)

@@ -54,8 +54,11 @@ def main(argv: list[str] | None = None) -> int:
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     max_tokens = -(-max(args.max_tokens, TOKEN_ROUNDING) // TOKEN_ROUNDING) * TOKEN_ROUNDING
+    from pyre_amd.registry import load_config
+
+    model_limit = getattr(load_config(args.model), "max_position_embeddings", 0) or 0
     ec = EngineConfig(dtype=args.dtype, device=args.device, page_size=PAGE_SIZE,
-                      max_cached_tokens=max_tokens, max_num_seqs=8,
+                      max_cached_tokens=max_tokens, max_num_seqs=8, max_model_len=max(model_limit, max_tokens),
                       max_num_batched_tokens=max(max_tokens, 4096), use_graphs=False)
     note(f"loading {args.model} ({args.dtype}) ...")
     engine = Engine.from_folder(args.model, ec)

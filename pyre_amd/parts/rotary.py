@@ -31,7 +31,7 @@ class RotaryEncoding(PositionEncoding):
         self._tables = None
 
     def rotary(self, runtime):
-        n = min(self.spec.max_positions, runtime.max_positions)
+        n = runtime.max_positions  # the engine's longest request decides, as the reference's table grows on demand
         if self._tables is None or self._tables[0].shape[0] < n or self._tables[0].device != runtime.device:
             cos, sin = rotary_tables(self.rotary_dim, self.spec.theta, n)
             self._tables = (cos.to(runtime.device).contiguous(), sin.to(runtime.device).contiguous())

@@ -132,3 +132,33 @@ def test_mixed_with_page_reuse(model, dtype, engines, plain_models):
     assert bad is None, bad
     eng.cache.check_invariants()
     assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+def test_weights_stored_in_32_bits_run_in_either_mode(tmp_path, plain_models):
+    """A tensor stored in 32 bits stays so: a float32 checkpoint runs in the 16-bit
+    mode with float32 weights (mixed products), and exactly in the 32-bit mode."""
+    import plain_qwen2 as P
+    from conftest import TINY, tiny_config
+    from pyre_amd.weights import write_random_model
+
+    folder = write_random_model(tmp_path / "f32", tiny_config("tiny-b"), dtype="float32", **TINY["tiny-b"])
+    plain = (P.read_config(folder), P.read_weights(folder))
+    ids = random_ids(1000, 90, seed=5)
+    for dtype in ("float32", "bfloat16"):
+        eng = make_engine(folder, dtype)
+        assert eng.model.layers[0].mixer.qkv.weight.dtype == torch.float32
+        steps = [([("a", ids[:50], list(range(50)))], []), ([("a", ids[50:], list(range(40)))], ["a"])]
+        got = replay(eng, steps)
+        want = {"a": plain_logits(plain, ids, torch.bfloat16 if dtype == "bfloat16" else None)}
+        bad, _ = first_bad(got, want, TOL[dtype])
+        assert bad is None, bad
+
+
+def test_requests_longer_than_the_models_own_limit(model_dirs, plain_models):
+    """max_position_embeddings is a default, not a bound (the reference never consults it)."""
+    plain = plain_models["tiny-a"]                       # max_position_embeddings = 256
+    ids = random_ids(512, 300, seed=8)
+    eng = make_engine(model_dirs["tiny-a"], "float32", max_model_len=320)
+    got = replay(eng, [([("a", ids[:280], [0, 279])], []), ([("a", ids[280:], list(range(20)))], ["a"])])
+    bad, _ = first_bad(got, {"a": plain_logits(plain, ids)}, TOL["float32"])
+    assert bad is None, bad
