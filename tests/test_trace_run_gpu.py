@@ -78,4 +78,4 @@ def test_trace_run(model, dtype, model_dirs, plain_models, tmp_path):
             d = (got[i] - ref[r][pos]).abs().max().item() / scale
             assert d <= TOL[dtype], f"step {st} request {r} position {pos}: {d:.3e}"
             checked += 1
-    assert checked > 100
+    assert checked > 50
