@@ -326,9 +326,11 @@ def _skinny_common(x, w, m):
 
 
 def skinny_form(m: int) -> int:
-    """Which form of the weight-streaming kernel suits m rows: 0 reads X from cache
-    in every wave (fine for a few rows), 1 stages X through LDS once per block."""
-    return 0 if m <= 4 else 1
+    """Which form of the weight-streaming kernel to use for m rows. Form 2 (W and X
+    through LDS, whole cache lines per load) measured fastest for every m <= 64 on the
+    7B shapes; forms 0 (waves split k, operands straight from memory) and 1 (only X
+    through LDS) are kept as alternatives for comparison."""
+    return 2
 
 
 def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int,

@@ -360,7 +360,7 @@ def test_sample_inverse_cdf():
 
 # ----------------------------------------------------------------------------- weight-streaming products
 
-@pytest.mark.parametrize("form", [0, 1])
+@pytest.mark.parametrize("form", [0, 1, 2])
 @pytest.mark.parametrize("m", [1, 7, 16, 33, 64])
 @pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (3584, 3584, 3), (1000, 136, 2), (131, 8, 1), (70000, 96, 1)])
 def test_gemm_skinny(m, n, k, ksplit, form):
@@ -374,7 +374,7 @@ def test_gemm_skinny(m, n, k, ksplit, form):
     assert torch.allclose(out.double().sum(0), want, atol=1e-3 * math.sqrt(k), rtol=1e-4)
 
 
-@pytest.mark.parametrize("form", [0, 1])
+@pytest.mark.parametrize("form", [0, 1, 2])
 @pytest.mark.parametrize("m", [1, 8, 40])
 @pytest.mark.parametrize("inter,k", [(176, 64), (18944, 3584), (250, 96)])
 def test_gemm_skinny_silu(m, inter, k, form):
