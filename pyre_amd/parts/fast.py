@@ -96,7 +96,9 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
 
 
 #: waves the split of decode attention aims at (256 CUs x 8)
-DECODE_TARGET_WAVES = 4096
+DECODE_TARGET_WAVES = 8192
+#: a split takes at least this many keys (two chunks): finer splits cost more in partial results than they gain
+DECODE_MIN_KEYS_PER_SPLIT = 64
 DECODE_MAX_SPLITS = 128
 
 
@@ -104,9 +106,9 @@ def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
                   target_waves: int = DECODE_TARGET_WAVES) -> int:
     """How many ways to split each request's keys so that the chip is full."""
     span = min(max_ctx, window + 32) if window > 0 else max_ctx
-    chunks = max(1, -(-span // 32))
+    pieces = max(1, -(-span // DECODE_MIN_KEYS_PER_SPLIT))
     items = n_tokens * nkv * -(-(nq // nkv) // 16)
-    return max(1, min(chunks, DECODE_MAX_SPLITS, -(-target_waves // items)))
+    return max(1, min(pieces, DECODE_MAX_SPLITS, -(-target_waves // items)))
 
 
 def attention(mixer, ctx, q, o, cache) -> bool:
