@@ -180,6 +180,48 @@ __device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bou
       });
 }
 
+// A chunk's operands held in registers, so that the loads of the next chunk can be
+// in flight while the current one is multiplied.
+template <int HD>
+struct ChunkRegs {
+  bf16x8 k[2][HD / 32];
+  uint2 v[HD / 16][2];
+  bool ok[2];
+};
+
+template <int HD>
+__device__ inline void load_chunk(const KV& kv, int key0, ChunkRegs<HD>& cr) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int k0 = key0 + 16 * t;
+    const int page = kv.table[k0 / kv.page_size], off = k0 % kv.page_size;
+    cr.ok[t] = page >= 0;
+    const size_t base = static_cast<size_t>(cr.ok[t] ? page : 0) * kv.nkv + kv.kvh;
+    const bf16* kp = kv.k + (base * kv.page_size + off + r) * HD + 8 * g;
+    const bf16* vp = kv.v + (base * HD + r) * kv.page_size + off + 4 * g;
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c) cr.k[t][c] = cr.ok[t] ? load_b128(kp + 32 * c) : zero_b128();
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt)
+      cr.v[dt][t] = cr.ok[t] ? *reinterpret_cast<const uint2*>(vp + static_cast<size_t>(dt) * 16 * kv.page_size)
+                             : uint2{0u, 0u};
+  }
+}
+
+template <int HD, int CT>
+__device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge, const Bounds<CT>& bd,
+                                   float scale_log2, const bf16x8 (&q)[CT][HD / 32],
+                                   f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
+  const bool ok[2] = {cr.ok[0], cr.ok[1]};
+  attend_core<HD, CT>(
+      key0, edge, ok, bd, scale_log2, q, o, m, l, [&](int t, int c) { return cr.k[t][c]; },
+      [&](int dt) {
+        const uint4 u = {cr.v[dt][0].x, cr.v[dt][0].y, cr.v[dt][1].x, cr.v[dt][1].y};
+        return __builtin_bit_cast(bf16x8, u);
+      });
+}
+
 // ---------------------------------------------------------------------------
 // Decode: grid (ceil(nsplits / 4), nkv * qtiles, tokens), 4 waves = 4 splits.
 // ---------------------------------------------------------------------------
@@ -216,8 +258,22 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int first = lo / kChunk, last = pos / kChunk;
   const int per = (last - first + 1 + nsplits - 1) / nsplits;
   const int begin = first + split * per, end = min(last + 1, begin + per);
-  for (int c = begin; c < end; ++c)
-    attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
+  if constexpr (HD <= 128) {
+    // Two register sets: while one chunk is multiplied the next one's loads are in flight.
+    ChunkRegs<HD> ra, rb;
+    if (begin < end) load_chunk<HD>(kv, begin * kChunk, ra);
+    for (int c = begin; c < end; c += 2) {
+      if (c + 1 < end) load_chunk<HD>(kv, (c + 1) * kChunk, rb);
+      attend_regs<HD, 1>(ra, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
+      if (c + 1 < end) {
+        if (c + 2 < end) load_chunk<HD>(kv, (c + 2) * kChunk, ra);
+        attend_regs<HD, 1>(rb, (c + 1) * kChunk, c + 1 == first || c + 1 == last, bd, scale_log2, qr, o, m, l);
+      }
+    }
+  } else {
+    for (int c = begin; c < end; ++c)
+      attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
+  }
 
   if (r < nheads) {
     const size_t slot = (static_cast<size_t>(idx) * nq + head0 + r) * nsplits + split;

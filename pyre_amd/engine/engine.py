@@ -19,13 +19,14 @@ from pyre_amd.config.model import ModelConfig
 from pyre_amd.engine.batch import Entry, build_host_batch, pad_decode_batch
 from pyre_amd.engine.context import (TORCH_DTYPES, KVLayerView, MetaBuffers, Runtime, StateLayerView,
                                      StepContext)
+from pyre_amd.parts.fast import DECODE_ROW_BUCKETS
 from pyre_amd.parts.model import LayeredModel
 from pyre_amd.registry import get_architecture, load_config
 from pyre_amd.weights.loader import adopt_state, load_weights
 
 
 #: decode steps of up to this many requests are captured in HIP graphs, at these sizes
-GRAPH_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64)
+GRAPH_ROW_BUCKETS = DECODE_ROW_BUCKETS
 GRAPH_MAX_ROWS = GRAPH_ROW_BUCKETS[-1]
 
 

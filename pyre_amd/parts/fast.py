@@ -95,20 +95,24 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
     return True
 
 
-#: waves the split of decode attention aims at (256 CUs x 8)
-DECODE_TARGET_WAVES = 8192
-#: a split takes at least this many keys (two chunks): finer splits cost more in partial results than they gain
+#: waves the split of decode attention aims at: the kernel holds two chunks of keys and
+#: values in registers, which leaves room for one wave on each of the 1,024 SIMDs; measured,
+#: time jumps as soon as a second round of waves is needed
+DECODE_TARGET_WAVES = 1024
+#: a split takes at least this many keys (two chunks)
 DECODE_MIN_KEYS_PER_SPLIT = 64
 DECODE_MAX_SPLITS = 128
+#: sizes (requests) at which decode steps are captured in HIP graphs
+DECODE_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64)
 
 
 def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
                   target_waves: int = DECODE_TARGET_WAVES) -> int:
-    """How many ways to split each request's keys so that the chip is full."""
+    """How many ways to split each request's keys so that the chip is full but not overfull."""
     span = min(max_ctx, window + 32) if window > 0 else max_ctx
     pieces = max(1, -(-span // DECODE_MIN_KEYS_PER_SPLIT))
     items = n_tokens * nkv * -(-(nq // nkv) // 16)
-    return max(1, min(pieces, DECODE_MAX_SPLITS, -(-target_waves // items)))
+    return max(1, min(pieces, DECODE_MAX_SPLITS, target_waves // items))
 
 
 def attention(mixer, ctx, q, o, cache) -> bool:
@@ -124,8 +128,14 @@ def attention(mixer, ctx, q, o, cache) -> bool:
     hb = ctx.host
     n_dec, n_tiles = len(hb.decode_tokens), len(hb.prefill_tiles)
     if n_dec:
+        # The split is chosen from rounded-up sizes (requests to the next captured-step
+        # size, context to a power of two of pages), so that a step gives bit for bit the
+        # same result whether it runs eagerly or as a replayed graph at those sizes.
+        rows = next((b for b in DECODE_ROW_BUCKETS if b >= n_dec), n_dec)
+        pages = max(1, -(-hb.max_decode_ctx // cache.page_size))
+        span = max(8, 1 << (pages - 1).bit_length()) * cache.page_size
         nsplits = ctx.runtime.options.get("decode_splits") or decode_splits(
-            n_dec, s.num_heads, s.num_kv_heads, hb.max_decode_ctx, cache.window,
+            rows, s.num_heads, s.num_kv_heads, span, cache.window,
             ctx.runtime.options.get("decode_target_waves", DECODE_TARGET_WAVES))
         acc = ctx.workspace.get("attn.part_acc", (n_dec, s.num_heads, nsplits, s.head_dim), torch.float32)
         ml = ctx.workspace.get("attn.part_ml", (n_dec, s.num_heads, nsplits, 2), torch.float32)
