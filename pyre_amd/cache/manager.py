@@ -24,6 +24,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import numpy as np
+
 from pyre_amd.cache.allocator import OutOfPages, PageAllocator
 from pyre_amd.parts.base import KVCacheSpec, StateCacheSpec
 
@@ -62,6 +64,9 @@ class _Request:
     length: int = 0                  #: tokens committed
     reserved: int = 0                #: tokens that pages exist for
     tables: list[list[int]] = field(default_factory=list)  #: one per page group
+    #: the same tables as int32 arrays (filled with RELEASED beyond their ends), kept in
+    #: step with the lists so that a step's batch copies rows instead of converting lists
+    arrays: list[np.ndarray] = field(default_factory=list)
 
 
 class CacheManager:
@@ -135,7 +140,9 @@ class CacheManager:
         if rid in self._requests:
             raise ValueError(f"request {rid!r} already exists")
         slot = self.slots.allocate()
-        self._requests[rid] = _Request(slot, tables=[[] for _ in self.page_groups])
+        self._requests[rid] = _Request(
+            slot, tables=[[] for _ in self.page_groups],
+            arrays=[np.full(self.max_pages_per_seq, RELEASED, dtype=np.int32) for _ in self.page_groups])
         for g in self.state_groups:
             if g.tensor is not None:
                 g.tensor[:, slot].zero_()
@@ -177,8 +184,10 @@ class CacheManager:
                 if g.allocator.num_free < add:
                     raise OutOfPages(f"page pool of group {g.index} exhausted "
                                      f"({add} needed, {g.allocator.num_free} of {g.num_pages} free)")
-            for g, table in zip(self.page_groups, req.tables):
+            for g, table, arr in zip(self.page_groups, req.tables, req.arrays):
+                have = len(table)
                 table.extend(g.allocator.allocate_many(add))
+                arr[have:have + add] = table[have:]
         req.reserved = max(req.reserved, new_len)
 
     def slot_mapping(self, rid, group: int, start: int, n: int) -> list[int]:
@@ -196,6 +205,11 @@ class CacheManager:
     def block_table(self, rid, group: int) -> list[int]:
         return self._requests[rid].tables[group]
 
+    def block_table_array(self, rid, group: int) -> np.ndarray:
+        """The request's block table as int32 ``[max_pages_per_seq]``; entries beyond
+        its pages are RELEASED. Do not write to it."""
+        return self._requests[rid].arrays[group]
+
     def commit(self, rid, n_new: int) -> None:
         """The step has run: the request is ``n_new`` tokens longer. Pages of a
         windowed group that no later query can see go back to the pool."""
@@ -203,7 +217,7 @@ class CacheManager:
         req.length += n_new
         if req.length > req.reserved:
             raise RuntimeError(f"request {rid!r}: committed past the reservation")
-        for g, table in zip(self.page_groups, req.tables):
+        for g, table, arr in zip(self.page_groups, req.tables, req.arrays):
             w = g.spec.window
             if w <= 0:
                 continue
@@ -214,6 +228,7 @@ class CacheManager:
                 if table[i] != RELEASED:
                     g.allocator.free(table[i])
                     table[i] = RELEASED
+                    arr[i] = RELEASED
 
     def free_request(self, rid) -> None:
         req = self._requests.pop(rid)

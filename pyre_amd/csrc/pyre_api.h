@@ -82,6 +82,10 @@ int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const 
 int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,
                 hipStream_t stream);
 
+// tokens[i] = ids[src[i]] where src[i] >= 0: a step's token that is the previous step's
+// sampled id, taken on the device so that the host need not wait for it.
+int pyre_feed_tokens(int* tokens, const int* src, const int* ids, int n, hipStream_t stream);
+
 int pyre_sample(const float* logits, long row_stride, const float* temperature,
                 const float* uniform, int* out, int m, int vocab, hipStream_t stream);
 

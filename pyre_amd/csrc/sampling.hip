@@ -114,7 +114,20 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(const float* __restric
   }
 }
 
+// tokens[i] = ids[src[i]] for the rows whose token is a result still on the device.
+__global__ __launch_bounds__(256) void feed_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ src,
+                                                           const int* __restrict__ ids, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n && src[i] >= 0) tokens[i] = ids[src[i]];
+}
+
 }  // namespace
+
+extern "C" int pyre_feed_tokens(int* tokens, const int* src, const int* ids, int n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(feed_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, tokens, src, ids, n);
+  return check_launch("feed_tokens");
+}
 
 // scratch: m * 64 floats followed by m * 64 ints.
 extern "C" int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,

@@ -23,6 +23,10 @@ class Entry:
     rid: object
     tokens: list[int]
     want: list[int] = field(default_factory=list)  #: indices into ``tokens``
+    #: the entry's single token is row ``feed`` of the ids that the caller hands to the
+    #: step on the device (a result that the host has not waited for); ``tokens`` is then
+    #: a placeholder of length one
+    feed: int | None = None
 
 
 @dataclass
@@ -45,10 +49,15 @@ class HostBatch:
     decode_tokens: np.ndarray = None   #: token indices of requests that bring one token
     prefill_tiles: np.ndarray = None   #: [T, 2] (first token, count <= TILE) of the others, longest context first
     max_decode_ctx: int = 0            #: longest context among the single-token requests
+    token_src: np.ndarray = None       #: [N] row of the device-side ids that a token comes from, or -1
 
     @property
     def decode_only(self) -> bool:
         return self.max_q_len == 1
+
+    @property
+    def feeds(self) -> bool:
+        return self.token_src is not None and bool((self.token_src >= 0).any())
 
 
 def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: int | None = None) -> HostBatch:
@@ -57,18 +66,18 @@ def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: 
     pages reserved for this step."""
     if not entries:
         raise ValueError("a step needs at least one entry")
+    n_seqs = len(entries)
     seen = set()
     tokens: list[int] = []
-    positions: list[int] = []
-    seq_of_token: list[int] = []
+    token_src: list[int] = []
     q_start = [0]
-    ctx_len: list[int] = []
+    starts: list[int] = []
     state_slots: list[int] = []
     logit_rows: list[int] = []
     n_groups = len(cache.page_groups)
-    slots: list[list[int]] = [[] for _ in range(n_groups)]
+    ps = cache.page_size
     width = table_width or cache.max_pages_per_seq
-    tables = [np.full((len(entries), width), -1, dtype=np.int32) for _ in range(n_groups)]
+    tables = [np.full((n_seqs, width), -1, dtype=np.int32) for _ in range(n_groups)]
     max_q = 0
     for s, e in enumerate(entries):
         if e.rid in seen:
@@ -77,45 +86,59 @@ def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: 
         n = len(e.tokens)
         if n == 0:
             raise ValueError(f"request {e.rid!r} brings no tokens")
-        for t in e.tokens:
-            if not (0 <= int(t) < vocab_size):
-                raise ValueError(f"token id {t} of request {e.rid!r} is outside the vocabulary (0..{vocab_size - 1})")
-        start = cache.length(e.rid)
+        if e.feed is not None and n != 1:
+            raise ValueError(f"request {e.rid!r}: only a single token can come from the device")
         base = len(tokens)
-        tokens.extend(int(t) for t in e.tokens)
-        positions.extend(range(start, start + n))
-        seq_of_token.extend([s] * n)
+        tokens.extend(e.tokens)
+        token_src.extend([-1] * n if e.feed is None else [int(e.feed)])
         q_start.append(base + n)
-        ctx_len.append(start + n)
+        starts.append(cache.length(e.rid))
         state_slots.append(cache.slot(e.rid))
         for w in e.want:
             if not (0 <= int(w) < n):
                 raise ValueError(f"request {e.rid!r}: wanted place {w} is outside its {n} tokens")
             logit_rows.append(base + int(w))
         for g in range(n_groups):
-            slots[g].extend(cache.slot_mapping(e.rid, g, start, n))
-            tbl = cache.block_table(e.rid, g)
-            if len(tbl) > width:
-                raise ValueError(f"request {e.rid!r} has {len(tbl)} pages, the table holds {width}")
-            tables[g][s, :len(tbl)] = tbl
+            have = len(cache.block_table(e.rid, g))
+            if have > width:
+                raise ValueError(f"request {e.rid!r} has {have} pages, the table holds {width}")
+            tables[g][s, :have] = cache.block_table_array(e.rid, g)[:have]
         max_q = max(max_q, n)
+    n_tokens = len(tokens)
     i32 = lambda x: np.asarray(x, dtype=np.int32)  # noqa: E731
-    decode_tokens, tiles, max_decode_ctx = [], [], 0
-    for s in range(len(entries)):
+    tok = np.asarray(tokens, dtype=np.int64)
+    if tok.min() < 0 or tok.max() >= vocab_size:
+        bad = next((e.rid, t) for e in entries for t in e.tokens if not (0 <= int(t) < vocab_size))
+        raise ValueError(f"token id {bad[1]} of request {bad[0]!r} is outside the vocabulary (0..{vocab_size - 1})")
+    q_start_a, starts_a = i32(q_start), i32(starts)
+    counts = q_start_a[1:] - q_start_a[:-1]
+    seq_of_token = np.repeat(np.arange(n_seqs, dtype=np.int32), counts)
+    # position of a token = its request's length before the step + its index within the run
+    positions = (starts_a - q_start_a[:-1])[seq_of_token] + np.arange(n_tokens, dtype=np.int32)
+    ctx_len = starts_a + counts
+    slots = []
+    for g in range(n_groups):
+        pages = tables[g][seq_of_token, positions // ps]
+        if (pages < 0).any():
+            t = int(np.argmax(pages < 0))
+            raise RuntimeError(f"position {int(positions[t])} of request {entries[int(seq_of_token[t])].rid!r} "
+                               "lies in a released page")
+        slots.append((pages * ps + positions % ps).astype(np.int32))
+    single = counts == 1
+    decode_tokens = q_start_a[:-1][single]
+    max_decode_ctx = int(ctx_len[single].max()) if single.any() else 0
+    tiles = []
+    for s in np.nonzero(~single)[0]:
         a, b = q_start[s], q_start[s + 1]
-        if b - a == 1:
-            decode_tokens.append(a)
-            max_decode_ctx = max(max_decode_ctx, ctx_len[s])
-        else:
-            tiles.extend((positions[t0] + min(TILE, b - t0), t0, min(TILE, b - t0)) for t0 in range(a, b, TILE))
+        tiles.extend((int(positions[t0]) + min(TILE, b - t0), t0, min(TILE, b - t0)) for t0 in range(a, b, TILE))
     tiles.sort(key=lambda t: -t[0])  # the tiles with the most keys start first
     return HostBatch(
         decode_tokens=i32(decode_tokens), prefill_tiles=i32([t[1:] for t in tiles]).reshape(-1, 2),
         max_decode_ctx=max_decode_ctx,
-        n_tokens=len(tokens), n_seqs=len(entries), rids=[e.rid for e in entries], tokens=i32(tokens),
-        positions=i32(positions), seq_of_token=i32(seq_of_token), q_start=i32(q_start),
-        ctx_len=i32(ctx_len), state_slots=i32(state_slots), logit_rows=i32(logit_rows),
-        slots=[i32(x) for x in slots], tables=tables, max_q_len=max_q)
+        n_tokens=n_tokens, n_seqs=n_seqs, rids=[e.rid for e in entries], tokens=tok.astype(np.int32),
+        positions=positions.astype(np.int32), seq_of_token=seq_of_token, q_start=q_start_a,
+        ctx_len=ctx_len.astype(np.int32), state_slots=i32(state_slots), logit_rows=i32(logit_rows),
+        slots=slots, tables=tables, max_q_len=max_q, token_src=i32(token_src))
 
 
 def pad_decode_batch(hb: HostBatch, n_rows: int, scratch_slot: int, max_ctx: int) -> HostBatch:
@@ -140,4 +163,4 @@ def pad_decode_batch(hb: HostBatch, n_rows: int, scratch_slot: int, max_ctx: int
         slots=[cat(s, [-1] * pad) for s in hb.slots],
         tables=[np.concatenate([t, np.full((pad, t.shape[1]), -1, dtype=np.int32)]) for t in hb.tables],
         max_q_len=1, decode_tokens=i32(range(n_rows)), prefill_tiles=i32([]).reshape(-1, 2),
-        max_decode_ctx=max_ctx)
+        max_decode_ctx=max_ctx, token_src=cat(hb.token_src, [-1] * pad))

@@ -67,7 +67,7 @@ def meta_layout(n_cap: int, s_cap: int, table_widths: list[int]) -> tuple[dict, 
         lay[name] = (off, n)
         off += (n + 3) // 4 * 4
 
-    for name in ("tokens", "positions", "seq_of_token", "logit_rows", "decode_tokens"):
+    for name in ("tokens", "positions", "seq_of_token", "logit_rows", "decode_tokens", "token_src"):
         put(name, n_cap)
     put("prefill_tiles", 2 * (n_cap // 32 + s_cap))
     put("q_start", s_cap + 1)
@@ -113,6 +113,10 @@ class MetaBuffers:
         fill("logit_rows", hb.logit_rows), fill("q_start", hb.q_start), fill("ctx_len", hb.ctx_len)
         fill("state_slots", hb.state_slots)
         fill("decode_tokens", hb.decode_tokens), fill("prefill_tiles", hb.prefill_tiles)
+        o, n = lay["token_src"]
+        h[o:o + n] = -1
+        if hb.token_src is not None:
+            fill("token_src", hb.token_src)
         for g, w in enumerate(widths):
             fill(f"slots{g}", hb.slots[g])
             o, _ = lay[f"table{g}"]

@@ -31,6 +31,9 @@ GRAPH_MAX_ROWS = GRAPH_ROW_BUCKETS[-1]
 
 
 class Engine:
+    #: ``step`` takes ``fed_ids``: tokens that are results still on the device
+    accepts_fed_ids = True
+
     def __init__(self, model: LayeredModel, config: ModelConfig, engine_config: EngineConfig):
         if not torch.cuda.is_available():
             raise RuntimeError("pyre_amd needs a GPU: there is no CPU execution path")
@@ -165,12 +168,17 @@ class Engine:
     def has(self, rid) -> bool:
         return rid in self.cache
 
-    def step(self, entries: list[Entry]) -> torch.Tensor | None:
+    def step(self, entries: list[Entry], fed_ids: torch.Tensor | None = None) -> torch.Tensor | None:
         """Run one batch. Requests not seen before are admitted (a slot and empty
         block tables); pages for all the step's tokens are reserved first, lengths
         are committed afterwards. Returns float32 ``[sum(len(want)), vocab]`` on the
         device, rows in the order of the entries and of each ``want`` (None if no
         logits are wanted).
+
+        An entry with ``feed = i`` takes its one token from ``fed_ids[i]`` (int32 on
+        the device, for instance the ids a sampler has just written) when the step
+        runs on the device: the host can put the step on the stream without waiting
+        for the previous step's result.
         """
         n_tokens = sum(len(e.tokens) for e in entries)
         ec = self.engine_config
@@ -195,18 +203,30 @@ class Engine:
         else:
             width = max(8, -(-pages // 8) * 8)
         hb = build_host_batch(entries, cache, self.vocab_size, table_width=width)
+        if hb.feeds and fed_ids is None:
+            raise ValueError("an entry takes its token from the device, but no ids were given")
         with torch.cuda.device(self.device):
             if graphable:
-                logits = self._step_captured(hb, rows, width)
+                logits = self._step_captured(hb, rows, width, fed_ids)
             else:
-                logits = self._run(hb)
+                logits = self._run(hb, fed_ids)
         for e in entries:
             cache.commit(e.rid, len(e.tokens))
         self.steps_run += 1
         return logits
 
-    def _context(self, hb, n_cap=None, s_cap=None):
+    def _upload(self, hb, fed_ids, n_cap=None, s_cap=None):
+        """The step's arrays to the device; tokens that are results still on the
+        device are put in place there."""
         views = self.meta.upload(hb, n_cap, s_cap)
+        if hb.feeds:
+            from pyre_amd.hip import ops
+
+            ops.feed_tokens(views["tokens"], views["token_src"], fed_ids, hb.n_tokens)
+        return views
+
+    def _context(self, hb, fed_ids=None, n_cap=None, s_cap=None):
+        views = self._upload(hb, fed_ids, n_cap, s_cap)
         ctx = StepContext(
             runtime=self.runtime, host=hb, n_tokens=hb.n_tokens, n_seqs=hb.n_seqs,
             n_logits=len(hb.logit_rows), tokens=views["tokens"], positions=views["positions"],
@@ -215,11 +235,11 @@ class Engine:
             decode_tokens=views["decode_tokens"], prefill_tiles=views["prefill_tiles"])
         return ctx, self._layer_views(views)
 
-    def _run(self, hb):
-        ctx, caches = self._context(hb)
+    def _run(self, hb, fed_ids=None):
+        ctx, caches = self._context(hb, fed_ids)
         return self.model.forward(ctx, caches)
 
-    def _step_captured(self, hb, rows: int, width: int):
+    def _step_captured(self, hb, rows: int, width: int, fed_ids=None):
         """A decode step at a fixed size (``rows`` requests, tables ``width`` pages
         wide): run eagerly the first time, captured in a HIP graph the second,
         replayed from then on. Only the metadata upload happens outside the graph."""
@@ -228,12 +248,12 @@ class Engine:
         padded = pad_decode_batch(hb, rows, self.cache.max_num_seqs, width * self.cache.page_size)
         state = self._graphs.get(key)
         if state is None:
-            ctx, caches = self._context(padded)
+            ctx, caches = self._context(padded, fed_ids)
             logits = self.model.forward(ctx, caches)
             self._graphs[key] = "warm"
             return logits[:live]
         if state == "warm":
-            ctx, caches = self._context(padded)
+            ctx, caches = self._context(padded, fed_ids)
             ws = self.runtime.workspace
             graph = torch.cuda.CUDAGraph()
             ws.frozen = True
@@ -244,7 +264,7 @@ class Engine:
                 ws.frozen = False
             state = self._graphs[key] = (graph, logits)
         else:
-            self.meta.upload(padded)
+            self._upload(padded, fed_ids)
         graph, logits = state
         graph.replay()
         self.graph_replays += 1

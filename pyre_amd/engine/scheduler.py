@@ -17,6 +17,15 @@ generated so far (which it keeps). A request that could not fit the pool even
 alone is refused when it is added. (The reference lets ``MemoryError`` escape,
 `pyre/paged_cache.py:58-67`.)
 
+While every running request is decoding and nobody waits, the next step is put on
+the device before the host has seen this step's tokens: its batch is known (the same
+requests, one position further, minus those that reach their length), and the tokens
+are fed on the device from the sampler's ids. The host then reads this step's tokens
+while the next step runs. A request that turns out to have ended (its end-of-sequence
+token) has one surplus row in that next step, which is ignored. This needs an engine
+whose ``step`` takes ``fed_ids`` and a sampler with ``launch``/``collect``/``ids``;
+with others every step waits for its tokens as before.
+
 This module needs neither torch nor a GPU: the engine and the sampler are passed in.
 """
 
@@ -29,7 +38,7 @@ from pyre_amd.sampling.params import SamplingParams
 from pyre_amd.sampling.rng import uniform
 
 
-@dataclass
+@dataclass(eq=False)
 class Request:
     seq_id: int
     prompt_ids: list[int]
@@ -42,6 +51,15 @@ class Request:
     @property
     def tokens(self) -> list[int]:
         return self.prompt_ids + self.generated
+
+    def token_slice(self, start: int, count: int) -> list[int]:
+        """``tokens[start:start + count]`` without joining the two lists."""
+        n = len(self.prompt_ids)
+        if start >= n:
+            return self.generated[start - n:start - n + count]
+        if start + count <= n:
+            return self.prompt_ids[start:start + count]
+        return self.prompt_ids[start:] + self.generated[:start + count - n]
 
     @property
     def cur_len(self) -> int:        # pyre/scheduler.py:22-24
@@ -89,6 +107,10 @@ class Scheduler:
         self.finished: dict[int, Request] = {}
         self._next_seq = 0
         self.steps = 0
+        #: put the next decode step on the device before this step's tokens are read
+        self.lookahead = bool(getattr(engine, "accepts_fed_ids", False)) and all(
+            hasattr(sampler, a) for a in ("launch", "collect", "ids"))
+        self._ahead: tuple[StepPlan, object] | None = None  #: (plan, logits) of a step already on the device
 
     # ------------------------------------------------------------------ requests
 
@@ -194,16 +216,20 @@ class Scheduler:
 
     def step(self) -> list[tuple[int, int]]:
         """Plan, run and sample one batch; returns (seq_id, new token) pairs."""
-        plan = self.plan()
-        if not plan.entries:
-            if self.has_work:
-                raise RuntimeError("scheduler made no progress (no request fits the pool or the budget)")
-            return []
-        entries = []
-        for e in plan.entries:
-            toks = e.request.tokens[e.start:e.start + e.count]
-            entries.append(Entry(e.request.seq_id, toks, [e.count - 1] if e.samples else []))
-        logits = self.engine.step(entries)
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and all(e.request.done for e in ahead[0].entries):
+            ahead = None  # every request of the step that ran ahead has ended meanwhile
+        if ahead is not None:
+            plan, logits = ahead
+        else:
+            plan = self.plan()
+            if not plan.entries:
+                if self.has_work:
+                    raise RuntimeError("scheduler made no progress (no request fits the pool or the budget)")
+                return []
+            entries = [Entry(e.request.seq_id, e.request.token_slice(e.start, e.count),
+                             [e.count - 1] if e.samples else []) for e in plan.entries]
+            logits = self.engine.step(entries)
         self.steps += 1
         for e in plan.entries:
             e.request.num_computed += e.count
@@ -213,8 +239,15 @@ class Scheduler:
             temps = [r.params.temperature for r in sampling]
             us = [uniform(r.params.seed, r.seq_id, len(r.generated)) if r.params.temperature > 0 else 0.0
                   for r in sampling]
-            new = self.sampler.sample(logits, temps, us)
+            if self.lookahead:
+                handle = self.sampler.launch(logits, temps, us)
+                self._ahead = self._run_ahead(plan, sampling)
+                new = self.sampler.collect(handle)
+            else:
+                new = self.sampler.sample(logits, temps, us)
             for r, tok in zip(sampling, new):
+                if r.done:
+                    continue  # a surplus row of a step that ran ahead
                 tok = int(tok)
                 r.generated.append(tok)
                 out.append((r.seq_id, tok))
@@ -228,6 +261,24 @@ class Scheduler:
             self.engine.finish(r.seq_id)
             self.finished[r.seq_id] = r
         return out
+
+    def _run_ahead(self, plan: StepPlan, sampling: list[Request]):
+        """Put the next step on the device if it is known without this step's tokens:
+        all running requests have just been sampled for, nobody waits, and the pages are
+        there. Returns (plan, logits) or None. The sampler's ids of this step must
+        already be on the stream."""
+        if self.waiting or len(sampling) != len(self.running) or len(plan.entries) != len(sampling):
+            return None
+        rows = [(i, r) for i, r in enumerate(sampling)
+                if not r.done and len(r.generated) + 1 < r.params.max_new_tokens]
+        if not rows or len(rows) > self.token_budget:
+            return None
+        if sum(self.cache.pages_needed(r.seq_id, 1) for _, r in rows) > self.cache.free_pages():
+            return None
+        nxt = StepPlan([PlannedEntry(r, r.num_computed, 1, True) for _, r in rows], [], [])
+        entries = [Entry(r.seq_id, [0], [0], feed=i) for i, r in rows]
+        logits = self.engine.step(entries, fed_ids=self.sampler.ids)
+        return nxt, logits
 
     def run(self) -> dict[int, list[int]]:
         """Run until every request is finished: {seq_id: generated tokens}

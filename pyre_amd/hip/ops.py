@@ -264,6 +264,13 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
          out.data_ptr(), m, logits.shape[1], _stream())
 
 
+def feed_tokens(tokens: torch.Tensor, src: torch.Tensor, ids: torch.Tensor, n: int) -> None:
+    """tokens[i] = ids[src[i]] for i < n with src[i] >= 0 (all int32 on the device)."""
+    _dev(tokens, src, ids)
+    _i32("tokens", tokens, n), _i32("src", src, n), _i32("ids", ids)
+    call("pyre_feed_tokens", tokens.data_ptr(), src.data_ptr(), ids.data_ptr(), n, _stream())
+
+
 def attn_mfma_supports(hd: int, page_size: int, nq: int, nkv: int) -> bool:
     from pyre_amd.hip.lib import lib
 

@@ -1,11 +1,12 @@
 """Per-kernel totals of a rocprofv3 kernel trace.
 
-    python -m pyre_amd.profile_summary RESULTS.db [TOP] [--match TEXT]
+    python -m pyre_amd.profile_summary RESULTS.db [TOP] [--match TEXT] [--tail-ms MS]
 
 reads the ``kernels`` view of the rocpd SQLite file that
 ``rocprofv3 --kernel-trace --stats -d DIR -o NAME -- <program>`` writes
 (``DIR/NAME_results.db``) and prints calls, total, share, mean, min and max time per
-kernel name, longest total first.
+kernel name, longest total first. ``--tail-ms MS`` keeps only the launches of the
+last MS milliseconds of the trace (the timed steps of a benchmark, without its set-up).
 """
 
 from __future__ import annotations
@@ -14,10 +15,13 @@ import sqlite3
 import sys
 
 
-def summarise(path: str, top: int = 25, match: str | None = None) -> str:
+def summarise(path: str, top: int = 25, match: str | None = None, tail_ms: float | None = None) -> str:
     con = sqlite3.connect(path)
+    since = 0
+    if tail_ms is not None:
+        since = con.execute("select max(end) from kernels").fetchone()[0] - int(tail_ms * 1e6)
     rows = con.execute("select name, count(*), sum(end - start), min(end - start), max(end - start) "
-                       "from kernels group by name order by 3 desc").fetchall()
+                       "from kernels where start >= ? group by name order by 3 desc", (since,)).fetchall()
     if match:
         rows = [r for r in rows if match in r[0]]
     total = sum(r[2] for r in rows) or 1
@@ -38,7 +42,12 @@ def main(argv: list[str]) -> int:
         i = argv.index("--match")
         match = argv[i + 1]
         del argv[i:i + 2]
-    print(summarise(argv[0], int(argv[1]) if len(argv) > 1 else 25, match))
+    tail_ms = None
+    if "--tail-ms" in argv:
+        i = argv.index("--tail-ms")
+        tail_ms = float(argv[i + 1])
+        del argv[i:i + 2]
+    print(summarise(argv[0], int(argv[1]) if len(argv) > 1 else 25, match, tail_ms))
     return 0
 
 

@@ -187,3 +187,80 @@ def test_batched_equals_alone():
         sid = s2.add_request(prompts[i], caps[i])
         assert s2.run()[sid] == together[i]
     assert not s.running and not s.waiting
+
+
+# ---------------------------------------------------------------------------
+# Running one step ahead: the next decode step goes to the engine before this
+# step's tokens are read; its tokens come from the sampler's ids "on the device".
+# ---------------------------------------------------------------------------
+class AheadEngine(FakeEngine):
+    accepts_fed_ids = True
+
+    def __init__(self, **kw):
+        super().__init__(**kw)
+        self.fed = {}  #: rid -> every token the engine has been given for it, in order
+        self.ahead_steps = 0
+
+    def step(self, entries, fed_ids=None):
+        for e in entries:
+            toks = [fed_ids[e.feed]] if e.feed is not None else list(e.tokens)
+            self.fed.setdefault(e.rid, []).extend(toks)
+        self.ahead_steps += any(e.feed is not None for e in entries)
+        return super().step(entries)
+
+
+class AheadSampler(FakeSampler):
+    """``ids`` stands for the ids on the device: written at launch, read by the engine
+    when a step that ran ahead is fed from them."""
+
+    ids = ()
+
+    def launch(self, rows, temps, us):
+        running = {r.seq_id: r for r in self.sched.running}
+        # a request that has ended has a surplus row in a step that ran ahead: any id will do
+        self.ids = [sum(running[e.rid].tokens) % 100 if e.rid in running else -1 for e in rows]
+        return list(self.ids)
+
+    def collect(self, handle):
+        return handle
+
+
+@pytest.mark.parametrize("eos", [None, 37])
+def test_running_ahead_gives_the_same_tokens(eos):
+    prompts = [[1, 2, 3], [7] * 20, [5, 9], [4, 4, 4, 4, 11]]
+    lens = [9, 17, 30, 12]
+
+    def run(ahead):
+        eng = AheadEngine(pages=64, max_num_seqs=4)
+        s = Scheduler(eng)
+        s.sampler = AheadSampler(s)
+        s.lookahead = ahead
+        ids = [s.add_request(p, n, eos_id=eos) for p, n in zip(prompts, lens)]
+        out = s.run()
+        eng.cache.check_invariants()
+        assert eng.cache.free_pages() == 64
+        return eng, s, [out[i] for i in ids]
+
+    eng0, _, plain = run(False)
+    eng1, s1, ahead = run(True)
+    assert ahead == plain == [expected(p, n, eos) for p, n in zip(prompts, lens)]
+    assert eng0.ahead_steps == 0 and eng1.ahead_steps > 10
+    # every request was fed exactly its prompt and the tokens it generated, bar the last one,
+    # plus at most one surplus token after an end-of-sequence token
+    for rid, (p, g) in enumerate(zip(prompts, ahead)):
+        want = p + g[:-1]
+        assert eng1.fed[rid][:len(want)] == want and len(eng1.fed[rid]) <= len(want) + 1
+
+
+def test_a_request_added_meanwhile_waits_one_step():
+    eng = AheadEngine(pages=64, max_num_seqs=4)
+    s = Scheduler(eng)
+    s.sampler = AheadSampler(s)
+    s.lookahead = True
+    a = s.add_request([1, 2, 3], 8)
+    s.step(), s.step()                      # the second step has put a third one on the device
+    b = s.add_request([9, 9], 4)
+    s.step()                                # consumes the step that ran ahead; b still waits
+    assert [r.seq_id for r in s.waiting] == [b]
+    out = s.run()
+    assert out[a] == expected([1, 2, 3], 8) and out[b] == expected([9, 9], 4)
