@@ -514,6 +514,212 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_lds_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Prefill on 32x32x16 tiles: the NW waves of a block take NW query heads of one
+// key/value head over the same 32 tokens (one MFMA tile of columns per wave);
+// keys and values come through LDS in chunks of 64, double-buffered, loaded once
+// per block. Per chunk and wave: S^T (64 keys x 32 tokens) in two tiles, one
+// exchange between the two lanes that share a column for the running maximum,
+// and O^T (HD x 32) += V^T P^T. The sum of a column is kept per lane (each lane
+// adds the keys it holds) and joined once at the end.
+//
+//   ks[stage][key][HD + 8]   K rows as stored; the padding puts 16 rows on distinct banks
+//   vs[stage][d][64 + 8]     V^T; within each run of 16 keys the order is
+//                            (4g + j, 8 + 4g + j -> 8g + j, 8g + 4 + j), so that the eight
+//                            keys a lane needs for one MFMA are 16 contiguous bytes
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+constexpr int kKeys = 64;
+
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
+    int nq, int nkv, int page_size, float scale_log2, int window) {
+  constexpr int KS = HD + 8, VS = kKeys + 8, T = NW * 64;
+  constexpr int SEG = HD / 8;                 // 16-byte pieces of one K row
+  constexpr int NPK = kKeys * SEG;            // pieces of K per chunk
+  constexpr int NPV = (kKeys / 16) * HD * 2;  // pieces of V per chunk: (run of 16 keys, d, half)
+  constexpr int NP = NPK + NPV;
+  constexpr int PER = (NP + T - 1) / T;
+  __shared__ __attribute__((aligned(16))) bf16 ks[2][kKeys][KS];
+  __shared__ __attribute__((aligned(16))) bf16 vs[2][HD][VS];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+  const int n_rep = nq / nkv, hgroups = (n_rep + NW - 1) / NW;
+  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int hin = hg * NW + wave;
+  const bool active = hin < n_rep;  // a wave without a head still helps loading
+  const int head = kvh * n_rep + (active ? hin : 0);
+  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+  const int pos0 = positions[t0];
+  const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
+
+  // Column r of this wave: token t0 + r; it sees keys lo..hi.
+  const bool live = active && r < ntok;
+  const int hi = r < ntok ? pos0 + r : pos0;
+  const int lo = window > 0 ? max(0, hi - window + 1) : 0;
+  bf16x8 qr[HD / 16];
+#pragma unroll
+  for (int c = 0; c < HD / 16; ++c)
+    qr[c] = live ? load_b128(q + (static_cast<size_t>(t0 + r) * nq + head) * HD + 16 * c + 8 * g) : zero_b128();
+  f32x16 o[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+  float m = -INFINITY, l = 0.f;  // m in raw score units; l is this lane's share of the column's sum
+
+  const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int hi_all = pos0 + ntok - 1;
+  const int first = lo_all / kKeys, last = hi_all / kKeys;
+  const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
+
+  auto fetch = [&](int key0, uint4 (&regs)[PER]) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = tid + i * T;
+      regs[i] = uint4{0u, 0u, 0u, 0u};
+      if (p >= NP) continue;
+      const bool is_k = p < NPK;
+      const int pv = p - NPK;
+      const int key = is_k ? key0 + p / SEG : key0 + 16 * (pv / (2 * HD)) + 8 * (pv & 1);
+      const int pi = key / page_size, slot = key % page_size;
+      const int page = pi < table_stride ? table[pi] : -1;
+      if (page < 0) continue;  // released, or not there yet: zeros, and every such key is out of bounds
+      const size_t base = static_cast<size_t>(page) * nkv + kvh;
+      const bf16* src = is_k ? k_cache + (base * page_size + slot) * HD + 8 * (p % SEG)
+                             : v_cache + (base * HD + (pv >> 1) % HD) * page_size + slot;
+      regs[i] = *reinterpret_cast<const uint4*>(src);
+    }
+  };
+  auto stash = [&](int stage, const uint4 (&regs)[PER]) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = tid + i * T;
+      if (p >= NP) continue;
+      if (p < NPK) {
+        *reinterpret_cast<uint4*>(&ks[stage][p / SEG][8 * (p % SEG)]) = regs[i];
+      } else {
+        const int pv = p - NPK, run = pv / (2 * HD), d = (pv >> 1) % HD, h = pv & 1;
+        // keys 8h .. 8h+3 of the run go to places 4h .. 4h+3, keys 8h+4 .. 8h+7 to 8+4h .. 8+4h+3
+        *reinterpret_cast<uint2*>(&vs[stage][d][16 * run + 4 * h]) = uint2{regs[i].x, regs[i].y};
+        *reinterpret_cast<uint2*>(&vs[stage][d][16 * run + 8 + 4 * h]) = uint2{regs[i].z, regs[i].w};
+      }
+    }
+  };
+
+  uint4 regs[PER];
+  fetch(first * kKeys, regs);
+  stash(0, regs);
+  for (int c = first; c <= last; ++c) {
+    const int st = (c - first) & 1;
+    __syncthreads();  // chunk c is in stage st; nobody reads stage st ^ 1 any more
+    if (c < last) fetch((c + 1) * kKeys, regs);
+    const int key0 = c * kKeys;
+    if (active) {
+      // All of the chunk's K operands are asked for before the first product, and all of
+      // its V operands before the softmax arithmetic, so that LDS latency hides behind work.
+      bf16x8 a[2][HD / 16];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int cc = 0; cc < HD / 16; ++cc)
+          a[kt][cc] = *reinterpret_cast<const bf16x8*>(&ks[st][32 * kt + r][16 * cc + 8 * g]);
+      __builtin_amdgcn_sched_barrier(0);
+      // S^T tile kt: rows = keys key0 + 32 kt + 8 (i / 4) + 4 g + i % 4, column r.
+      f32x16 s[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+#pragma unroll
+      for (int cc = 0; cc < HD / 16; ++cc)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kt][cc], qr[cc], s[kt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // V^T operands: for O^T tile dt and the keys of P^T operand (kt, h).
+      bf16x8 va[HD / 32][2][2];
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            va[dt][kt][h] = *reinterpret_cast<const bf16x8*>(&vs[st][32 * dt + r][32 * kt + 16 * h + 8 * g]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (key0 + kKeys - 1 > pos0 || key0 < lo_max) {  // some key of the chunk may be hidden from some column
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + 32 * kt + 8 * (i >> 2) + 4 * g + (i & 3);
+            if (key < lo || key > hi) s[kt][i] = -INFINITY;
+          }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;  // column without a visible key so far
+      const float alpha = __builtin_amdgcn_exp2f((m - m_use) * scale_log2);
+      const float mc = m_use * scale_log2;
+      m = m_new;
+      float sum = 0.f;
+      bf16x8 p[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float x[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][8 * h + e], scale_log2, -mc));
+            sum += x[e];
+          }
+          const uint4 u = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+          p[kt][h] = __builtin_bit_cast(bf16x8, u);
+        }
+      l = l * alpha + sum;
+      if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // O^T tile dt: rows d = 32 dt + ..., k = the chunk's keys in the order P^T holds them.
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int dt = 0; dt < HD / 32; ++dt)
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][kt][h], p[kt][h], o[dt], 0, 0, 0);
+    }
+    if (c < last) stash(st ^ 1, regs);
+  }
+
+  if (!active) return;
+  l += __shfl_xor(l, 32, 64);
+  if (r >= ntok) return;
+  const float inv = 1.f / l;
+  bf16* dst = out + (static_cast<size_t>(t0 + r) * nq + head) * HD + 4 * g;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const float v0 = o[dt][4 * b] * inv, v1 = o[dt][4 * b + 1] * inv, v2 = o[dt][4 * b + 2] * inv,
+                  v3 = o[dt][4 * b + 3] * inv;
+      *reinterpret_cast<uint2*>(dst + 32 * dt + 8 * b) = uint2{pack2(v0, v1), pack2(v2, v3)};
+    }
+}
+
 template <typename F>
 int dispatch_head(int hd, F&& f) {
   switch (hd) {
@@ -582,30 +788,41 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
   const bf16* kp = static_cast<const bf16*>(k_cache);
   const bf16* vp = static_cast<const bf16*>(v_cache);
   bf16* op = static_cast<bf16*>(out);
-  // Up to 128 elements per head, K and V go through LDS (two stages fit in 64 KB);
-  // larger heads read the cache directly in every wave.
+  // Up to 128 elements per head, K and V go through LDS (two stages of 64 keys fit);
+  // larger heads read the cache directly in every wave. form 1: 32x32 tiles, chunks of
+  // 64 keys; forms 2 and 3: 16x16 tiles, chunks of 32 keys (four waves; eight for larger
+  // groups), kept for comparison.
   const bool staged = hd <= 128 && form != 0;
-  const int nw = staged ? (n_rep > 4 && form != 2 ? 8 : 4) : 4;  // form 2: four heads per block even for larger groups
+  const bool tile32 = staged && form == 1;
+  const int nw = staged ? (n_rep > 4 && form != 2 ? 8 : 4) : 4;
   const int hgroups = (n_rep + nw - 1) / nw;
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
   const dim3 grid(n_tiles, nkv * hgroups);
+#define PYRE_PREFILL_ARGS \
+  qp, kp, vp, op, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
     if constexpr (HD <= 128) {
+      if (tile32 && nw == 8) {
+        hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
+        return;
+      }
+      if (tile32) {
+        hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
+        return;
+      }
       if (staged && nw == 8) {
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 8>), grid, dim3(512), 0, stream, qp, kp, vp, op, tiles,
-                           positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window);
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 8>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
         return;
       }
       if (staged) {
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 4>), grid, dim3(256), 0, stream, qp, kp, vp, op, tiles,
-                           positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window);
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 4>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
         return;
       }
     }
-    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, qp, kp, vp, op, tiles, positions,
-                       seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window);
+    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
   });
+#undef PYRE_PREFILL_ARGS
   PYRE_REQUIRE(rc == 0, "attn_prefill_bf16: no kernel for head_dim %d", hd);
   return check_launch("attn_prefill_bf16");
 }
