@@ -531,22 +531,31 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_lds_kernel(
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 64;
 
+// A barrier that waits for this wave's LDS traffic only. __syncthreads() also waits for
+// every global load in flight, which would put the latency of the next chunks' loads
+// into each half-step; their registers are waited for where they are used.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int HD, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
     const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
     int nq, int nkv, int page_size, float scale_log2, int window) {
-  constexpr int KS = HD + 8, VS = kKeys + 8, T = NW * 64;
-  constexpr int SEG = HD / 8;                 // 16-byte pieces of one K row
-  constexpr int NPK = kKeys * SEG;            // pieces of K per chunk
-  constexpr int NPV = (kKeys / 16) * HD * 2;  // pieces of V per chunk: (run of 16 keys, d, half)
-  constexpr int NP = NPK + NPV;
-  constexpr int PER = (NP + T - 1) / T;
-  __shared__ __attribute__((aligned(16))) bf16 ks[2][kKeys][KS];
-  __shared__ __attribute__((aligned(16))) bf16 vs[2][HD][VS];
+  constexpr int KS = HD + 8, VS = kKeys + 8;
+  constexpr int SEG = HD / 8;            // 16-byte pieces of one K row
+  // A run of 16 keys is HD / 32 blocks of 64 pieces (1 KB) of K, contiguous in its page,
+  // and as many of V^T. Block `blk` of a run: K for blk < HD / 32, else V^T; a wave loads
+  // blocks wave, wave + NW, ... of each of the chunk's four runs, one piece per lane.
+  constexpr int BR = 2 * (HD / 32);      // blocks per run
+  constexpr int PB = (BR + NW - 1) / NW;  // blocks per run and wave
+  constexpr int PER = (kKeys / 16) * PB;
+  constexpr int NS = 3;                  // stages: a chunk is read during four half-steps (see below)
+  constexpr int kBytesK = 2 * kKeys * KS, kStage = kBytesK + 2 * HD * VS;  // bytes: a stage is K rows, then V^T rows
+  __shared__ __attribute__((aligned(16))) unsigned char lds[NS * kStage];
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r = lane & 31,
+            g = lane >> 5;
   const int n_rep = nq / nkv, hgroups = (n_rep + NW - 1) / NW;
   const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
   const int hin = hg * NW + wave;
@@ -576,134 +585,211 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   const int first = lo_all / kKeys, last = hi_all / kKeys;
   const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
 
-  auto fetch = [&](int key0, uint4 (&regs)[PER]) {
+  // Where this wave's pieces come from and go to, fixed for the whole kernel. Block j of
+  // a run is K (rows of 16 keys as stored) or V^T (HD rows of 16 keys); the addresses of
+  // a piece differ from run to run by a multiple of the run's slot and of the run's index:
+  //   global: cache + ((page * nkv + kvh) * page_size * HD + slot * g_mul) + g_lane
+  //   LDS:    stage * kStage + run * l_run + l_lane, two 8-byte halves 8 or 16 bytes apart
+  // No branch depends on the page, the block or the run: scalar branches cost far more
+  // here than the few values they would save.
+  const bf16* g_ptr[PB];
+  int g_lane[PB], g_mul[PB], l_lane[PB], l_run[PB], l_half[PB];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = tid + i * T;
-      regs[i] = uint4{0u, 0u, 0u, 0u};
-      if (p >= NP) continue;
-      const bool is_k = p < NPK;
-      const int pv = p - NPK;
-      const int key = is_k ? key0 + p / SEG : key0 + 16 * (pv / (2 * HD)) + 8 * (pv & 1);
-      const int pi = key / page_size, slot = key % page_size;
-      const int page = pi < table_stride ? table[pi] : -1;
-      if (page < 0) continue;  // released, or not there yet: zeros, and every such key is out of bounds
-      const size_t base = static_cast<size_t>(page) * nkv + kvh;
-      const bf16* src = is_k ? k_cache + (base * page_size + slot) * HD + 8 * (p % SEG)
-                             : v_cache + (base * HD + (pv >> 1) % HD) * page_size + slot;
-      regs[i] = *reinterpret_cast<const uint4*>(src);
+  for (int j = 0; j < PB; ++j) {
+    const int blk = min(wave + NW * j, BR - 1);  // a wave beyond the last block repeats it (same bytes, same place)
+    const bool is_k = blk < HD / 32;
+    const int idx = (is_k ? blk : blk - HD / 32) * 64 + lane;
+    g_ptr[j] = is_k ? k_cache : v_cache;
+    g_mul[j] = is_k ? HD : 1;
+    g_lane[j] = is_k ? 8 * idx : (idx >> 1) * page_size + 8 * (idx & 1);
+    // V^T: keys 8h .. 8h+3 of the run go to places 4h .. 4h+3, keys 8h+4 .. 8h+7 to 8+4h .. 8+4h+3
+    l_lane[j] = is_k ? 2 * ((idx / SEG) * KS + 8 * (idx % SEG)) : kBytesK + 2 * ((idx >> 1) * VS + 4 * (idx & 1));
+    l_run[j] = is_k ? 2 * 16 * KS : 2 * 16;
+    l_half[j] = is_k ? 8 : 16;
+  }
+  // (pi, sl): index into the block table and slot within that page of the first key of
+  // the next chunk to look up; both advance by whole runs, without a division per chunk.
+  // The pages of a chunk are looked up one load ahead of the chunk's own loads, so that
+  // the latency of the table is never waited for. A page that is not there (released, or
+  // past the request's end) reads page 0 instead: all its keys are out of every column's bounds.
+  int pi = (first * kKeys) / page_size, sl = (first * kKeys) % page_size;
+  int run_page[kKeys / 16], run_slot[kKeys / 16];
+  auto lookup = [&]() {
+#pragma unroll
+    for (int run = 0; run < kKeys / 16; ++run) {
+      run_page[run] = table[min(pi, table_stride - 1)];
+      run_slot[run] = sl;
+      sl += 16;
+      const bool wrap = sl >= page_size;
+      sl = wrap ? 0 : sl;
+      pi += wrap ? 1 : 0;
     }
+  };
+  const size_t page_elems = static_cast<size_t>(page_size) * HD;
+  auto fetch = [&](uint4 (&regs)[PER]) {
+    size_t base[kKeys / 16];
+    int slot[kKeys / 16];
+#pragma unroll
+    for (int run = 0; run < kKeys / 16; ++run) {
+      base[run] = (static_cast<size_t>(max(run_page[run], 0)) * nkv + kvh) * page_elems;
+      slot[run] = run_slot[run];
+    }
+    lookup();  // for the chunk after this one
+#pragma unroll
+    for (int run = 0; run < kKeys / 16; ++run)
+#pragma unroll
+      for (int j = 0; j < PB; ++j)
+        regs[run * PB + j] = *reinterpret_cast<const uint4*>(g_ptr[j] + base[run] + slot[run] * g_mul[j] + g_lane[j]);
   };
   auto stash = [&](int stage, const uint4 (&regs)[PER]) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = tid + i * T;
-      if (p >= NP) continue;
-      if (p < NPK) {
-        *reinterpret_cast<uint4*>(&ks[stage][p / SEG][8 * (p % SEG)]) = regs[i];
-      } else {
-        const int pv = p - NPK, run = pv / (2 * HD), d = (pv >> 1) % HD, h = pv & 1;
-        // keys 8h .. 8h+3 of the run go to places 4h .. 4h+3, keys 8h+4 .. 8h+7 to 8+4h .. 8+4h+3
-        *reinterpret_cast<uint2*>(&vs[stage][d][16 * run + 4 * h]) = uint2{regs[i].x, regs[i].y};
-        *reinterpret_cast<uint2*>(&vs[stage][d][16 * run + 8 + 4 * h]) = uint2{regs[i].z, regs[i].w};
+    for (int run = 0; run < kKeys / 16; ++run)
+#pragma unroll
+      for (int j = 0; j < PB; ++j) {
+        unsigned char* dst = lds + stage * kStage + run * l_run[j] + l_lane[j];
+        const uint4 v = regs[run * PB + j];
+        *reinterpret_cast<uint2*>(dst) = uint2{v.x, v.y};
+        *reinterpret_cast<uint2*>(dst + l_half[j]) = uint2{v.z, v.w};
       }
-    }
   };
 
+  // The loop runs in half-steps with a barrier after each. A wave alternates between a
+  // matrix half-step (O^T += V^T P^T of the previous chunk, then S^T of the next) and an
+  // arithmetic half-step (softmax of that S^T, its share of the loads). The second wave of
+  // each SIMD (waves NW/2 ..) runs one half-step behind the first, so that at any time one
+  // of the two is on the matrix cores and the other on the vector ALU.
+  //   chunk x (counted from `first`) is read in half-steps 2x .. 2x+3, lies in stage x % 3,
+  //   and is written in half-steps 2x-2 (second waves) and 2x-1 (first waves).
+  const int n = last - first + 1;
+  const int off = NW == 8 ? wave >> 2 : 0;
   uint4 regs[PER];
-  fetch(first * kKeys, regs);
+  lookup();
+  fetch(regs);
   stash(0, regs);
-  for (int c = first; c <= last; ++c) {
-    const int st = (c - first) & 1;
-    __syncthreads();  // chunk c is in stage st; nobody reads stage st ^ 1 any more
-    if (c < last) fetch((c + 1) * kKeys, regs);
-    const int key0 = c * kKeys;
-    if (active) {
-      // All of the chunk's K operands are asked for before the first product, and all of
-      // its V operands before the softmax arithmetic, so that LDS latency hides behind work.
-      bf16x8 a[2][HD / 16];
+  int held = 1, held_stage = 1;  // the chunk whose pieces `regs` holds, and its stage
+  if (held < n) fetch(regs);
+  // The query operands have arrived before the loop starts. Without this the compiler,
+  // which cannot tell the first round from the others, waits for all loads in flight
+  // (the next chunk's among them) before the first product of every round.
+#pragma unroll
+  for (int c = 0; c < HD / 16; ++c) asm volatile("" : "+v"(qr[c]));
+  lds_barrier();
+  f32x16 s[2];
+  bf16x8 p[2][2];
+
+  // S^T of the chunk in stage sk: tile kt has rows = keys key0 + 32 kt + 8 (i / 4) + 4 g + i % 4, column r.
+  auto scores = [&](int sk) {
+    constexpr int AHEAD = 4;  // head slices whose operands are in flight
+    bf16x8 a[AHEAD][2];
+    auto load_k = [&](int slot, int cc) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+        a[slot][kt] = *reinterpret_cast<const bf16x8*>(lds + sk * kStage + 2 * ((32 * kt + r) * KS + 16 * cc + 8 * g));
+    };
+#pragma unroll
+    for (int cc = 0; cc < AHEAD && cc < HD / 16; ++cc) load_k(cc, cc);
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+#pragma unroll
+    for (int cc = 0; cc < HD / 16; ++cc) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cc % AHEAD][kt], qr[cc], s[kt], 0, 0, 0);
+      if (cc + AHEAD < HD / 16) load_k(cc % AHEAD, cc + AHEAD);
+    }
+  };
+  // O^T += V^T P^T for the chunk in stage sv; k = the chunk's keys in the order P^T holds them.
+  auto weighted_values = [&](int sv) {
+    bf16x8 va[2][HD / 32];
+    auto load_v = [&](int slot, int pair) {  // pair = 2 kt + h
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+        va[slot][dt] = *reinterpret_cast<const bf16x8*>(lds + sv * kStage + kBytesK + 2 * ((32 * dt + r) * VS + 16 * pair + 8 * g));
+    };
+    load_v(0, 0);
+    load_v(1, 1);
+#pragma unroll
+    for (int pair = 0; pair < 4; ++pair) {
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[pair & 1][dt], p[pair >> 1][pair & 1], o[dt], 0, 0, 0);
+      if (pair + 2 < 4) load_v(pair & 1, pair + 2);
+    }
+  };
+  // P^T = exp2(S^T scale - running maximum), packed as the next product's operands.
+  auto softmax = [&](int key0) {
+    if (key0 + kKeys - 1 > pos0 || key0 < lo_max) {  // some key of the chunk may be hidden from some column
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int cc = 0; cc < HD / 16; ++cc)
-          a[kt][cc] = *reinterpret_cast<const bf16x8*>(&ks[st][32 * kt + r][16 * cc + 8 * g]);
-      __builtin_amdgcn_sched_barrier(0);
-      // S^T tile kt: rows = keys key0 + 32 kt + 8 (i / 4) + 4 g + i % 4, column r.
-      f32x16 s[2];
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + 32 * kt + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (key < lo || key > hi) s[kt][i] = -INFINITY;
+        }
+    }
+    float mx = -INFINITY;
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // column without a visible key so far
+    const float alpha = __builtin_amdgcn_exp2f((m - m_use) * scale_log2);
+    const float mc = m_use * scale_log2;
+    m = m_new;
+    float sum = 0.f;
 #pragma unroll
-      for (int cc = 0; cc < HD / 16; ++cc)
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kt][cc], qr[cc], s[kt], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      // V^T operands: for O^T tile dt and the keys of P^T operand (kt, h).
-      bf16x8 va[HD / 32][2][2];
+      for (int h = 0; h < 2; ++h) {
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][8 * h + e], scale_log2, -mc));
+          sum += x[e];
+        }
+        const uint4 w = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+        p[kt][h] = __builtin_bit_cast(bf16x8, w);
+      }
+    l = l * alpha + sum;
+    if (__any(alpha != 1.f)) {
 #pragma unroll
       for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int h = 0; h < 2; ++h)
-            va[dt][kt][h] = *reinterpret_cast<const bf16x8*>(&vs[st][32 * dt + r][32 * kt + 16 * h + 8 * g]);
-      __builtin_amdgcn_sched_barrier(0);
-      if (key0 + kKeys - 1 > pos0 || key0 < lo_max) {  // some key of the chunk may be hidden from some column
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = key0 + 32 * kt + 8 * (i >> 2) + 4 * g + (i & 3);
-            if (key < lo || key > hi) s[kt][i] = -INFINITY;
-          }
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;  // column without a visible key so far
-      const float alpha = __builtin_amdgcn_exp2f((m - m_use) * scale_log2);
-      const float mc = m_use * scale_log2;
-      m = m_new;
-      float sum = 0.f;
-      bf16x8 p[2][2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          float x[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][8 * h + e], scale_log2, -mc));
-            sum += x[e];
-          }
-          const uint4 u = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
-          p[kt][h] = __builtin_bit_cast(bf16x8, u);
-        }
-      l = l * alpha + sum;
-      if (__any(alpha != 1.f)) {
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // O^T tile dt: rows d = 32 dt + ..., k = the chunk's keys in the order P^T holds them.
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int dt = 0; dt < HD / 32; ++dt)
-            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[dt][kt][h], p[kt][h], o[dt], 0, 0, 0);
+        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
     }
-    if (c < last) stash(st ^ 1, regs);
+  };
+  // This wave's share of the loads: the held chunk into its stage, the next one into registers.
+  auto load_work = [&]() {
+    if (held < n) stash(held_stage, regs);
+    ++held;
+    held_stage = held_stage == NS - 1 ? 0 : held_stage + 1;
+    if (held < n) fetch(regs);
+  };
+
+  if (off) {  // the second waves start one half-step later
+    load_work();
+    lds_barrier();
   }
+  if (active) scores(0);
+  int st = 0;  // stage of chunk c
+  for (int c = 0; c < n; ++c) {
+    lds_barrier();
+    if (active) softmax((first + c) * kKeys);
+    load_work();
+    lds_barrier();
+    const int nx = st == NS - 1 ? 0 : st + 1;
+    if (active) {
+      weighted_values(st);
+      if (c + 1 < n) scores(nx);
+    }
+    st = nx;
+  }
+  lds_barrier();
+  if (!off) lds_barrier();  // every wave passes the same number of barriers
 
   if (!active) return;
   l += __shfl_xor(l, 32, 64);
