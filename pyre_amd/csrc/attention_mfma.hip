@@ -517,16 +517,16 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_lds_kernel(
 // ---------------------------------------------------------------------------
 // Prefill on 32x32x16 tiles: the NW waves of a block take NW query heads of one
 // key/value head over the same 32 tokens (one MFMA tile of columns per wave);
-// keys and values come through LDS in chunks of 64, double-buffered, loaded once
+// keys and values come through LDS in chunks of 64, three stages, loaded once
 // per block. Per chunk and wave: S^T (64 keys x 32 tokens) in two tiles, one
 // exchange between the two lanes that share a column for the running maximum,
 // and O^T (HD x 32) += V^T P^T. The sum of a column is kept per lane (each lane
 // adds the keys it holds) and joined once at the end.
 //
-//   ks[stage][key][HD + 8]   K rows as stored; the padding puts 16 rows on distinct banks
-//   vs[stage][d][64 + 8]     V^T; within each run of 16 keys the order is
-//                            (4g + j, 8 + 4g + j -> 8g + j, 8g + 4 + j), so that the eight
-//                            keys a lane needs for one MFMA are 16 contiguous bytes
+// A stage is K rows as stored, [key][HD + 8] (the padding puts 16 rows on distinct
+// banks), followed by V^T, [d][64 + 8]; within each run of 16 keys the V^T order is
+// (4g + j, 8 + 4g + j -> 8g + j, 8g + 4 + j), so that the eight keys a lane needs
+// for one MFMA are 16 contiguous bytes.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 64;

@@ -70,8 +70,10 @@ int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache, const v
                           int page_size, float scale, int window, hipStream_t stream);
 
 // Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
-// all tokens of a tile from one request at consecutive positions. form 1 stages
-// K and V through LDS (heads of up to 128 elements), form 0 never does.
+// all tokens of a tile from one request at consecutive positions. Heads of up to 128
+// elements: form 1 stages K and V through LDS in chunks of 64 keys for 32x32 MFMA tiles,
+// forms 2 and 3 in chunks of 32 keys for 16x16 tiles (kept for comparison); form 0, and
+// every larger head, reads the cache directly in each wave.
 int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
                            const int* tiles, int n_tiles, const int* positions,
                            const int* seq_of_token, const int* block_table, int table_stride,
