@@ -109,8 +109,17 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
 
   auto value4 = [&](int col) {
-    float4 v = Vec4<TI>::load(qkv + in_row + col);
-    for (int p = 1; p < n_partials; ++p) v = add4(v, Vec4<TI>::load(qkv + p * partial_stride + in_row + col));
+    const TI* src = qkv + in_row + col;
+    float4 v = Vec4<TI>::load(src);
+    int p = 1;
+    for (; p + 3 < n_partials; p += 4) {  // four loads in flight, added in the order p, p+1, ...
+      const float4 d0 = Vec4<TI>::load(src + p * partial_stride);
+      const float4 d1 = Vec4<TI>::load(src + (p + 1) * partial_stride);
+      const float4 d2 = Vec4<TI>::load(src + (p + 2) * partial_stride);
+      const float4 d3 = Vec4<TI>::load(src + (p + 3) * partial_stride);
+      v = add4(add4(add4(add4(v, d0), d1), d2), d3);
+    }
+    for (; p < n_partials; ++p) v = add4(v, Vec4<TI>::load(src + p * partial_stride));
     if (bias) {
       v.x += load_as_float(bias, bias_dt, col);
       v.y += load_as_float(bias, bias_dt, col + 1);

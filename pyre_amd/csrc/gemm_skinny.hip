@@ -34,6 +34,12 @@ constexpr int kRun = 128;  // k elements a wave takes at a time
 __device__ inline bf16x8 ld128(const bf16* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
+// Weights are read once per step: a non-temporal load keeps them from displacing what
+// the caches hold and streams measurably faster from HBM.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ inline bf16x8 ld128_stream(const bf16* p) {
+  return __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+}
 __device__ inline bf16x8 zero128() {
   uint4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, z);
@@ -364,7 +370,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_staged_kernel(const bf16* __r
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
       const int k = kr + 8 * ((tid + 256 * i) % (kRun / 8));
-      wr[i] = (wsrc[i] && k < kend) ? ld128(wsrc[i] + kr) : zero128();
+      wr[i] = (wsrc[i] && k < kend) ? ld128_stream(wsrc[i] + kr) : zero128();
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
