@@ -56,6 +56,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has")
     ap.add_argument("--points", default="1,64", help="further decode batch sizes ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiling): no decode steps")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-tune", action="store_true", help="keep the BLAS library's default kernels for prefill")
     ap.add_argument("--opt", action="append", default=[], metavar="KEY=VALUE",
@@ -146,6 +147,10 @@ def main() -> int:
                    "frac": round(fl / (ms / 1e3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12), 4)}
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
 
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s (%s shape, %d tokens)" % (args.model, PREFILL_TOKENS),
+                          "prefill": prefill, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32"}))
+        return 0
     value, ms_per_step = decode(args.batch, args.steps, args.warmup)
     mean_ctx = args.context - args.steps / 2
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token

@@ -7,6 +7,11 @@ reads the ``kernels`` view of the rocpd SQLite file that
 (``DIR/NAME_results.db``) and prints calls, total, share, mean, min and max time per
 kernel name, longest total first. ``--tail-ms MS`` keeps only the launches of the
 last MS milliseconds of the trace (the timed steps of a benchmark, without its set-up).
+
+    python -m pyre_amd.profile_summary --counters COUNTERS.csv [--match TEXT]
+
+reads the ``*_counter_collection.csv`` of ``rocprofv3 --pmc ... --output-format csv`` and
+prints, per kernel name, the mean of each counter over the kernel's launches.
 """
 
 from __future__ import annotations
@@ -33,6 +38,27 @@ def summarise(path: str, top: int = 25, match: str | None = None, tail_ms: float
     return "\n".join(out)
 
 
+def counters(path: str, match: str | None = None) -> str:
+    import collections
+    import csv
+
+    total: dict = collections.defaultdict(lambda: collections.defaultdict(float))
+    count: dict = collections.Counter()
+    with open(path, newline="") as f:
+        for row in csv.DictReader(f):
+            name = row["Kernel_Name"]
+            if match and match not in name:
+                continue
+            total[name][row["Counter_Name"]] += float(row["Counter_Value"])
+            count[(name, row["Counter_Name"])] += 1
+    out = []
+    for name, vals in total.items():
+        out.append(name[:100])
+        for c, v in sorted(vals.items()):
+            out.append(f"    {c:34s} {v / count[(name, c)]:18.1f}   (mean of {count[(name, c)]} launches)")
+    return "\n".join(out)
+
+
 def main(argv: list[str]) -> int:
     if not argv:
         print(__doc__)
@@ -42,6 +68,9 @@ def main(argv: list[str]) -> int:
         i = argv.index("--match")
         match = argv[i + 1]
         del argv[i:i + 2]
+    if "--counters" in argv:
+        print(counters(argv[argv.index("--counters") + 1], match))
+        return 0
     tail_ms = None
     if "--tail-ms" in argv:
         i = argv.index("--tail-ms")
