@@ -362,7 +362,8 @@ def test_sample_inverse_cdf():
 
 @pytest.mark.parametrize("form", [0, 1, 2])
 @pytest.mark.parametrize("m", [1, 7, 16, 33, 64])
-@pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (3584, 3584, 3), (1000, 136, 2), (131, 8, 1), (70000, 96, 1)])
+@pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (3584, 3584, 3), (1000, 136, 2), (131, 8, 1), (70000, 96, 1),
+                                        (3584, 18944, 8)])
 def test_gemm_skinny(m, n, k, ksplit, form):
     ops = _ops()
     assert ops.gemm_skinny_supports(m, n, k, k, k)
