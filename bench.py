@@ -106,8 +106,9 @@ def main() -> int:
         """(tokens per second, ms per step) of `steps` decode steps at `batch`."""
         sched = Scheduler(engine, max_batch=batch)
         # Requests whose prompt is done decode while the others are still being
-        # prefilled (about two steps each), so leave room for those tokens too.
-        start_ctx = args.context - (steps + warmup) - 2 * batch - 2
+        # prefilled (one step per portion of a prompt), so leave room for those tokens too.
+        portions = -(-args.context // PREFILL_TOKENS)
+        start_ctx = args.context - (steps + warmup) - portions * batch - 2
         for _ in range(batch):
             sched.add_request(prompt(start_ctx), max_new_tokens=args.context - start_ctx)
         t_fill = time.perf_counter()
