@@ -151,3 +151,39 @@ def test_cli_generates(model_dirs, tmp_path, capsys):
 
     res = json.loads(out.read_text())
     assert [len(g) for g in res["generated"]] == [5, 5]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_one_step_ahead_changes_no_token(dtype, model_dirs):
+    """Staggered requests of different lengths, some sampled with a temperature, one
+    ending early by its end-of-sequence token, on few pages: the tokens with decode steps
+    put on the device one step ahead (tokens fed there) are those of a scheduler that
+    waits for every step."""
+    from pyre_amd.api import Scheduler
+
+    eng = _load(model_dirs["tiny-c"], dtype, use_graphs=True, max_cached_tokens=640)
+    vocab = eng.vocab_size
+    prompts = [random_ids(vocab, n, seed=100 + n) for n in (5, 40, 17, 64, 9, 33)]
+    lens = [30, 12, 44, 20, 37, 25]
+
+    def run(ahead, eos):
+        s = Scheduler(eng, max_batch=4)
+        s.lookahead = ahead
+        ids, steps = [], 0
+        for i, (p, n) in enumerate(zip(prompts, lens)):
+            ids.append(s.add_request(p, n, eos_id=eos if i == 2 else None, temperature=0.7 if i % 2 else 0.0, seed=i))
+            s.step()                      # requests arrive while others run
+            steps += 1
+        out = s.run()
+        assert eng.cache.page_groups[0].allocator.num_used == 0
+        return [out[i] for i in ids], s
+
+    base, _ = run(False, None)
+    eos = base[2][10]                     # request 2 will now end at the first occurrence of this token
+    want, s0 = run(False, eos)
+    got, s1 = run(True, eos)
+    assert got == want
+    assert len(want[2]) <= 11 and want[2][-1] == eos
+    assert s1.lookahead and not s0.lookahead
+    # the steps that ran ahead are fewer host round trips, not fewer engine steps
+    assert eng.graph_replays > 0
