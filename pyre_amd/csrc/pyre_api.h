@@ -44,7 +44,8 @@ int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, cons
 int pyre_gemm_skinny_supports(int M, int N, int K, long ldx, long ldw);
 
 // out: float32 [ksplit][M][N] partial sums of X[M, K] W[N, K]^T. form 0: the waves
-// of a block split k (fewest rows); form 1: X staged through LDS (more rows).
+// of a block split k, operands straight from memory; form 1: X staged through LDS;
+// form 2: W and X staged through LDS, whole cache lines per load.
 int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N,
                           int K, int ksplit, int form, hipStream_t stream);
 
