@@ -17,7 +17,8 @@ generated so far (which it keeps). A request that could not fit the pool even
 alone is refused when it is added. (The reference lets ``MemoryError`` escape,
 `pyre/paged_cache.py:58-67`.)
 
-While every running request is decoding and nobody waits, the next step is put on
+While every running request is decoding and no waiting request could be admitted
+(nobody waits, or as many run as may), the next step is put on
 the device before the host has seen this step's tokens: its batch is known (the same
 requests, one position further, minus those that reach their length), and the tokens
 are fed on the device from the sampler's ids. The host then reads this step's tokens
@@ -264,15 +265,17 @@ class Scheduler:
 
     def _run_ahead(self, plan: StepPlan, sampling: list[Request]):
         """Put the next step on the device if it is known without this step's tokens:
-        all running requests have just been sampled for, nobody waits, and the pages are
-        there. Returns (plan, logits) or None. The sampler's ids of this step must
+        all running requests have just been sampled for, no waiting request could join
+        them, and the pages are there. Returns (plan, logits) or None. The sampler's ids of this step must
         already be on the stream."""
-        if self.waiting or len(sampling) != len(self.running) or len(plan.entries) != len(sampling):
+        if len(sampling) != len(self.running) or len(plan.entries) != len(sampling):
             return None
         rows = [(i, r) for i, r in enumerate(sampling)
                 if not r.done and len(r.generated) + 1 < r.params.max_new_tokens]
         if not rows or len(rows) > self.token_budget:
             return None
+        if self.waiting and len(rows) < self.max_batch:
+            return None  # the next step may admit a waiting request: it has to be planned with this step's results
         if sum(self.cache.pages_needed(r.seq_id, 1) for _, r in rows) > self.cache.free_pages():
             return None
         nxt = StepPlan([PlannedEntry(r, r.num_computed, 1, True) for _, r in rows], [], [])

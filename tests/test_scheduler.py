@@ -264,3 +264,29 @@ def test_a_request_added_meanwhile_waits_one_step():
     assert [r.seq_id for r in s.waiting] == [b]
     out = s.run()
     assert out[a] == expected([1, 2, 3], 8) and out[b] == expected([9, 9], 4)
+
+
+def test_running_ahead_while_others_wait_for_a_free_place():
+    """With as many running as may run, nobody can be admitted next step, so the steps run
+    ahead although requests wait; when one reaches its length, the next step is planned
+    as usual and admits the first of them."""
+    prompts = [[i + 1, i + 2] for i in range(6)]
+    lens = [12, 7, 9, 12, 5, 6]
+
+    def run(ahead):
+        eng = AheadEngine(pages=64, max_num_seqs=2)
+        s = Scheduler(eng)
+        s.sampler = AheadSampler(s)
+        s.lookahead = ahead
+        ids = [s.add_request(p, n) for p, n in zip(prompts, lens)]
+        out = s.run()
+        assert eng.cache.free_pages() == 64
+        return eng, [out[i] for i in ids]
+
+    eng0, plain = run(False)
+    eng1, ahead = run(True)
+    assert ahead == plain == [expected(p, n) for p, n in zip(prompts, lens)]
+    assert eng1.ahead_steps > 15
+    # the order of admission is first come, first served in both
+    first_seen = lambda eng: [rid for step in eng.steps for rid, _, _ in step if not any(rid == r for st in eng.steps[:eng.steps.index(step)] for r, _, _ in st)]  # noqa: E731
+    assert first_seen(eng1) == first_seen(eng0) == list(range(6))
