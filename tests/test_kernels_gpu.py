@@ -243,7 +243,7 @@ def test_attn_generic(dtype, nq, nkv, hd, page, window):
         assert torch.allclose(out[0].double().cpu(), dense[0][1][0].double().repeat_interleave(nq // nkv, 0), atol=tol)
 
 
-MFMA_SHAPES = [(28, 4, 128, 16), (8, 8, 64, 16), (6, 1, 32, 32), (40, 2, 96, 16), (3, 1, 256, 48)]
+MFMA_SHAPES = [(28, 4, 128, 16), (8, 8, 64, 16), (6, 1, 32, 32), (40, 2, 96, 16), (3, 1, 256, 48), (4, 2, 64, 48)]
 
 
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
