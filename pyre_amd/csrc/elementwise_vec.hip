@@ -120,11 +120,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
       v = add4(add4(add4(add4(v, d0), d1), d2), d3);
     }
     for (; p < n_partials; ++p) v = add4(v, Vec4<TI>::load(src + p * partial_stride));
-    if (bias) {
-      v.x += load_as_float(bias, bias_dt, col);
-      v.y += load_as_float(bias, bias_dt, col + 1);
-      v.z += load_as_float(bias, bias_dt, col + 2);
-      v.w += load_as_float(bias, bias_dt, col + 3);
+    if (bias) {  // col is a multiple of 4: one load of four
+      v = add4(v, bias_dt == kF32 ? Vec4<float>::load(static_cast<const float*>(bias) + col)
+                                  : Vec4<bf16>::load(static_cast<const bf16*>(bias) + col));
     }
     return v;
   };
