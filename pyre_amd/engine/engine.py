@@ -235,9 +235,19 @@ class Engine:
             decode_tokens=views["decode_tokens"], prefill_tiles=views["prefill_tiles"])
         return ctx, self._layer_views(views)
 
+    def _forward(self, ctx, caches):
+        """The model's kernels on torch's current stream, asked for once."""
+        from pyre_amd.hip import ops
+
+        ops.use_stream(torch.cuda.current_stream().cuda_stream)
+        try:
+            return self.model.forward(ctx, caches)
+        finally:
+            ops.use_stream(None)
+
     def _run(self, hb, fed_ids=None):
         ctx, caches = self._context(hb, fed_ids)
-        return self.model.forward(ctx, caches)
+        return self._forward(ctx, caches)
 
     def _step_captured(self, hb, rows: int, width: int, fed_ids=None):
         """A decode step at a fixed size (``rows`` requests, tables ``width`` pages
@@ -249,7 +259,7 @@ class Engine:
         state = self._graphs.get(key)
         if state is None:
             ctx, caches = self._context(padded, fed_ids)
-            logits = self.model.forward(ctx, caches)
+            logits = self._forward(ctx, caches)
             self._graphs[key] = "warm"
             return logits[:live]
         if state == "warm":
@@ -259,7 +269,7 @@ class Engine:
             ws.frozen = True
             try:
                 with torch.cuda.graph(graph):
-                    logits = self.model.forward(ctx, caches)
+                    logits = self._forward(ctx, caches)
             finally:
                 ws.frozen = False
             state = self._graphs[key] = (graph, logits)

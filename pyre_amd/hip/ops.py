@@ -25,8 +25,18 @@ def dtype_code(t: torch.Tensor | torch.dtype) -> int:
         raise KernelError(f"unsupported element type {dt}; kernels take float32 and bfloat16") from None
 
 
+_STREAM: int | None = None
+
+
+def use_stream(handle: int | None) -> None:
+    """Put every kernel on this HIP stream until told otherwise (None: ask torch for its
+    current stream at every call again). A step asks once instead of once per kernel."""
+    global _STREAM
+    _STREAM = handle
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return _STREAM if _STREAM is not None else torch.cuda.current_stream().cuda_stream
 
 
 def _dev(*tensors: torch.Tensor | None) -> None:
