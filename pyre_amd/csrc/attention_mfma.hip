@@ -225,16 +225,19 @@ __device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge,
 // ---------------------------------------------------------------------------
 // Decode: grid (ceil(nsplits / 4), nkv * qtiles, tokens), 4 waves = 4 splits.
 // ---------------------------------------------------------------------------
-template <int HD>
+// ONE_BLOCK: at most four splits, the four waves of a single block: they join their
+// partial results through LDS and store the finished rows in `out`; the partial buffers
+// and the second kernel are not needed.
+template <int HD, bool ONE_BLOCK>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int* __restrict__ tokens, const int* __restrict__ positions,
     const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, int nq, int nkv, int page_size,
-    float scale_log2, int window, int nsplits) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml, bf16* __restrict__ out, int nq, int nkv,
+    int page_size, float scale_log2, int window, int nsplits) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int split = blockIdx.x * 4 + wave;
-  if (split >= nsplits) return;
+  if (!ONE_BLOCK && split >= nsplits) return;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
   const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
   const int head0 = kvh * n_rep + qt * 16, nheads = min(16, n_rep - qt * 16);
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
   const int first = lo / kChunk, last = pos / kChunk;
   const int per = (last - first + 1 + nsplits - 1) / nsplits;
-  const int begin = first + split * per, end = min(last + 1, begin + per);
+  const int begin = first + split * per, end = split < nsplits ? min(last + 1, begin + per) : begin;
   if constexpr (HD <= 128) {
     // Two register sets: while one chunk is multiplied the next one's loads are in flight.
     ChunkRegs<HD> ra, rb;
@@ -275,7 +278,37 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
   }
 
-  if (r < nheads) {
+  if constexpr (ONE_BLOCK) {
+    // out[head, :] = sum_w o_w 2^(m_w - M) / sum_w l_w 2^(m_w - M), waves in the order 0..3.
+    __shared__ float acc_s[4][16][HD + 4];
+    __shared__ float ml_s[4][16][2];
+    if (g == 0) {
+      ml_s[wave][r][0] = m[0];
+      ml_s[wave][r][1] = l[0];
+    }
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) *reinterpret_cast<f32x4*>(&acc_s[wave][r][dt * 16 + 4 * g]) = o[dt][0];
+    __syncthreads();
+    for (int i = threadIdx.x; i < nheads * (HD / 4); i += 256) {
+      const int h = i / (HD / 4), d = 4 * (i % (HD / 4));
+      float M = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_s[w][h][0]);
+      float L = 0.f;
+      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float mw = ml_s[w][h][0];
+        const float ww = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+        L += ml_s[w][h][1] * ww;
+        sum += *reinterpret_cast<const f32x4*>(&acc_s[w][h][d]) * ww;
+      }
+      // L is 0 only for a row that sees no key at all (padding of a captured step).
+      const float inv = L > 0.f ? 1.f / L : 0.f;
+      *reinterpret_cast<uint2*>(out + (static_cast<size_t>(tok) * nq + head0 + h) * HD + d) =
+          uint2{pack2(sum[0] * inv, sum[1] * inv), pack2(sum[2] * inv, sum[3] * inv)};
+    }
+  } else if (r < nheads) {
     const size_t slot = (static_cast<size_t>(idx) * nq + head0 + r) * nsplits + split;
     if (g == 0) {
       part_ml[2 * slot] = m[0];
@@ -846,10 +879,17 @@ extern "C" int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cac
   const float scale_log2 = scale * kLog2e;
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
-    hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
+    if (nsplits <= 4) {  // one block per (token, key/value head): its waves join their results themselves
+      hipLaunchKernelGGL((attn_decode_kernel<HD, true>), grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
+                         static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), tokens,
+                         positions, seq_of_token, block_table, table_stride, part_acc, part_ml,
+                         static_cast<bf16*>(out), nq, nkv, page_size, scale_log2, window, nsplits);
+      return;
+    }
+    hipLaunchKernelGGL((attn_decode_kernel<HD, false>), grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
                        static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), tokens,
-                       positions, seq_of_token, block_table, table_stride, part_acc, part_ml, nq, nkv,
-                       page_size, scale_log2, window, nsplits);
+                       positions, seq_of_token, block_table, table_stride, part_acc, part_ml,
+                       static_cast<bf16*>(out), nq, nkv, page_size, scale_log2, window, nsplits);
     hipLaunchKernelGGL(attn_decode_reduce<HD>, dim3(n_tokens, nq), dim3(128), 0, stream,
                        part_acc, part_ml, tokens, static_cast<bf16*>(out), nq, nsplits);
   });
