@@ -569,7 +569,10 @@ constexpr int kKeys = 64;
 // into each half-step; their registers are waited for where they are used.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int HD, int NW>
+// LOADER: the block's last wave has no head of its own (the group has fewer heads than
+// the block has waves) and does all the loading; the others only compute, and keep the
+// registers and the instructions of the loads for themselves.
+template <int HD, int NW, bool LOADER>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
@@ -617,6 +620,69 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   const int hi_all = pos0 + ntok - 1;
   const int first = lo_all / kKeys, last = hi_all / kKeys;
   const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
+
+  const int n = last - first + 1;
+  if (LOADER && wave == NW - 1) {
+    // Chunk x is written in half-step 2x - 2, as soon as the chunk that lay in its stage
+    // has been left, and its loads were asked for two half-steps before that.
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    int pi = (first * kKeys) / page_size, sl = (first * kKeys) % page_size;
+    const size_t page_elems = static_cast<size_t>(page_size) * HD;
+    u32x4 lr[(kKeys / 16) * BR];
+    auto fetch_all = [&]() {
+#pragma unroll
+      for (int run = 0; run < kKeys / 16; ++run) {
+        const int page = table[min(pi, table_stride - 1)];
+        const size_t base = (static_cast<size_t>(max(page, 0)) * nkv + kvh) * page_elems;
+#pragma unroll
+        for (int blk = 0; blk < BR; ++blk) {
+          constexpr int kHalfBlocks = HD / 32;
+          const bool is_k = blk < kHalfBlocks;
+          const int idx = (is_k ? blk : blk - kHalfBlocks) * 64 + lane;
+          const bf16* src = is_k ? k_cache + base + static_cast<size_t>(sl) * HD + 8 * idx
+                                 : v_cache + base + static_cast<size_t>(idx >> 1) * page_size + sl + 8 * (idx & 1);
+          lr[run * BR + blk] = *reinterpret_cast<const u32x4*>(src);
+        }
+        sl += 16;
+        const bool wrap = sl >= page_size;
+        sl = wrap ? 0 : sl;
+        pi += wrap ? 1 : 0;
+      }
+    };
+    auto stash_all = [&](int stage) {
+#pragma unroll
+      for (int run = 0; run < kKeys / 16; ++run)
+#pragma unroll
+        for (int blk = 0; blk < BR; ++blk) {
+          const u32x4 v = lr[run * BR + blk];
+          if (blk < HD / 32) {
+            const int idx = blk * 64 + lane;
+            *reinterpret_cast<u32x4*>(lds + stage * kStage + 2 * ((16 * run + idx / SEG) * KS + 8 * (idx % SEG))) = v;
+          } else {
+            const int idx = (blk - HD / 32) * 64 + lane, d = idx >> 1, h = idx & 1;
+            // keys 8h .. 8h+3 of the run go to places 4h .. 4h+3, keys 8h+4 .. 8h+7 to 8+4h .. 8+4h+3
+            unsigned char* dst = lds + stage * kStage + kBytesK + 2 * (d * VS + 16 * run + 4 * h);
+            *reinterpret_cast<uint2*>(dst) = uint2{v.x, v.y};
+            *reinterpret_cast<uint2*>(dst + 16) = uint2{v.z, v.w};
+          }
+        }
+    };
+    fetch_all();
+    stash_all(0);
+    if (1 < n) fetch_all();
+    lds_barrier();
+    int stage = 1;
+    for (int t = 0; t < 2 * n + 2; ++t) {
+      const int x = t / 2 + 1;
+      if ((t & 1) == 0 && x < n) {
+        stash_all(stage);
+        stage = stage == NS - 1 ? 0 : stage + 1;
+        if (x + 1 < n) fetch_all();
+      }
+      lds_barrier();
+    }
+    return;
+  }
 
   // Where this wave's pieces come from and go to, fixed for the whole kernel. Block j of
   // a run is K (rows of 16 keys as stored) or V^T (HD rows of 16 keys); the addresses of
@@ -693,14 +759,15 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   // of the two is on the matrix cores and the other on the vector ALU.
   //   chunk x (counted from `first`) is read in half-steps 2x .. 2x+3, lies in stage x % 3,
   //   and is written in half-steps 2x-2 (second waves) and 2x-1 (first waves).
-  const int n = last - first + 1;
   const int off = NW == 8 ? wave >> 2 : 0;
   uint4 regs[PER];
-  lookup();
-  fetch(regs);
-  stash(0, regs);
   int held = 1, held_stage = 1;  // the chunk whose pieces `regs` holds, and its stage
-  if (held < n) fetch(regs);
+  if (!LOADER) {
+    lookup();
+    fetch(regs);
+    stash(0, regs);
+    if (held < n) fetch(regs);
+  }
   // The query operands have arrived before the loop starts. Without this the compiler,
   // which cannot tell the first round from the others, waits for all loads in flight
   // (the next chunk's among them) before the first product of every round.
@@ -797,6 +864,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   };
   // This wave's share of the loads: the held chunk into its stage, the next one into registers.
   auto load_work = [&]() {
+    if (LOADER) return;
     if (held < n) stash(held_stage, regs);
     ++held;
     held_stage = held_stage == NS - 1 ? 0 : held_stage + 1;
@@ -919,7 +987,7 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
   // 64 keys; forms 2 and 3: 16x16 tiles, chunks of 32 keys (four waves; eight for larger
   // groups), kept for comparison.
   const bool staged = hd <= 128 && form != 0;
-  const bool tile32 = staged && form == 1;
+  const bool tile32 = staged && (form == 1 || form == 5);  // form 5: as 1, never with a loading wave
   const int nw = staged ? (n_rep > 4 && form != 2 ? 8 : 4) : 4;
   const int hgroups = (n_rep + nw - 1) / nw;
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
@@ -929,12 +997,20 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
     if constexpr (HD <= 128) {
+      // a wave to spare in every block (one group of fewer heads than waves): it loads for the others
+      const bool loader = n_rep < nw && form != 5;
       if (tile32 && nw == 8) {
-        hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
+        if (loader)
+          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8, true>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
+        else
+          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8, false>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
         return;
       }
       if (tile32) {
-        hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
+        if (loader)
+          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, true>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
+        else
+          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, false>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
         return;
       }
       if (staged && nw == 8) {

@@ -266,7 +266,7 @@ def test_attn_decode_mfma(nq, nkv, hd, page, window, nsplits):
     assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("form", [0, 1, 2])
+@pytest.mark.parametrize("form", [0, 1, 2, 5])
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 50])
 def test_attn_prefill_mfma(nq, nkv, hd, page, window, form):
