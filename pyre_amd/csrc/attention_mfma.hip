@@ -39,6 +39,11 @@ constexpr int kChunk = 32;  // keys per iteration: two MFMA row tiles
 __device__ inline bf16x8 load_b128(const bf16* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
+// The same for data that is read once: it is not to displace other lines from the caches.
+__device__ inline bf16x8 load_b128_stream(const bf16* p) {
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  return __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+}
 __device__ inline bf16x8 zero_b128() {
   uint4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, z);
@@ -70,7 +75,12 @@ struct Bounds {
 //   tile_ok[t]    false for a tile whose page is not there: all its keys are hidden
 // `edge` says that some key of the chunk may be hidden from some column;
 // interior chunks skip all masking.
-template <int HD, int CT, typename LoadK, typename LoadV>
+// RUNS8 deals the keys to the tiles differently, so that a lane's eight values of P^T
+// belong to eight consecutive keys and V^T comes in 16-byte loads: row 4 g + j of tile t
+// is key key0 + 8 g + 4 t + j; load_k(t, c) gives lane (r, g) the row of key
+// key0 + 8 (r / 4) + 4 t + r % 4, load_v(dt) the keys 8 g .. 8 g + 7 in its slots, and
+// tile_ok[h] stands for the chunk's keys 16 h .. 16 h + 15.
+template <int HD, int CT, bool RUNS8 = false, typename LoadK, typename LoadV>
 __device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2], const Bounds<CT>& bd,
                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT],
@@ -82,7 +92,7 @@ __device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2]
   for (int t = 0; t < 2; ++t) {
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) s[t][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (!tile_ok[t]) continue;
+    if (!RUNS8 && !tile_ok[t]) continue;
 #pragma unroll
     for (int c = 0; c < HD / 32; ++c) {
       const bf16x8 a = load_k(t, c);
@@ -105,8 +115,8 @@ __device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2]
       for (int j = 0; j < 4; ++j) {
         float v = s[t][ct][j] * scale_log2;
         if (edge) {
-          const int key = key0 + 16 * t + 4 * g + j;
-          if (!tile_ok[t] || key < bd.lo[ct] || key > bd.hi[ct]) v = -INFINITY;
+          const int key = key0 + (RUNS8 ? 8 * g + 4 * t + j : 16 * t + 4 * g + j);
+          if (!tile_ok[RUNS8 ? g >> 1 : t] || key < bd.lo[ct] || key > bd.hi[ct]) v = -INFINITY;
         }
         x[4 * t + j] = v;
         mx = fmaxf(mx, v);
@@ -181,31 +191,67 @@ __device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bou
 }
 
 // A chunk's operands held in registers, so that the loads of the next chunk can be
-// in flight while the current one is multiplied.
+// in flight while the current one is multiplied. Keys are dealt as attend_core's RUNS8
+// says: a lane's part of V^T is one 16-byte run of eight keys.
 template <int HD>
 struct ChunkRegs {
   bf16x8 k[2][HD / 32];
-  uint2 v[HD / 16][2];
-  bool ok[2];
+  bf16x8 v[HD / 16];
+  bool ok[2];  // the pages of the chunk's keys 0..15 and 16..31 are there
 };
 
-template <int HD>
-__device__ inline void load_chunk(const KV& kv, int key0, ChunkRegs<HD>& cr) {
+// 64 consecutive entries of a request's block table, one in each lane of a wave: a
+// chunk's pages then come out of a register, not out of a load that the chunk's own
+// loads would have to wait for. Entries are asked for in rising order.
+struct TableWindow {
+  const int* table;
+  int width;  // entries of the request's row
+  int first;  // the entry that lane 0 holds
+  int held;
+  __device__ void fill(int entry) {
+    first = entry;
+    const int i = entry + static_cast<int>(threadIdx.x & 63);
+    held = i < width ? table[i] : -1;
+  }
+  // `entry` is the same in all lanes.
+  __device__ int page(int entry) {
+    if (entry - first >= 64) fill(entry);
+    return __builtin_amdgcn_readlane(held, entry - first);
+  }
+};
+
+template <int HD, bool STREAM_V>
+__device__ inline void load_chunk(const KV& kv, TableWindow& tw, int key0, ChunkRegs<HD>& cr) {
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  size_t base[2];  // (page, key/value head) of each half, in units of page_size * HD elements
+  int off[2];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int k0 = key0 + 16 * t;
-    const int page = kv.table[k0 / kv.page_size], off = k0 % kv.page_size;
-    cr.ok[t] = page >= 0;
-    const size_t base = static_cast<size_t>(cr.ok[t] ? page : 0) * kv.nkv + kv.kvh;
-    const bf16* kp = kv.k + (base * kv.page_size + off + r) * HD + 8 * g;
-    const bf16* vp = kv.v + (base * HD + r) * kv.page_size + off + 4 * g;
+  for (int h = 0; h < 2; ++h) {
+    const int k0 = key0 + 16 * h;
+    const int entry = k0 / kv.page_size;
+    const int page = tw.page(entry);
+    off[h] = k0 - entry * kv.page_size;
+    cr.ok[h] = page >= 0;
+    base[h] = static_cast<size_t>(cr.ok[h] ? page : 0) * kv.nkv + kv.kvh;
+  }
+  // K: rows 0..7 of a tile are keys of the first half, rows 8..15 of the second.
+  const int kh = r >> 3;
+  const bool k_ok = kh ? cr.ok[1] : cr.ok[0];
+  const bf16* kp = kv.k + ((kh ? base[1] : base[0]) * kv.page_size + (kh ? off[1] : off[0]) + 8 * ((r >> 2) & 1) + (r & 3)) * HD + 8 * g;
 #pragma unroll
-    for (int c = 0; c < HD / 32; ++c) cr.k[t][c] = cr.ok[t] ? load_b128(kp + 32 * c) : zero_b128();
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt)
-      cr.v[dt][t] = cr.ok[t] ? *reinterpret_cast<const uint2*>(vp + static_cast<size_t>(dt) * 16 * kv.page_size)
-                             : uint2{0u, 0u};
+    for (int c = 0; c < HD / 32; ++c) cr.k[t][c] = k_ok ? load_b128(kp + 4 * t * HD + 32 * c) : zero_b128();
+  // V^T: lanes g = 0, 1 take keys of the first half, g = 2, 3 of the second.
+  const int vh = g >> 1;
+  const bool v_ok = vh ? cr.ok[1] : cr.ok[0];
+  const bf16* vp = kv.v + ((vh ? base[1] : base[0]) * HD + r) * kv.page_size + (vh ? off[1] : off[0]) + 8 * (g & 1);
+  // STREAM_V (pages of at most 32 keys): the 16 rows of a load are whole cache lines, and
+  // these lines, read once, go past the caches. Halves of lines would come from memory twice.
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) {
+    const bf16* p = vp + static_cast<size_t>(dt) * 16 * kv.page_size;
+    cr.v[dt] = !v_ok ? zero_b128() : STREAM_V ? load_b128_stream(p) : load_b128(p);
   }
 }
 
@@ -214,12 +260,9 @@ __device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge,
                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
   const bool ok[2] = {cr.ok[0], cr.ok[1]};
-  attend_core<HD, CT>(
+  attend_core<HD, CT, true>(
       key0, edge, ok, bd, scale_log2, q, o, m, l, [&](int t, int c) { return cr.k[t][c]; },
-      [&](int dt) {
-        const uint4 u = {cr.v[dt][0].x, cr.v[dt][0].y, cr.v[dt][1].x, cr.v[dt][1].y};
-        return __builtin_bit_cast(bf16x8, u);
-      });
+      [&](int dt) { return cr.v[dt]; });
 }
 
 // ---------------------------------------------------------------------------
@@ -228,14 +271,15 @@ __device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge,
 // ONE_BLOCK: at most four splits, the four waves of a single block: they join their
 // partial results through LDS and store the finished rows in `out`; the partial buffers
 // and the second kernel are not needed.
-template <int HD, bool ONE_BLOCK>
+template <int HD, bool ONE_BLOCK, bool STREAM_V>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int* __restrict__ tokens, const int* __restrict__ positions,
     const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
     float* __restrict__ part_acc, float* __restrict__ part_ml, bf16* __restrict__ out, int nq, int nkv,
     int page_size, float scale_log2, int window, int nsplits) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int split = blockIdx.x * 4 + wave;
   if (!ONE_BLOCK && split >= nsplits) return;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
@@ -264,12 +308,17 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   if constexpr (HD <= 128) {
     // Two register sets: while one chunk is multiplied the next one's loads are in flight.
     ChunkRegs<HD> ra, rb;
-    if (begin < end) load_chunk<HD>(kv, begin * kChunk, ra);
+    // No entry beyond those of the chunks up to `last` is read.
+    TableWindow tw{kv.table, min(table_stride, (last * kChunk + 16) / page_size + 1), 0, -1};
+    if (begin < end) {
+      tw.fill(begin * kChunk / page_size);
+      load_chunk<HD, STREAM_V>(kv, tw, begin * kChunk, ra);
+    }
     for (int c = begin; c < end; c += 2) {
-      if (c + 1 < end) load_chunk<HD>(kv, (c + 1) * kChunk, rb);
+      if (c + 1 < end) load_chunk<HD, STREAM_V>(kv, tw, (c + 1) * kChunk, rb);
       attend_regs<HD, 1>(ra, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
       if (c + 1 < end) {
-        if (c + 2 < end) load_chunk<HD>(kv, (c + 2) * kChunk, ra);
+        if (c + 2 < end) load_chunk<HD, STREAM_V>(kv, tw, (c + 2) * kChunk, ra);
         attend_regs<HD, 1>(rb, (c + 1) * kChunk, c + 1 == first || c + 1 == last, bd, scale_log2, qr, o, m, l);
       }
     }
@@ -947,17 +996,21 @@ extern "C" int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cac
   const float scale_log2 = scale * kLog2e;
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
+    auto launch = [&](auto one_block, auto stream_v) {
+      hipLaunchKernelGGL((attn_decode_kernel<HD, decltype(one_block)::value, decltype(stream_v)::value>), grid,
+                         dim3(256), 0, stream, static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),
+                         static_cast<const bf16*>(v_cache), tokens, positions, seq_of_token, block_table,
+                         table_stride, part_acc, part_ml, static_cast<bf16*>(out), nq, nkv, page_size,
+                         scale_log2, window, nsplits);
+    };
+    const bool stream_v = page_size <= 32;
     if (nsplits <= 4) {  // one block per (token, key/value head): its waves join their results themselves
-      hipLaunchKernelGGL((attn_decode_kernel<HD, true>), grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
-                         static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), tokens,
-                         positions, seq_of_token, block_table, table_stride, part_acc, part_ml,
-                         static_cast<bf16*>(out), nq, nkv, page_size, scale_log2, window, nsplits);
+      if (stream_v) launch(std::true_type{}, std::true_type{});
+      else launch(std::true_type{}, std::false_type{});
       return;
     }
-    hipLaunchKernelGGL((attn_decode_kernel<HD, false>), grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
-                       static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), tokens,
-                       positions, seq_of_token, block_table, table_stride, part_acc, part_ml,
-                       static_cast<bf16*>(out), nq, nkv, page_size, scale_log2, window, nsplits);
+    if (stream_v) launch(std::false_type{}, std::true_type{});
+    else launch(std::false_type{}, std::false_type{});
     hipLaunchKernelGGL(attn_decode_reduce<HD>, dim3(n_tokens, nq), dim3(128), 0, stream,
                        part_acc, part_ml, tokens, static_cast<bf16*>(out), nq, nsplits);
   });
