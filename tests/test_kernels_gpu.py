@@ -108,6 +108,21 @@ def test_silu_mul(dtype):
     assert torch.allclose(out.double(), want, atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("n,inter", [(129, 24), (300, 1544), (130, 20)])
+def test_silu_mul_of_a_prompt_portion(n, inter):
+    """bfloat16 in and out, one partial, many rows: the kernel with eight features per
+    thread where the width allows it (24, 1544), the ordinary one where it does not (20)."""
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+
+    gu = rnd(1, n, 2 * inter, seed=6, scale=3.0).to(torch.bfloat16)
+    out = torch.full((n, inter), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops.silu_mul(Partials(gu), out, n)
+    s = gu[0].double()
+    want = torch.nn.functional.silu(s[:, :inter]) * s[:, inter:]
+    assert torch.allclose(out.double(), want, atol=2e-2, rtol=2e-2)
+
+
 # ----------------------------------------------------------------------------- rotary + cache write
 
 def rope_plain(x, pos, theta, rot):
