@@ -1,18 +1,23 @@
 // bfloat16 attention over the paged cache on the matrix cores (MFMA 16x16x32),
 // for head sizes that are multiples of 32 up to 256 and page sizes that are
-// multiples of 16. Two kernels share one inner loop:
+// multiples of 16. Two kernels share one inner loop on 16x16x32 tiles:
 //
 //   attn_decode_kernel   one new token per request; the keys of a request are
-//                        split over many waves, each writing a partial
-//                        (max, sum, unnormalised output) that attn_decode_reduce
-//                        merges. One wave serves up to 16 query heads that share
-//                        a key/value head, so K and V are read once per group.
+//                        split over many waves, each with a partial result
+//                        (max, sum, unnormalised output); the four waves of a
+//                        block merge theirs if they are all, else
+//                        attn_decode_reduce does. One wave serves up to 16 query
+//                        heads that share a key/value head, so K and V are read
+//                        once per group.
 //   attn_prefill_kernel  portions of prompts: a wave takes 32 consecutive tokens
 //                        of one request and one query head; the four waves of a
 //                        block take four heads of one key/value head, so their
 //                        K/V reads hit the same cache lines.
 //
-// Both compute the transposed problem so that no operand needs a transpose:
+// and attn_prefill_tile32_kernel, for heads of up to 128 elements, takes prompt
+// portions on 32x32x16 tiles with K and V staged through LDS (see there).
+//
+// All compute the transposed problem so that no operand needs a transpose:
 //   S^T[key, col]  = K[key, :] . Q[col, :]          A = K rows (cache, as stored)
 //   O^T[d, col]   += V^T[d, key] P^T[key, col]      A = V^T rows (cache stores V
 //                                                       transposed), B = P^T, which
@@ -474,129 +479,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Prefill with K and V staged through LDS: the NW waves of a block take NW query
-// heads of one key/value head over the same 32 tokens, so each chunk of keys is
-// read from memory once per block, double-buffered: the next chunk's loads are in
-// flight while the current one is multiplied.
-//   ks[stage][key][HD + 8]     rows padded so that 16 rows fall on different banks
-//   vs[stage][d][32 + 8]       V^T: 32 keys of the chunk per output element
-// ---------------------------------------------------------------------------
-template <int HD, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_prefill_lds_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-    bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
-    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
-    int nq, int nkv, int page_size, float scale_log2, int window) {
-  constexpr int CT = 2, KS = HD + 8, VS = kChunk + 8, T = NW * 64;
-  constexpr int NPK = kChunk * HD / 8, NP = 2 * NPK;   // 16-byte pieces of K and of V per chunk
-  constexpr int PER = (NP + T - 1) / T;
-  __shared__ __attribute__((aligned(16))) bf16 ks[2][kChunk][KS];
-  __shared__ __attribute__((aligned(16))) bf16 vs[2][HD][VS];
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
-  const int n_rep = nq / nkv, hgroups = (n_rep + NW - 1) / NW;
-  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
-  const int hin = hg * NW + wave;
-  const bool active = hin < n_rep;           // a wave without a head still helps loading
-  const int head = kvh * n_rep + (active ? hin : 0);
-  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
-  const int pos0 = positions[t0];
-  const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
-
-  Bounds<CT> bd;
-  bf16x8 qr[CT][HD / 32];
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    const int col = 16 * ct + r;
-    const bool live = active && col < ntok;
-    bd.hi[ct] = col < ntok ? pos0 + col : pos0;
-    bd.lo[ct] = window > 0 ? max(0, bd.hi[ct] - window + 1) : 0;
-#pragma unroll
-    for (int c = 0; c < HD / 32; ++c)
-      qr[ct][c] = live ? load_b128(q + (static_cast<size_t>(t0 + col) * nq + head) * HD + 32 * c + 8 * g) : zero_b128();
-  }
-  f32x4 o[HD / 16][CT];
-#pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt)
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) o[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m[CT], l[CT];
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) { m[ct] = -INFINITY; l[ct] = 0.f; }
-
-  const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int hi_all = pos0 + ntok - 1;
-  const int first = lo_all / kChunk, last = hi_all / kChunk;
-  const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
-
-  // Piece p < NPK: K[key p / (HD/8)][8 (p % (HD/8)) ..]; else V^T[d][8 part ..] with
-  // d = (p - NPK) / 4, part = (p - NPK) % 4 (eight keys, always within one page).
-  auto fetch = [&](int key0, uint4 (&regs)[PER]) {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = tid + i * T;
-      regs[i] = uint4{0u, 0u, 0u, 0u};
-      if (p >= NP) continue;
-      const bool is_k = p < NPK;
-      const int key = is_k ? key0 + p / (HD / 8) : key0 + 8 * ((p - NPK) % 4);
-      const int page = table[key / page_size], slot = key % page_size;
-      if (page < 0) continue;
-      const size_t base = static_cast<size_t>(page) * nkv + kvh;
-      const bf16* src = is_k ? k_cache + (base * page_size + slot) * HD + 8 * (p % (HD / 8))
-                             : v_cache + (base * HD + (p - NPK) / 4) * page_size + slot;
-      regs[i] = *reinterpret_cast<const uint4*>(src);
-    }
-  };
-  auto stash = [&](int stage, const uint4 (&regs)[PER]) {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = tid + i * T;
-      if (p >= NP) continue;
-      if (p < NPK) *reinterpret_cast<uint4*>(&ks[stage][p / (HD / 8)][8 * (p % (HD / 8))]) = regs[i];
-      else *reinterpret_cast<uint4*>(&vs[stage][(p - NPK) / 4][8 * ((p - NPK) % 4)]) = regs[i];
-    }
-  };
-
-  uint4 regs[PER];
-  fetch(first * kChunk, regs);
-  stash(0, regs);
-  for (int c = first; c <= last; ++c) {
-    const int st = (c - first) & 1;
-    __syncthreads();  // chunk c is in stage st; nobody reads stage st ^ 1 any more
-    if (c < last) fetch((c + 1) * kChunk, regs);
-    const int key0 = c * kChunk;
-    if (active) {
-      const bool edge = key0 + kChunk - 1 > pos0 || key0 < lo_max;
-      const bool ok[2] = {true, true};  // a missing page holds zeros and its keys lie outside every column's bounds
-      attend_core<HD, CT>(
-          key0, edge, ok, bd, scale_log2, qr, o, m, l,
-          [&](int t, int cc) { return *reinterpret_cast<const bf16x8*>(&ks[st][16 * t + r][32 * cc + 8 * g]); },
-          [&](int dt) {
-            const uint2 lo = *reinterpret_cast<const uint2*>(&vs[st][16 * dt + r][4 * g]);
-            const uint2 hi = *reinterpret_cast<const uint2*>(&vs[st][16 * dt + r][16 + 4 * g]);
-            const uint4 u = {lo.x, lo.y, hi.x, hi.y};
-            return __builtin_bit_cast(bf16x8, u);
-          });
-    }
-    if (c < last) stash(st ^ 1, regs);
-  }
-
-  if (!active) return;
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    const int col = 16 * ct + r;
-    if (col >= ntok) continue;
-    const float inv = 1.f / l[ct];
-    bf16* dst = out + (static_cast<size_t>(t0 + col) * nq + head) * HD + 4 * g;
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) {
-      const f32x4 v = o[dt][ct];
-      *reinterpret_cast<uint2*>(dst + dt * 16) = uint2{pack2(v[0] * inv, v[1] * inv), pack2(v[2] * inv, v[3] * inv)};
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------
 // Prefill on 32x32x16 tiles: the NW waves of a block take NW query heads of one
 // key/value head over the same 32 tokens (one MFMA tile of columns per wave);
 // keys and values come through LDS in chunks of 64, three stages, loaded once
@@ -1035,13 +917,11 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
   const bf16* kp = static_cast<const bf16*>(k_cache);
   const bf16* vp = static_cast<const bf16*>(v_cache);
   bf16* op = static_cast<bf16*>(out);
-  // Up to 128 elements per head, K and V go through LDS (two stages of 64 keys fit);
-  // larger heads read the cache directly in every wave. form 1: 32x32 tiles, chunks of
-  // 64 keys; forms 2 and 3: 16x16 tiles, chunks of 32 keys (four waves; eight for larger
-  // groups), kept for comparison.
-  const bool staged = hd <= 128 && form != 0;
-  const bool tile32 = staged && (form == 1 || form == 5);  // form 5: as 1, never with a loading wave
-  const int nw = staged ? (n_rep > 4 && form != 2 ? 8 : 4) : 4;
+  // Up to 128 elements per head, K and V go through LDS in chunks of 64 keys for 32x32 MFMA
+  // tiles (form 1; form 5: the same, never with a loading wave); larger heads, and form 0,
+  // read the cache directly in every wave.
+  const bool tile32 = hd <= 128 && form != 0;
+  const int nw = tile32 && n_rep > 4 ? 8 : 4;
   const int hgroups = (n_rep + nw - 1) / nw;
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
   const dim3 grid(n_tiles, nkv * hgroups);
@@ -1064,14 +944,6 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
           hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, true>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
         else
           hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, false>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
-        return;
-      }
-      if (staged && nw == 8) {
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 8>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
-        return;
-      }
-      if (staged) {
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, 4>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
         return;
       }
     }

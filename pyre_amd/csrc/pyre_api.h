@@ -43,15 +43,13 @@ int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, cons
 // bfloat16 products with 1..64 rows (decode): 1 if the kernel takes the shape.
 int pyre_gemm_skinny_supports(int M, int N, int K, long ldx, long ldw);
 
-// out: float32 [ksplit][M][N] partial sums of X[M, K] W[N, K]^T. form 0: the waves
-// of a block split k, operands straight from memory; form 1: X staged through LDS;
-// form 2: W and X staged through LDS, whole cache lines per load.
+// out: float32 [ksplit][M][N] partial sums of X[M, K] W[N, K]^T over ksplit parts of k.
 int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N,
-                          int K, int ksplit, int form, hipStream_t stream);
+                          int K, int ksplit, hipStream_t stream);
 
 // W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
 int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
-                               int two_i, int K, int form, hipStream_t stream);
+                               int two_i, int K, hipStream_t stream);
 
 int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                       const void* v_cache, int cache_dt, const int* positions,
@@ -72,9 +70,9 @@ int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache, const v
 
 // Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
 // all tokens of a tile from one request at consecutive positions. Heads of up to 128
-// elements: form 1 stages K and V through LDS in chunks of 64 keys for 32x32 MFMA tiles,
-// forms 2 and 3 in chunks of 32 keys for 16x16 tiles (kept for comparison); form 0, and
-// every larger head, reads the cache directly in each wave.
+// elements: form 1 stages K and V through LDS in chunks of 64 keys for 32x32 MFMA tiles
+// (form 5: the same, never with a wave that only loads); form 0, and every larger head,
+// reads the cache directly in each wave.
 int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
                            const int* tiles, int n_tiles, const int* positions,
                            const int* seq_of_token, const int* block_table, int table_stride,

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class KernelError(RuntimeError):
@@ -34,8 +34,8 @@ _SIGNATURES = {
     "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
     "pyre_gemm_skinny_supports": [I, I, I, L, L],
-    "pyre_gemm_skinny_bf16": [P, L, P, L, P, I, I, I, I, I, P],
-    "pyre_gemm_skinny_silu_bf16": [P, L, P, L, P, I, I, I, I, P],
+    "pyre_gemm_skinny_bf16": [P, L, P, L, P, I, I, I, I, P],
+    "pyre_gemm_skinny_silu_bf16": [P, L, P, L, P, I, I, I, P],
     "pyre_sample": [P, L, P, P, P, I, I, P],
     "pyre_feed_tokens": [P, P, P, I, P],
 }

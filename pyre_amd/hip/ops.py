@@ -342,27 +342,17 @@ def _skinny_common(x, w, m):
         raise KernelError("gemm_skinny: rows must be contiguous")
 
 
-def skinny_form(m: int) -> int:
-    """Which form of the weight-streaming kernel to use for m rows. Form 2 (W and X
-    through LDS, whole cache lines per load) measured fastest for every m <= 64 on the
-    7B shapes; forms 0 (waves split k, operands straight from memory) and 1 (only X
-    through LDS) are kept as alternatives for comparison."""
-    return 2
-
-
-def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int,
-                     form: int | None = None) -> None:
+def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int) -> None:
     """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 64."""
     _skinny_common(x, w, m)
     n = w.shape[0]
     if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() < ksplit * m * n or not out.is_cuda:
         raise KernelError("gemm_skinny: out must be contiguous float32 [ksplit, m, N] on the GPU")
     call("pyre_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), m, n,
-         w.shape[1], ksplit, skinny_form(m) if form is None else form, _stream())
+         w.shape[1], ksplit, _stream())
 
 
-def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int,
-                          form: int | None = None) -> None:
+def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int) -> None:
     """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up]."""
     _skinny_common(x, w_gate_up, m)
     two_i = w_gate_up.shape[0]
@@ -370,7 +360,7 @@ def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.T
             or out.shape[1] * 2 != two_i or out.shape[0] < m):
         raise KernelError("gemm_skinny_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
     call("pyre_gemm_skinny_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
-         out.data_ptr(), m, two_i, w_gate_up.shape[1], skinny_form(m) if form is None else form, _stream())
+         out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
 
 
 def read_bandwidth(device: str = "cuda:0", gib: float = 2.0, blocks: int = 4096, repeats: int = 10) -> float:

@@ -16,26 +16,20 @@ from pyre_amd.hip.ops import Partials
 
 #: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the BLAS library
 SKINNY_MAX_ROWS = 64
-#: blocks a weight-streaming product is spread over at least, by form of the kernel
-SKINNY_TARGET_BLOCKS = {0: 6000, 1: 900, 2: 500}
-SKINNY_MAX_KSPLIT = {0: 12, 1: 12, 2: 8}
+#: blocks a weight-streaming product is spread over at least, and the most partial sums
+SKINNY_TARGET_BLOCKS = 500
+SKINNY_MAX_KSPLIT = 8
 #: up to this many rows the gate/up product and the SiLU-gate are one kernel
 FUSED_SILU_MAX_ROWS = 64
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
-    """Blocks per output tile, so that a product with few columns still fills the chip
-    (measured on the 7B shapes with weights that are not in cache: about 6,000
-    blocks of form 0, 900 of form 1 or 500 of form 2, and at most 12, 12 or 8 partial sums)."""
-    from pyre_amd.hip.ops import skinny_form
-
-    form = skinny_form(m)
+    """Blocks per set of output rows, so that a product with few columns still fills the
+    chip (measured on the 7B shapes with weights that are not in cache: about 500 blocks
+    and at most 8 partial sums). A block takes 64 rows of the weights, 128 of wide ones."""
     tiles = -(-n_out // 16)
-    if form == 0:
-        blocks = -(-tiles // 2) if tiles >= 4096 else tiles
-    else:
-        blocks = -(-tiles // (8 if tiles >= 2048 else 4))
-    return max(1, min(-(-SKINNY_TARGET_BLOCKS[form] // blocks), k // 512, SKINNY_MAX_KSPLIT[form]))
+    blocks = -(-tiles // (8 if tiles >= 2048 else 4))
+    return max(1, min(-(-SKINNY_TARGET_BLOCKS // blocks), k // 512, SKINNY_MAX_KSPLIT))
 
 
 #: products whose library result is kept in float32 instead of being rounded to 16 bits:
