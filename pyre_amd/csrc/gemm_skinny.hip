@@ -48,15 +48,77 @@ __device__ inline bf16x8 zero128() {
 }
 __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
+#ifndef SILU_RT
+#define SILU_RT 2
+#endif
 constexpr int kPad = 8;  // bf16 elements of padding per LDS row: rows land on different banks
 
+// What a wave does with its finished tiles. acc[t][mt]: lane (r, g) holds output rows
+// m = 16 mt + r, columns n0[t] + 4 g .. + 3.
 template <int RT, int MT, int EPI>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ X, size_t ldx,
-                                                                 const bf16* __restrict__ W, size_t ldw,
-                                                                 void* __restrict__ out, int M, int N, int K,
-                                                                 int kper) {
-  constexpr int R = 64 * RT;               // rows of W per block
-  constexpr int WP = R * (kRun / 8) / 256;  // 16-byte pieces of W per thread and run
+__device__ inline void store_tiles(const f32x4 (&acc)[RT][MT], const int (&n0)[RT], void* out, int ks, int M, int N) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  if (EPI == kPartials) {
+    float* o = static_cast<float*>(out) + static_cast<size_t>(ks) * M * N;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const int n = n0[t] + 4 * g;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = 16 * mt + r;
+        if (m >= M || n >= N) continue;
+        float* dst = o + static_cast<size_t>(m) * N + n;
+        if (n + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<f32x4*>(dst) = acc[t][mt];
+        } else {
+          for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = acc[t][mt][j];
+        }
+      }
+    }
+  } else {  // tiles 2 p and 2 p + 1: gate and up of the 16 features from n0[2 p]
+    bf16* o = static_cast<bf16*>(out);
+    const int half = N / 2;
+#pragma unroll
+    for (int p = 0; p < RT / 2; ++p) {
+      const int n = n0[2 * p] + 4 * g;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = 16 * mt + r;
+        if (m >= M || n >= half) continue;
+        float y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float gate = acc[2 * p][mt][j], up = acc[2 * p + 1][mt][j];
+          y[j] = gate / (1.f + __expf(-gate)) * up;
+        }
+        bf16* dst = o + static_cast<size_t>(m) * half + n;
+        if (n + 3 < half && (half & 3) == 0) {
+          *reinterpret_cast<uint2*>(dst) = uint2{pack2(y[0], y[1]), pack2(y[2], y[3])};
+        } else {
+          for (int j = 0; j < 4 && n + j < half; ++j) dst[j] = from_float<bf16>(y[j]);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 17 to 64 rows of X: a block of NWV waves owns 16 RT NWV rows of W (kSiluMul: gate rows,
+// then the up rows of the same features). Its threads load each run of 128 k with 16
+// consecutive threads on 256 contiguous bytes of one row; W and X go through LDS, X once
+// per block, and the waves, each on RT tiles, read their operands there. The next run's
+// loads are in flight while the current run is multiplied.
+// ---------------------------------------------------------------------------
+template <int RT, int MT, int EPI, int NWV>
+__global__ __launch_bounds__(64 * NWV) void gemm_skinny_kernel(const bf16* __restrict__ X, size_t ldx,
+                                                              const bf16* __restrict__ W, size_t ldw,
+                                                              void* __restrict__ out, int M, int N, int K,
+                                                              int kper) {
+  constexpr int NT = 64 * NWV;                    // threads
+  constexpr int R = 16 * RT * NWV;                // rows of W per block
+  constexpr int PR = kRun / 8;                    // 16-byte pieces of a row per run
+  constexpr int WP = R * PR / NT;                 // pieces of W per thread and run
+  constexpr int XP = (MT * 16 * PR + NT - 1) / NT;  // pieces of X per thread and run (the last may lie past the end)
   __shared__ __attribute__((aligned(16))) bf16 wl[R][kRun + kPad];
   __shared__ __attribute__((aligned(16))) bf16 xl[MT * 16][kRun + kPad];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
@@ -65,11 +127,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
   const int kbeg = ks * kper, kend = min(K, kbeg + kper);
   const int nruns = (kend - kbeg + kRun - 1) / kRun;
 
-  // Global row of LDS row `lr`, or -1 past the end.
+  // Global row of LDS row `lr`, or -1 past the end. kSiluMul: the block's gate rows, then
+  // the up rows of the same features.
   auto global_row = [&](int lr) {
     if (EPI == kSiluMul) {
-      const int f = blockIdx.x * 64 + (lr & 63);
-      return f < half ? (lr >> 6) * half + f : -1;
+      const int f = blockIdx.x * (R / 2) + lr % (R / 2);
+      return f < half ? (lr / (R / 2)) * half + f : -1;
     }
     const int n = blockIdx.x * R + lr;
     return n < N ? n : -1;
@@ -77,31 +140,31 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
   const bf16* wsrc[WP];
 #pragma unroll
   for (int i = 0; i < WP; ++i) {
-    const int p = tid + 256 * i, gr = global_row(p / (kRun / 8));
-    wsrc[i] = gr < 0 ? nullptr : W + static_cast<size_t>(gr) * ldw + 8 * (p % (kRun / 8));
+    const int p = tid + NT * i, gr = global_row(p / PR);
+    wsrc[i] = gr < 0 ? nullptr : W + static_cast<size_t>(gr) * ldw + 8 * (p % PR);
   }
-  auto fetch = [&](int kr, bf16x8 (&wr)[WP], bf16x8 (&xr)[MT]) {
+  auto fetch = [&](int kr, bf16x8 (&wr)[WP], bf16x8 (&xr)[XP]) {
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
-      const int k = kr + 8 * ((tid + 256 * i) % (kRun / 8));
+      const int k = kr + 8 * ((tid + NT * i) % PR);
       wr[i] = (wsrc[i] && k < kend) ? ld128_stream(wsrc[i] + kr) : zero128();
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int p = tid + 256 * i, xrow = p / (kRun / 8), k = kr + 8 * (p % (kRun / 8));
+    for (int i = 0; i < XP; ++i) {
+      const int p = tid + NT * i, xrow = p / PR, k = kr + 8 * (p % PR);
       xr[i] = (xrow < M && k < kend) ? ld128(X + static_cast<size_t>(xrow) * ldx + k) : zero128();
     }
   };
-  auto stash = [&](const bf16x8 (&wr)[WP], const bf16x8 (&xr)[MT]) {
+  auto stash = [&](const bf16x8 (&wr)[WP], const bf16x8 (&xr)[XP]) {
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
-      const int p = tid + 256 * i;
-      *reinterpret_cast<bf16x8*>(&wl[p / (kRun / 8)][8 * (p % (kRun / 8))]) = wr[i];
+      const int p = tid + NT * i;
+      *reinterpret_cast<bf16x8*>(&wl[p / PR][8 * (p % PR)]) = wr[i];
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int p = tid + 256 * i;
-      *reinterpret_cast<bf16x8*>(&xl[p / (kRun / 8)][8 * (p % (kRun / 8))]) = xr[i];
+    for (int i = 0; i < XP; ++i) {
+      const int p = tid + NT * i;
+      if (p < MT * 16 * PR) *reinterpret_cast<bf16x8*>(&xl[p / PR][8 * (p % PR)]) = xr[i];
     }
   };
 
@@ -113,9 +176,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
   // LDS rows of this wave's tiles.
   int lrow[RT];
 #pragma unroll
-  for (int t = 0; t < RT; ++t) lrow[t] = (EPI == kSiluMul ? t * 64 + wave * 16 : (wave * RT + t) * 16) + r;
+  for (int t = 0; t < RT; ++t) lrow[t] = (EPI == kSiluMul ? t * (R / 2) + wave * 16 : (wave * RT + t) * 16) + r;
 
-  bf16x8 wr[WP], xr[MT];
+  bf16x8 wr[WP], xr[XP];
   if (nruns > 0) fetch(kbeg, wr, xr);
   for (int c = 0; c < nruns; ++c) {
     stash(wr, xr);
@@ -137,51 +200,96 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
     __syncthreads();  // everyone is done with this run before the next one overwrites it
   }
 
-  if (EPI == kPartials) {
-    float* o = static_cast<float*>(out) + static_cast<size_t>(ks) * M * N;
+  int n0[RT];  // first output column (kSiluMul: feature) of each tile of this wave
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
-      const int n = blockIdx.x * R + (wave * RT + t) * 16 + 4 * g;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int m = 16 * mt + r;
-        if (m >= M || n >= N) continue;
-        float* dst = o + static_cast<size_t>(m) * N + n;
-        if (n + 3 < N && (N & 3) == 0) {
-          *reinterpret_cast<f32x4*>(dst) = acc[t][mt];
-        } else {
-          for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = acc[t][mt][j];
-        }
-      }
-    }
-  } else {
-    bf16* o = static_cast<bf16*>(out);
-    const int n = blockIdx.x * 64 + wave * 16 + 4 * g;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = 16 * mt + r;
-      if (m >= M || n >= half) continue;
-      float y[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float gate = acc[0][mt][j], up = acc[RT - 1][mt][j];
-        y[j] = gate / (1.f + __expf(-gate)) * up;
-      }
-      bf16* dst = o + static_cast<size_t>(m) * half + n;
-      if (n + 3 < half && (half & 3) == 0) {
-        *reinterpret_cast<uint2*>(dst) = uint2{pack2(y[0], y[1]), pack2(y[2], y[3])};
-      } else {
-        for (int j = 0; j < 4 && n + j < half; ++j) dst[j] = from_float<bf16>(y[j]);
-      }
-    }
-  }
+  for (int t = 0; t < RT; ++t)
+    n0[t] = EPI == kSiluMul ? blockIdx.x * (R / 2) + wave * 16 : blockIdx.x * R + (wave * RT + t) * 16;
+  store_tiles<RT, MT, EPI>(acc, n0, out, ks, M, N);
 }
 
+// ---------------------------------------------------------------------------
+// Up to 16 rows of X: one wave per block, on its own. It owns RT tiles of 16 rows of W
+// (kSiluMul: gate tile and up tile of 16 features, alternating), loads a run of them as it lies
+// in memory (16 lanes on the 256 bytes of a row, four rows per load, past the caches), sorts
+// it into MFMA operands through LDS of its own and takes X straight from cache in operand
+// layout. No wave waits for another: a run is late only by its own slowest load, and two
+// runs are in flight per wave. Many small blocks also spread evenly over the compute units.
+// ---------------------------------------------------------------------------
 template <int RT, int EPI>
+__global__ __launch_bounds__(64) void gemm_skinny_wave_kernel(const bf16* __restrict__ X, size_t ldx,
+                                                              const bf16* __restrict__ W, size_t ldw,
+                                                              void* __restrict__ out, int M, int N, int K,
+                                                              int kper) {
+  constexpr int U = kRun / 32;  // MFMA steps per run
+  __shared__ __attribute__((aligned(16))) bf16 wl[RT][16][kRun + kPad];
+  const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+  const int ks = blockIdx.y, half = N / 2;
+  const int kbeg = ks * kper, kend = min(K, kbeg + kper);
+  const int nruns = (kend - kbeg + kRun - 1) / kRun;
+
+  int n0[RT];
+  const bf16* wsrc[RT][4];  // this lane's piece of rows 4 i + g of tile t: 16 bytes at 16 r of a run
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    n0[t] = EPI == kSiluMul ? (blockIdx.x * (RT / 2) + t / 2) * 16 : (blockIdx.x * RT + t) * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0[t] + 4 * i + g;
+      const bool there = EPI == kSiluMul ? n < half : n < N;
+      const size_t row = EPI == kSiluMul ? static_cast<size_t>(t & 1) * half + n : n;
+      wsrc[t][i] = there ? W + row * ldw + 8 * r : nullptr;
+    }
+  }
+  const bf16* xsrc = r < M ? X + static_cast<size_t>(r) * ldx + 8 * g : nullptr;
+
+  auto fetch = [&](int kr, bf16x8 (&wr)[RT][4], bf16x8 (&xr)[U]) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        wr[t][i] = (wsrc[t][i] && kr + 8 * r < kend) ? ld128_stream(wsrc[t][i] + kr) : zero128();
+#pragma unroll
+    for (int u = 0; u < U; ++u) xr[u] = (xsrc && kr + 32 * u + 8 * g < kend) ? ld128(xsrc + kr + 32 * u) : zero128();
+  };
+  f32x4 acc[RT][1];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) acc[t][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // The wave's own LDS traffic is in order; the waits keep the compiler from moving
+  // accesses across them.
+  auto use = [&](const bf16x8 (&wr)[RT][4], const bf16x8 (&xr)[U]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(&wl[t][4 * i + g][8 * r]) = wr[t][i];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&wl[t][r][32 * u + 8 * g]);
+        acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xr[u], acc[t][0], 0, 0, 0);
+      }
+  };
+
+  bf16x8 wa[RT][4], xa[U], wb[RT][4], xb[U];
+  if (nruns > 0) fetch(kbeg, wa, xa);
+  for (int c = 0; c < nruns; c += 2) {
+    if (c + 1 < nruns) fetch(kbeg + (c + 1) * kRun, wb, xb);
+    use(wa, xa);
+    if (c + 1 < nruns) {
+      if (c + 2 < nruns) fetch(kbeg + (c + 2) * kRun, wa, xa);
+      use(wb, xb);
+    }
+  }
+  store_tiles<RT, 1, EPI>(acc, n0, out, ks, M, N);
+}
+
+template <int RT, int EPI, int NWV>
 int launch_skinny(int mt, dim3 grid, hipStream_t stream, const bf16* X, size_t ldx, const bf16* W, size_t ldw,
                   void* out, int M, int N, int K, int kper) {
-#define PYRE_LAUNCH_MT(MTV)                                                                                 \
-  hipLaunchKernelGGL((gemm_skinny_kernel<RT, MTV, EPI>), grid, dim3(256), 0, stream, X, ldx, W, ldw, \
+#define PYRE_LAUNCH_MT(MTV)                                                                                  \
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, MTV, EPI, NWV>), grid, dim3(64 * NWV), 0, stream, X, ldx, W, ldw, \
                      out, M, N, K, kper)
   switch (mt) {
     case 1: PYRE_LAUNCH_MT(1); return 0;
@@ -191,6 +299,23 @@ int launch_skinny(int mt, dim3 grid, hipStream_t stream, const bf16* X, size_t l
   }
 #undef PYRE_LAUNCH_MT
   return 1;
+}
+
+// Waves per block (each takes 16 features) for the SiLU-gate product over `tiles` tiles of 16
+// features. A block streams at the pace of its own dependent runs, so the product is as fast
+// as the compute unit with the most blocks: choose the block size that spreads the tiles most
+// evenly over the chip's units (a 7B gate/up product, 1,184 tiles: 5 waves give 237 blocks for
+// 256 units, 4 waves 296, of which 40 units would get two).
+int silu_waves(int tiles) {
+  constexpr int kUnits = 256;
+  int best = 4;
+  double best_eff = 0.0;
+  for (int w = 8; w >= 3; --w) {
+    const int blocks = (tiles + w - 1) / w, rounds = (blocks + kUnits - 1) / kUnits;
+    const double eff = static_cast<double>(tiles) / (static_cast<double>(w) * kUnits * rounds);
+    if (eff > best_eff + 1e-9) best = w, best_eff = eff;
+  }
+  return best;
 }
 
 int check_common(const char* who, int M, int N, int K, long ldx, long ldw) {
@@ -217,11 +342,16 @@ extern "C" int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, lon
   const int tiles = (N + 15) / 16;
   const int rt = tiles >= 2048 ? 2 : 1;  // wide products: 128 rows per block
   const int kper = ((K + ksplit - 1) / ksplit + kRun - 1) / kRun * kRun;
-  const dim3 grid((tiles + 4 * rt - 1) / (4 * rt), ksplit);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
-  const int rc = rt == 2 ? launch_skinny<2, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper)
-                         : launch_skinny<1, kPartials>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
+  if (mt == 1) {  // every wave on its own, on two tiles: X, which every wave reads, comes half as often
+    hipLaunchKernelGGL((gemm_skinny_wave_kernel<2, kPartials>), dim3((tiles + 1) / 2, ksplit), dim3(64), 0, stream,
+                       x, ldx, w, ldw, out, M, N, K, kper);
+    return check_launch("gemm_skinny_bf16");
+  }
+  const dim3 grid((tiles + 4 * rt - 1) / (4 * rt), ksplit);
+  const int rc = rt == 2 ? launch_skinny<2, kPartials, 4>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper)
+                         : launch_skinny<1, kPartials, 4>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
   PYRE_REQUIRE(rc == 0, "gemm_skinny_bf16: no kernel for %d rows", M);
   return check_launch("gemm_skinny_bf16");
 }
@@ -233,9 +363,21 @@ extern "C" int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W
   PYRE_REQUIRE(two_i % 2 == 0, "gemm_skinny_silu_bf16: gate and up rows must be equally many");
   const int mt = (M + 15) / 16;
   const int kper = (K + kRun - 1) / kRun * kRun;
-  const dim3 grid(((two_i / 2 + 15) / 16 + 3) / 4, 1);
-  const int rc = launch_skinny<2, kSiluMul>(mt, grid, stream, static_cast<const bf16*>(X), ldx,
-                                            static_cast<const bf16*>(W), ldw, out, M, two_i, K, kper);
+  const int tiles = (two_i / 2 + 15) / 16, waves = silu_waves(tiles);
+  const bf16* x = static_cast<const bf16*>(X);
+  const bf16* w = static_cast<const bf16*>(W);
+  if (mt == 1) {  // every wave on its own
+    hipLaunchKernelGGL((gemm_skinny_wave_kernel<SILU_RT, kSiluMul>), dim3((tiles + SILU_RT / 2 - 1) / (SILU_RT / 2), 1), dim3(64), 0, stream, x, ldx, w, ldw,
+                       out, M, two_i, K, kper);
+    return check_launch("gemm_skinny_silu_bf16");
+  }
+  const dim3 grid((tiles + waves - 1) / waves, 1);
+  int rc = 1;
+  switch (waves) {
+#define PYRE_CASE(NWV) case NWV: rc = launch_skinny<2, kSiluMul, NWV>(mt, grid, stream, x, ldx, w, ldw, out, M, two_i, K, kper); break
+    PYRE_CASE(3); PYRE_CASE(4); PYRE_CASE(5); PYRE_CASE(6); PYRE_CASE(7); PYRE_CASE(8);
+#undef PYRE_CASE
+  }
   PYRE_REQUIRE(rc == 0, "gemm_skinny_silu_bf16: no kernel for %d rows", M);
   return check_launch("gemm_skinny_silu_bf16");
 }

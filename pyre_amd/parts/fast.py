@@ -16,20 +16,37 @@ from pyre_amd.hip.ops import Partials
 
 #: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the BLAS library
 SKINNY_MAX_ROWS = 64
-#: blocks a weight-streaming product is spread over at least, and the most partial sums
-SKINNY_TARGET_BLOCKS = 500
-SKINNY_MAX_KSPLIT = 8
+#: the most partial sums of a weight-streaming product
+SKINNY_MAX_KSPLIT = 12
 #: up to this many rows the gate/up product and the SiLU-gate are one kernel
 FUSED_SILU_MAX_ROWS = 64
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
-    """Blocks per set of output rows, so that a product with few columns still fills the
-    chip (measured on the 7B shapes with weights that are not in cache: about 500 blocks
-    and at most 8 partial sums). A block takes 64 rows of the weights, 128 of wide ones."""
+    """Into how many parts of k to split a weight-streaming product. A block (64 rows of the
+    weights, 128 of wide ones) walks its part of k in dependent runs of 128, about 0.9 us
+    each, and the blocks of a compute unit share its time: the product takes as long as the
+    longest walk or as the unit with the most blocks needs for its bytes (6.5 TB/s over the
+    256 units, measured on the 7B shapes), whichever is more; every part costs its consumer
+    one more addend. The split with the least of that is chosen, at least four runs a part."""
+    units, run_us, bytes_per_us, part_us = 256, 0.9, 6.5e6, 0.1
     tiles = -(-n_out // 16)
-    blocks = -(-tiles // (8 if tiles >= 2048 else 4))
-    return max(1, min(-(-SKINNY_TARGET_BLOCKS // blocks), k // 512, SKINNY_MAX_KSPLIT))
+    row_blocks = -(-n_out // (128 if tiles >= 2048 else 64))
+    runs = -(-k // 128)
+    stream_us = 2.0 * n_out * k / bytes_per_us
+    best, best_cost = 1, None
+    for ks in range(1, SKINNY_MAX_KSPLIT + 1):
+        per = -(-runs // ks)
+        if ks > 1 and per < 4:
+            break
+        if -(-runs // per) != ks:
+            continue  # would leave parts empty
+        blocks = row_blocks * ks
+        busiest = -(-blocks // units)
+        cost = max(per * run_us, stream_us * busiest * units / blocks) + part_us * ks
+        if best_cost is None or cost < best_cost - 1e-9:
+            best, best_cost = ks, cost
+    return best
 
 
 #: products whose library result is kept in float32 instead of being rounded to 16 bits:
