@@ -6,17 +6,17 @@
 // read along k as they are stored: A = 16 rows of W, B = 16 rows of X, D = a
 // 16 (n) x 16 (m) tile with four consecutive n per lane (MFMA 16x16x32).
 //
-// A block owns 64 RT consecutive rows of W and walks its k range in runs of 128. Its
-// threads load a run with 16 consecutive threads on 256 contiguous bytes of one row, so
-// that the memory system sees whole cache lines, not the 64-byte pieces of the MFMA
-// operand layout; W and X go through LDS, and the four waves, each on RT tiles of 16
-// rows, read their operands there. The next run's loads are in flight while the current
-// run is multiplied. `ksplit` blocks may share rows (grid.y); each then writes a
-// partial sum that the consumer adds in the order 0..ksplit-1, so that the result does
-// not depend on which block finishes first.
+// Two kernels, both walking k in runs of 128 that are loaded as they lie in memory (16
+// lanes on 256 contiguous bytes of a row of W: whole cache lines, not the 64-byte pieces
+// of the MFMA operand layout, past the caches) and sorted into operands through LDS:
+// gemm_skinny_kernel, blocks of several waves that share X in LDS, and
+// gemm_skinny_wave_kernel, single waves on their own (the SiLU-gate product of up to 16
+// rows). `ksplit` blocks may share rows (grid.y); each then writes a partial sum that the
+// consumer adds in the order 0..ksplit-1, so that the result does not depend on which
+// block finishes first.
 //
-// Epilogues: kPartials stores float32 [ksplit][M][N]; kSiluMul (RT = 2: 64 gate rows
-// and the 64 up rows of the same features, ksplit = 1) stores bfloat16
+// Epilogues: kPartials stores float32 [ksplit][M][N]; kSiluMul (tiles 2 p and 2 p + 1 of a
+// wave: 16 gate rows and the up rows of the same features, ksplit = 1) stores bfloat16
 // silu(gate) * up, [M][N/2].
 #include <type_traits>
 
@@ -48,9 +48,6 @@ __device__ inline bf16x8 zero128() {
 }
 __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
-#ifndef SILU_RT
-#define SILU_RT 2
-#endif
 constexpr int kPad = 8;  // bf16 elements of padding per LDS row: rows land on different banks
 
 // What a wave does with its finished tiles. acc[t][mt]: lane (r, g) holds output rows
@@ -344,11 +341,6 @@ extern "C" int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, lon
   const int kper = ((K + ksplit - 1) / ksplit + kRun - 1) / kRun * kRun;
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
-  if (mt == 1) {  // every wave on its own, on two tiles: X, which every wave reads, comes half as often
-    hipLaunchKernelGGL((gemm_skinny_wave_kernel<2, kPartials>), dim3((tiles + 1) / 2, ksplit), dim3(64), 0, stream,
-                       x, ldx, w, ldw, out, M, N, K, kper);
-    return check_launch("gemm_skinny_bf16");
-  }
   const dim3 grid((tiles + 4 * rt - 1) / (4 * rt), ksplit);
   const int rc = rt == 2 ? launch_skinny<2, kPartials, 4>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper)
                          : launch_skinny<1, kPartials, 4>(mt, grid, stream, x, ldx, w, ldw, out, M, N, K, kper);
@@ -366,8 +358,8 @@ extern "C" int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W
   const int tiles = (two_i / 2 + 15) / 16, waves = silu_waves(tiles);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
-  if (mt == 1) {  // every wave on its own
-    hipLaunchKernelGGL((gemm_skinny_wave_kernel<SILU_RT, kSiluMul>), dim3((tiles + SILU_RT / 2 - 1) / (SILU_RT / 2), 1), dim3(64), 0, stream, x, ldx, w, ldw,
+  if (mt == 1) {  // every wave on its own: measured 45 us against 50 on the 7B gate/up product (the other products gain nothing)
+    hipLaunchKernelGGL((gemm_skinny_wave_kernel<2, kSiluMul>), dim3(tiles, 1), dim3(64), 0, stream, x, ldx, w, ldw,
                        out, M, two_i, K, kper);
     return check_launch("gemm_skinny_silu_bf16");
   }
