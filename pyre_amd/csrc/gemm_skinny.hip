@@ -298,19 +298,22 @@ int launch_skinny(int mt, dim3 grid, hipStream_t stream, const bf16* X, size_t l
   return 1;
 }
 
-// Waves per block (each takes 16 features) for the SiLU-gate product over `tiles` tiles of 16
-// features. A block streams at the pace of its own dependent runs, so the product is as fast
-// as the compute unit with the most blocks: choose the block size that spreads the tiles most
-// evenly over the chip's units (a 7B gate/up product, 1,184 tiles: 5 waves give 237 blocks for
-// 256 units, 4 waves 296, of which 40 units would get two).
+// Waves per block (each takes 16 features) for the SiLU-gate product of 17 to 64 rows over
+// `tiles` tiles of 16 features. Measured at 32 / 64 rows (us; 1 to 6 waves per block):
+//   1.5B gate/up,   560 tiles:  19.9/25.3  21.1/24.0   18.5/21.3   19.9/21.6   23.1/25.4   24.4/26.5
+//   7B gate/up,   1,184 tiles:  54.7/71.7  56.1/66.7   48.5/57.7   54.9/67.1   56.9/60.7   58.4/62.1
+//   32B gate/up,  1,728 tiles: 108.7/187  106.4/126   112.3/152    95.3/111   114.0/161   162.3/173
+// Small blocks wait for fewer loads per run and more of them share a compute unit, but each
+// stages X again. The fastest had about 1.6 blocks per compute unit (or, with fewer tiles
+// than that, three waves): that is the rule.
 int silu_waves(int tiles) {
-  constexpr int kUnits = 256;
-  int best = 4;
-  double best_eff = 0.0;
-  for (int w = 8; w >= 3; --w) {
-    const int blocks = (tiles + w - 1) / w, rounds = (blocks + kUnits - 1) / kUnits;
-    const double eff = static_cast<double>(tiles) / (static_cast<double>(w) * kUnits * rounds);
-    if (eff > best_eff + 1e-9) best = w, best_eff = eff;
+  constexpr double kUnits = 256.0, kBlocksPerUnit = 1.6;
+  int best = 3;
+  double best_dist = 1e30;
+  for (int w = 3; w <= 6; ++w) {
+    const int blocks = (tiles + w - 1) / w;
+    const double dist = blocks / kUnits > kBlocksPerUnit ? blocks / kUnits - kBlocksPerUnit : kBlocksPerUnit - blocks / kUnits;
+    if (dist < best_dist - 1e-9) best = w, best_dist = dist;
   }
   return best;
 }
@@ -367,7 +370,7 @@ extern "C" int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W
   int rc = 1;
   switch (waves) {
 #define PYRE_CASE(NWV) case NWV: rc = launch_skinny<2, kSiluMul, NWV>(mt, grid, stream, x, ldx, w, ldw, out, M, two_i, K, kper); break
-    PYRE_CASE(3); PYRE_CASE(4); PYRE_CASE(5); PYRE_CASE(6); PYRE_CASE(7); PYRE_CASE(8);
+    PYRE_CASE(3); PYRE_CASE(4); PYRE_CASE(5); PYRE_CASE(6);
 #undef PYRE_CASE
   }
   PYRE_REQUIRE(rc == 0, "gemm_skinny_silu_bf16: no kernel for %d rows", M);
