@@ -123,7 +123,10 @@ def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
     span = min(max_ctx, window + 32) if window > 0 else max_ctx
     pieces = max(1, -(-span // DECODE_MIN_KEYS_PER_SPLIT))
     items = n_tokens * nkv * -(-(nq // nkv) // 16)
-    return max(1, min(pieces, DECODE_MAX_SPLITS, target_waves // items))
+    splits = max(1, min(pieces, DECODE_MAX_SPLITS, target_waves // items))
+    # The four waves of a block are four splits: a number that leaves waves of the last block
+    # idle is rounded down (five splits would be two blocks and a second kernel to merge them).
+    return splits - splits % 4 if splits > 4 else splits
 
 
 def attention(mixer, ctx, q, o, cache) -> bool:
