@@ -22,9 +22,14 @@ class Workspace:
     def __init__(self, device: torch.device):
         self.device = device
         self._bufs: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+        self._views: dict[tuple[str, torch.dtype, tuple[int, ...]], torch.Tensor] = {}
         self.frozen = False  #: set while a HIP graph is captured or replayed: growing is an error
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         numel = max(1, math.prod(shape))
         key = (name, dtype)
         buf = self._bufs.get(key)
@@ -33,7 +38,12 @@ class Workspace:
                 raise RuntimeError(f"workspace buffer {name!r} would have to grow inside a captured step")
             buf = torch.empty(numel, device=self.device, dtype=dtype)
             self._bufs[key] = buf
-        return buf[:math.prod(shape)].view(shape)
+            for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[k]  # views of the buffer that this one replaces
+        view = buf[:math.prod(shape)].view(shape)
+        if len(self._views) < 4096:
+            self._views[(name, dtype, shape)] = view
+        return view
 
     def nbytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())

@@ -85,10 +85,10 @@ def linear(lin, ctx, x, n, out):
         return None
     if lin.role in rt.options.get("library_f32_roles", LIBRARY_F32_ROLES):
         buf = ctx.workspace.get(f"linear32.{lin.role}", (n, n_out), torch.float32)
-        torch.mm(x[:n], lin.weight.t(), out_dtype=torch.float32, out=buf)
+        torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out_dtype=torch.float32, out=buf)
     else:
         buf = ctx.workspace.get(f"linear16.{lin.role}", (n, n_out), torch.bfloat16)
-        torch.mm(x[:n], lin.weight.t(), out=buf)
+        torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out=buf)
     return Partials(buf.view(1, n, n_out), lin.bias)
 
 
