@@ -41,3 +41,26 @@ def test_decode_splits_stay_within_what_the_kernel_takes():
         assert 1 <= s <= DECODE_MAX_SPLITS
         span = min(ctx, window + 32) if window > 0 else ctx
         assert s == 1 or (s - 1) * DECODE_MIN_KEYS_PER_SPLIT < span  # no split without keys of its own
+
+
+def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():
+    import torch
+
+    from pyre_amd.engine.context import Workspace
+
+    ws = Workspace(torch.device("cpu"))
+    a = ws.get("x", (4, 8), torch.float32)
+    assert ws.get("x", (4, 8), torch.float32) is a                     # the cached view
+    b = ws.get("x", (2, 8), torch.float32)
+    assert b.data_ptr() == a.data_ptr() and b.shape == (2, 8)          # a smaller view of the same buffer
+    assert ws.get("x", (4, 8), torch.bfloat16).data_ptr() != a.data_ptr()  # another element type, another buffer
+    big = ws.get("x", (16, 8), torch.float32)                          # grows: the old views are forgotten
+    assert ws.get("x", (4, 8), torch.float32).data_ptr() == big.data_ptr()
+    ws.frozen = True
+    assert ws.get("x", (16, 8), torch.float32) is big
+    try:
+        ws.get("x", (32, 8), torch.float32)
+    except RuntimeError as e:
+        assert "grow" in str(e)
+    else:
+        raise AssertionError("a frozen workspace must not grow")
