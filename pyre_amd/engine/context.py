@@ -24,6 +24,10 @@ class Workspace:
         self._bufs: dict[tuple[str, torch.dtype], torch.Tensor] = {}
         self._views: dict[tuple[str, torch.dtype, tuple[int, ...]], torch.Tensor] = {}
         self.frozen = False  #: set while a HIP graph is captured or replayed: growing is an error
+        #: set once a step has been captured: a captured step keeps using the memory it was
+        #: captured with, so a buffer that grows afterwards leaves its old memory allocated
+        self.keep_replaced = False
+        self._replaced: list[torch.Tensor] = []
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         shape = tuple(shape)
@@ -36,6 +40,8 @@ class Workspace:
         if buf is None or buf.numel() < numel:
             if self.frozen:
                 raise RuntimeError(f"workspace buffer {name!r} would have to grow inside a captured step")
+            if buf is not None and self.keep_replaced:
+                self._replaced.append(buf)
             buf = torch.empty(numel, device=self.device, dtype=dtype)
             self._bufs[key] = buf
             for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
@@ -46,7 +52,7 @@ class Workspace:
         return view
 
     def nbytes(self) -> int:
-        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+        return sum(b.numel() * b.element_size() for b in [*self._bufs.values(), *self._replaced])
 
 
 @dataclass

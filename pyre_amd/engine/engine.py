@@ -272,6 +272,7 @@ class Engine:
                     logits = self._forward(ctx, caches)
             finally:
                 ws.frozen = False
+            ws.keep_replaced = True
             state = self._graphs[key] = (graph, logits)
         else:
             self._upload(padded, fed_ids)

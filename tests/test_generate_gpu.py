@@ -187,3 +187,29 @@ def test_running_one_step_ahead_changes_no_token(dtype, model_dirs):
     assert s1.lookahead and not s0.lookahead
     # the steps that ran ahead are fewer host round trips, not fewer engine steps
     assert eng.graph_replays > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_after_steps_were_captured(dtype, model_dirs):
+    """Decode steps are captured while every buffer is still small (a 3-token prompt); then a
+    prompt of 200 tokens in portions of 128 makes scratch buffers grow. The captured steps go
+    on using their memory: the first request's tokens are those of an engine without graphs."""
+    from pyre_amd.api import Scheduler
+
+    short, long_ = random_ids(777, 3, seed=5), random_ids(777, 200, seed=6)
+    outs = []
+    for graphs in (False, True):
+        eng = _load(model_dirs["tiny-c"], dtype, use_graphs=graphs, prefill_chunk=128)
+        s = Scheduler(eng, max_batch=4)
+        a = s.add_request(short, max_new_tokens=60, temperature=0.7, seed=3)
+        for _ in range(12):
+            s.step()
+        if graphs:
+            assert eng.graph_replays > 0
+        b = s.add_request(long_, max_new_tokens=20, temperature=0.7, seed=4)
+        # other tensors take what the allocator has to give between the steps
+        junk = [torch.full((1 << 16,), float("nan"), device="cuda:0") for _ in range(32)]
+        done = s.run()
+        del junk
+        outs.append((done[a], done[b]))
+    assert outs[0] == outs[1]

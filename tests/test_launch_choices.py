@@ -56,10 +56,15 @@ def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():
     assert ws.get("x", (4, 8), torch.bfloat16).data_ptr() != a.data_ptr()  # another element type, another buffer
     big = ws.get("x", (16, 8), torch.float32)                          # grows: the old views are forgotten
     assert ws.get("x", (4, 8), torch.float32).data_ptr() == big.data_ptr()
+    ws.keep_replaced = True                                            # as after a captured step
+    before = big.data_ptr()
+    bigger = ws.get("x", (64, 8), torch.float32)
+    assert any(t.data_ptr() == before for t in ws._replaced)           # the captured step's memory stays allocated
+    big = bigger
     ws.frozen = True
-    assert ws.get("x", (16, 8), torch.float32) is big
+    assert ws.get("x", (64, 8), torch.float32) is big
     try:
-        ws.get("x", (32, 8), torch.float32)
+        ws.get("x", (128, 8), torch.float32)
     except RuntimeError as e:
         assert "grow" in str(e)
     else:
