@@ -157,6 +157,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
 // for bfloat16 without partial sums (a prompt portion's gate/up product, read once).
 // ---------------------------------------------------------------------------
 __device__ inline float silu_gate(float g, float u) { return g / (1.f + expf(-g)) * u; }
+// For results that are rounded to bfloat16: the hardware's exponential and reciprocal (errors of a
+// few units in the last place of float32), as in the epilogue of the decode step's gate/up product.
+__device__ inline float silu_gate_fast(float g, float u) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u; }
 
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict__ gu, int n_partials,
@@ -189,8 +192,8 @@ __global__ __launch_bounds__(256) void silu_mul_stream_kernel(const bf16* __rest
   u32x4 y;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const float lo = silu_gate(__uint_as_float(g[j] << 16), __uint_as_float(u[j] << 16));
-    const float hi = silu_gate(__uint_as_float(g[j] & 0xffff0000u), __uint_as_float(u[j] & 0xffff0000u));
+    const float lo = silu_gate_fast(__uint_as_float(g[j] << 16), __uint_as_float(u[j] << 16));
+    const float hi = silu_gate_fast(__uint_as_float(g[j] & 0xffff0000u), __uint_as_float(u[j] & 0xffff0000u));
     y[j] = pack_bf16x2(lo, hi);
   }
   *reinterpret_cast<u32x4*>(out + n * inter + c) = y;
