@@ -83,6 +83,19 @@ int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const 
 int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,
                 hipStream_t stream);
 
+// pyre_argmax without a scratch argument and without any allocation. It has no counterpart in
+// the reference; it is for callers that cannot allocate device memory: code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc. The slices' partial results
+// go to an array that is part of the library's device image (128 KB on every GPU the library
+// runs on, until the process ends), so m is at most PYRE_ARGMAX_STATIC_MAX_ROWS; more rows are
+// refused with an error. The caller makes the GPU of `stream`, `logits` and `out` the current
+// device. Same kernels and same results as pyre_argmax. All calls on one GPU share that GPU's
+// array: calls that may overlap there (two streams, two threads) race; put them on one stream
+// or use pyre_argmax with scratch of their own.
+#define PYRE_ARGMAX_STATIC_MAX_ROWS 256
+int pyre_argmax_static(const float* logits, long row_stride, int* out, int m, int vocab,
+                       hipStream_t stream);
+
 // tokens[i] = ids[src[i]] where src[i] >= 0: a step's token that is the previous step's
 // sampled id, taken on the device so that the host need not wait for it.
 int pyre_feed_tokens(int* tokens, const int* src, const int* ids, int n, hipStream_t stream);

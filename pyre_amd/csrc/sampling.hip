@@ -1,10 +1,19 @@
 // Next-token choice on the device: argmax (pyre/scheduler.py:80,94) and
 // temperature sampling by the inverse of the cumulative distribution, all in fp32.
 // One block per row of logits. A row's result depends on that row alone.
+#include <mutex>
+
 #include "pyre_api.h"
 #include "pyre_common.h"
 
 using namespace pyre;
+
+// Scratch of pyre_argmax_static: the slices' best values (64 floats per row) followed by
+// their indices (64 ints per row) for up to PYRE_ARGMAX_STATIC_MAX_ROWS rows, 128 KB on
+// every GPU the library runs on, held until the process ends. In host code this name is a
+// stand-in for the symbol, not a device address: the address of a device's copy comes from
+// hipGetSymbolAddress (static_scratch_of below) and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[PYRE_ARGMAX_STATIC_MAX_ROWS * 128 * 4];
 
 namespace {
 
@@ -142,6 +151,53 @@ extern "C" int pyre_argmax(const float* logits, long row_stride, int* out, void*
                      static_cast<size_t>(row_stride), pv, pi, vocab);
   hipLaunchKernelGGL(argmax_final_kernel, dim3(m), dim3(kWave), 0, stream, pv, pi, out);
   return check_launch("argmax");
+}
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+void* g_static_scratch[kMaxDevices] = {};  // the address of `scratch` on each device, once asked for
+
+// The current device's copy of `scratch`. Every GPU holds its own copy of the array at its own
+// address, so the address is asked for once per device, with that device current.
+int static_scratch_of(int device, void** ptr) {
+  std::lock_guard<std::mutex> guard(g_static_mutex);
+  if (!g_static_scratch[device]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    PYRE_REQUIRE(e == hipSuccess && p, "argmax_static: hipGetSymbolAddress on device %d: %s", device,
+                 hipGetErrorString(e));
+    g_static_scratch[device] = p;
+  }
+  *ptr = g_static_scratch[device];
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int pyre_argmax_static(const float* logits, long row_stride, int* out, int m, int vocab,
+                                  hipStream_t stream) {
+  PYRE_REQUIRE(vocab > 0 && row_stride >= vocab, "argmax_static: bad sizes");
+  PYRE_REQUIRE(m <= PYRE_ARGMAX_STATIC_MAX_ROWS,
+               "argmax_static: %d rows; the built-in scratch holds %d (use pyre_argmax with scratch of your own)", m,
+               PYRE_ARGMAX_STATIC_MAX_ROWS);
+  if (m <= 0) return 0;
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  PYRE_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+  PYRE_REQUIRE(device >= 0 && device < kMaxDevices, "argmax_static: device %d is beyond the %d this entry point knows",
+               device, kMaxDevices);
+  void* base = nullptr;
+  if (int rc = static_scratch_of(device, &base)) return rc;
+  // Nothing has to start at zero: the first stage writes all 64 slices of every row before
+  // the second stage reads them, whatever an earlier (larger) call left behind.
+  float* pv = static_cast<float*>(base);
+  int* pi = reinterpret_cast<int*>(pv + static_cast<size_t>(m) * kSlices);
+  hipLaunchKernelGGL(argmax_slices_kernel, dim3(m, kSlices), dim3(kArgThreads), 0, stream, logits,
+                     static_cast<size_t>(row_stride), pv, pi, vocab);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(m), dim3(kWave), 0, stream, pv, pi, out);
+  return check_launch("argmax_static");
 }
 
 extern "C" int pyre_sample(const float* logits, long row_stride, const float* temperature,

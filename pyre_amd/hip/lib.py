@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class KernelError(RuntimeError):
@@ -33,6 +33,7 @@ _SIGNATURES = {
     "pyre_attn_decode_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
+    "pyre_argmax_static": [P, L, P, I, I, P],
     "pyre_gemm_skinny_supports": [I, I, I, L, L],
     "pyre_gemm_skinny_bf16": [P, L, P, L, P, I, I, I, I, P],
     "pyre_gemm_skinny_silu_bf16": [P, L, P, L, P, I, I, I, P],
@@ -51,10 +52,24 @@ def lib() -> ctypes.CDLL:
         handle.pyre_last_error.restype = ctypes.c_char_p
         handle.pyre_abi_version.restype = c_int
         if handle.pyre_abi_version() != ABI_VERSION:
-            # An older library from a previous checkout: rebuild once.
+            # An older library from a previous checkout: rebuild once. The loader keeps the
+            # mapping of a path it has already opened, so the new build is opened under a
+            # name of its own.
+            import os
+            import shutil
+
             path = _build.build(force=True)
-            handle = ctypes.CDLL(str(path))
+            fresh = path.with_name(f"{path.stem}.{os.getpid()}{path.suffix}")
+            shutil.copyfile(path, fresh)
+            try:
+                handle = ctypes.CDLL(str(fresh))
+            finally:
+                os.unlink(fresh)
             handle.pyre_last_error.restype = ctypes.c_char_p
+            handle.pyre_abi_version.restype = c_int
+            if handle.pyre_abi_version() != ABI_VERSION:
+                raise KernelError(f"kernel library has ABI {handle.pyre_abi_version()}, the binding expects "
+                                  f"{ABI_VERSION}: sources and binding are out of step")
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.argtypes = argtypes

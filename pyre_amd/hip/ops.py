@@ -258,6 +258,23 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor | None
          logits.shape[1], _stream())
 
 
+ARGMAX_STATIC_MAX_ROWS = 256  #: rows that the library's built-in scratch holds
+
+
+def argmax_static(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """:func:`argmax` for callers that must not allocate: the partial results go to an
+    array inside the library's device image (at most 256 rows; calls that overlap on one
+    GPU race)."""
+    _dev(logits, out)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("argmax: float32 [M, V] logits expected")
+    m = logits.shape[0]
+    _i32("out", out, m)
+    with torch.cuda.device(logits.device):
+        call("pyre_argmax_static", logits.data_ptr(), logits.stride(0), out.data_ptr(), m, logits.shape[1],
+             _stream())
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
            out: torch.Tensor) -> None:
     """Rows with temperature > 0 get a token drawn by inverse CDF with their
