@@ -1,13 +1,17 @@
 """The cache manager: page pools, block tables, state slots.
 
 Every entry of a model's layer order declares what it keeps
-(:class:`~pyre_amd.parts.base.KVCacheSpec`, :class:`~pyre_amd.parts.base.StateCacheSpec`
+(:class:`~pyre_amd.parts.base.PagedCacheSpec`, :class:`~pyre_amd.parts.base.StateCacheSpec`
 or nothing). Entries with the same needs form a *group*:
 
 * a **page group** has a pool of pages of its own and, for each request, a block
   table of its own. One page id addresses that page in every layer of the group
   (`pyre/paged_cache.py:96-109` lays the reference's single pool out the same way).
+  Which tensors a page holds, and how a page of each is laid out, is what the
+  description says (the mixer's choice); the manager allocates
+  ``[layers, pages, *page_shape]`` for each and knows nothing of their meaning.
   A group with a window gives a page back as soon as no later query can see it.
+  All groups share one page size.
 * a **state group** has one fixed-size state per (layer, slot).
 
 A request holds one *slot* from admission to its end; the slot indexes the state
@@ -18,6 +22,14 @@ and `tests/test_paged_cache.py:203-213` records the bug that came of it).
 
 This module is bookkeeping only and runs without a GPU; ``materialize`` allocates
 the pools' tensors.
+
+``fill(tensor, ids, value)`` sets ``tensor[:, id]`` to ``value`` for the listed pages or
+slots (the engine passes its fill kernel; without one torch does it). It zeroes a state
+slot when a request starts. Debugging aid: with ``poison=True`` every page and every state
+slot that goes back to a pool is filled with NaN at once, and the whole pool at the start,
+so that a read of memory which no live request owns shows in the results instead of hiding
+behind stale, finite data; a page is zeroed when a request takes it (slots of its own pages
+that it has not written yet are read, and weighted with 0, by kernels that load whole chunks).
 """
 
 from __future__ import annotations
@@ -27,7 +39,7 @@ from dataclasses import dataclass, field
 import numpy as np
 
 from pyre_amd.cache.allocator import OutOfPages, PageAllocator
-from pyre_amd.parts.base import KVCacheSpec, StateCacheSpec
+from pyre_amd.parts.base import PagedCacheSpec, StateCacheSpec
 
 RELEASED = -1  #: block-table entry of a page that a window has passed
 
@@ -35,13 +47,13 @@ RELEASED = -1  #: block-table entry of a page that a window has passed
 @dataclass
 class PageGroup:
     index: int
-    spec: KVCacheSpec
+    spec: PagedCacheSpec
     entries: list[int]               #: positions in the layer order, ascending
     page_size: int
     num_pages: int
     allocator: PageAllocator
-    k: object = None                 #: [len(entries), num_pages, nkv, page_size, hd]
-    v: object = None                 #: [len(entries), num_pages, nkv, hd, page_size]
+    #: name -> [len(entries), num_pages, *page_shape] for every tensor of the description
+    tensors: dict = field(default_factory=dict)
 
     def layer_index(self, entry: int) -> int:
         return self.entries.index(entry)
@@ -71,8 +83,10 @@ class _Request:
 
 class CacheManager:
     def __init__(self, cache_specs: list, page_size: int, num_pages: int, max_num_seqs: int,
-                 max_model_len: int):
+                 max_model_len: int, fill=None, poison: bool = False):
         """``cache_specs[i]`` is what entry i of the layer order keeps (or None)."""
+        self.fill = fill
+        self.poison = poison
         if page_size <= 0 or num_pages <= 0 or max_num_seqs <= 0:
             raise ValueError("page_size, num_pages and max_num_seqs must be positive")
         self.page_size = page_size
@@ -81,7 +95,7 @@ class CacheManager:
         self.max_pages_per_seq = -(-max_model_len // page_size)
         self.page_groups: list[PageGroup] = []
         self.state_groups: list[StateGroup] = []
-        #: entry -> ("kv" | "state", group index) for entries that keep something
+        #: entry -> ("paged" | "state", group index) for entries that keep something
         self.group_of_entry: dict[int, tuple[str, int]] = {}
         by_spec: dict[object, object] = {}
         for entry, spec in enumerate(cache_specs):
@@ -89,7 +103,7 @@ class CacheManager:
                 continue
             grp = by_spec.get(spec)
             if grp is None:
-                if isinstance(spec, KVCacheSpec):
+                if isinstance(spec, PagedCacheSpec):
                     grp = PageGroup(len(self.page_groups), spec, [], page_size, num_pages,
                                     PageAllocator(num_pages))
                     self.page_groups.append(grp)
@@ -100,29 +114,47 @@ class CacheManager:
                     raise TypeError(f"entry {entry}: unknown cache description {spec!r}")
                 by_spec[spec] = grp
             grp.entries.append(entry)
-            self.group_of_entry[entry] = ("kv" if isinstance(grp, PageGroup) else "state", grp.index)
+            self.group_of_entry[entry] = ("paged" if isinstance(grp, PageGroup) else "state", grp.index)
         self.slots = PageAllocator(max_num_seqs, what="slot")
         self._requests: dict[object, _Request] = {}
 
     # ------------------------------------------------------------------ tensors
 
     def materialize(self, device, dtype) -> None:
-        """Allocate the pools on ``device`` (keys and values in ``dtype``)."""
+        """Allocate the pools on ``device`` ("model" tensors in ``dtype``)."""
         import torch
 
         for g in self.page_groups:
-            s = g.spec
             n = len(g.entries)
-            g.k = torch.zeros((n, g.num_pages, s.num_kv_heads, g.page_size, s.head_dim), device=device, dtype=dtype)
-            g.v = torch.zeros((n, g.num_pages, s.num_kv_heads, s.head_dim, g.page_size), device=device, dtype=dtype)
+            for t in g.spec.tensors:
+                dt = torch.float32 if t.dtype == "float32" else dtype
+                g.tensors[t.name] = torch.zeros((n, g.num_pages, *t.page_shape(g.page_size)), device=device, dtype=dt)
+            self._poison_pages(g, range(g.num_pages))
         for g in self.state_groups:
             dt = torch.float32 if g.spec.dtype == "float32" else dtype
             # one slot more than requests: padding rows of a captured step write there
             g.tensor = torch.zeros((len(g.entries), self.max_num_seqs + 1, *g.spec.shape), device=device, dtype=dt)
+            if self.poison:
+                self._fill(g.tensor, list(range(self.max_num_seqs)), float("nan"))
+
+    def _fill(self, tensor, ids: list[int], value: float) -> None:
+        if tensor is None or not ids:
+            return
+        if self.fill is not None:
+            self.fill(tensor, ids, value)
+        else:
+            tensor[:, ids] = value
+
+    def _poison_pages(self, g: PageGroup, pages) -> None:
+        if not self.poison:
+            return
+        pages = list(pages)
+        for t in g.tensors.values():
+            self._fill(t, pages, float("nan"))
 
     def bytes_per_page(self, dtype_bytes: int) -> int:
-        return sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * g.page_size * dtype_bytes
-                   for g in self.page_groups)
+        return sum(len(g.entries) * t.elements_per_token() * g.page_size * (4 if t.dtype == "float32" else dtype_bytes)
+                   for g in self.page_groups for t in g.spec.tensors)
 
     # ------------------------------------------------------------------ requests
 
@@ -144,8 +176,7 @@ class CacheManager:
             slot, tables=[[] for _ in self.page_groups],
             arrays=[np.full(self.max_pages_per_seq, RELEASED, dtype=np.int32) for _ in self.page_groups])
         for g in self.state_groups:
-            if g.tensor is not None:
-                g.tensor[:, slot].zero_()
+            self._fill(g.tensor, [slot], 0.0)
         return slot
 
     def slot(self, rid) -> int:
@@ -188,6 +219,11 @@ class CacheManager:
                 have = len(table)
                 table.extend(g.allocator.allocate_many(add))
                 arr[have:have + add] = table[have:]
+                if self.poison:
+                    # What a request has not yet written of its own pages reads as zero: the
+                    # attention kernels load whole chunks and weight hidden keys with an exact 0.
+                    for t in g.tensors.values():
+                        self._fill(t, table[have:], 0.0)
         req.reserved = max(req.reserved, new_len)
 
     def slot_mapping(self, rid, group: int, start: int, n: int) -> list[int]:
@@ -224,19 +260,41 @@ class CacheManager:
             # The next query sits at position req.length and sees keys > length - w.
             dead_upto = req.length - w  # keys <= dead_upto are never read again
             last_dead_page = (dead_upto + 1) // self.page_size - 1
+            dead = []
             for i in range(min(last_dead_page + 1, len(table))):
                 if table[i] != RELEASED:
                     g.allocator.free(table[i])
+                    dead.append(table[i])
                     table[i] = RELEASED
                     arr[i] = RELEASED
+            self._poison_pages(g, dead)
 
     def free_request(self, rid) -> None:
         req = self._requests.pop(rid)
         for g, table in zip(self.page_groups, req.tables):
-            for page in reversed(table):
+            held = [page for page in table if page != RELEASED]
+            for page in reversed(held):
+                g.allocator.free(page)
+            self._poison_pages(g, held)
+        self.slots.free(req.slot)
+        if self.poison:
+            for g in self.state_groups:
+                self._fill(g.tensor, [req.slot], float("nan"))
+
+    def unreserve(self, rid) -> None:
+        """Give back the pages that were reserved beyond the request's committed length
+        (a step that was prepared and then not run)."""
+        req = self._requests[rid]
+        keep = -(-req.length // self.page_size)
+        for g, table, arr in zip(self.page_groups, req.tables, req.arrays):
+            extra = table[keep:]
+            for page in reversed(extra):
                 if page != RELEASED:
                     g.allocator.free(page)
-        self.slots.free(req.slot)
+            self._poison_pages(g, [p for p in extra if p != RELEASED])
+            del table[keep:]
+            arr[keep:] = RELEASED
+        req.reserved = req.length
 
     # ------------------------------------------------------------------ checks
 

@@ -30,6 +30,9 @@ class EngineConfig:
     #: row counts (tokens in a step) for which the BLAS library is asked, once at start-up,
     #: to time its kernels for this model's many-row 16-bit products and keep the fastest
     tune_gemm_rows: tuple = ()
+    #: debugging aid: fill every cache page and state slot with NaN when it goes back to its
+    #: pool (and all of them at the start), so that a read of freed memory shows in the logits
+    debug_poison: bool = False
 
     def __post_init__(self) -> None:
         if self.dtype not in DTYPE_NAMES:

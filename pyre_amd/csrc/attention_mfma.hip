@@ -572,7 +572,10 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
           const int idx = (is_k ? blk : blk - kHalfBlocks) * 64 + lane;
           const bf16* src = is_k ? k_cache + base + static_cast<size_t>(sl) * HD + 8 * idx
                                  : v_cache + base + static_cast<size_t>(idx >> 1) * page_size + sl + 8 * (idx & 1);
-          lr[run * BR + blk] = *reinterpret_cast<const u32x4*>(src);
+          // a page that is not there reads page 0, which may belong to anyone: its bytes are dropped
+          const unsigned keep = page < 0 ? 0u : ~0u;
+          const u32x4 got = *reinterpret_cast<const u32x4*>(src);
+          lr[run * BR + blk] = u32x4{got.x & keep, got.y & keep, got.z & keep, got.w & keep};
         }
         sl += 16;
         const bool wrap = sl >= page_size;
@@ -641,7 +644,9 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   // the next chunk to look up; both advance by whole runs, without a division per chunk.
   // The pages of a chunk are looked up one load ahead of the chunk's own loads, so that
   // the latency of the table is never waited for. A page that is not there (released, or
-  // past the request's end) reads page 0 instead: all its keys are out of every column's bounds.
+  // past the request's end) reads page 0 instead and is replaced by zeros: all its keys are
+  // out of every column's bounds, and a hidden key's value is weighted with an exact 0,
+  // which only a finite value survives.
   int pi = (first * kKeys) / page_size, sl = (first * kKeys) % page_size;
   int run_page[kKeys / 16], run_slot[kKeys / 16];
   auto lookup = [&]() {
@@ -659,17 +664,21 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   auto fetch = [&](uint4 (&regs)[PER]) {
     size_t base[kKeys / 16];
     int slot[kKeys / 16];
+    unsigned keep[kKeys / 16];
 #pragma unroll
     for (int run = 0; run < kKeys / 16; ++run) {
       base[run] = (static_cast<size_t>(max(run_page[run], 0)) * nkv + kvh) * page_elems;
       slot[run] = run_slot[run];
+      keep[run] = run_page[run] < 0 ? 0u : ~0u;  // page 0 stands in, and may belong to anyone: its bytes are dropped
     }
     lookup();  // for the chunk after this one
 #pragma unroll
     for (int run = 0; run < kKeys / 16; ++run)
 #pragma unroll
-      for (int j = 0; j < PB; ++j)
-        regs[run * PB + j] = *reinterpret_cast<const uint4*>(g_ptr[j] + base[run] + slot[run] * g_mul[j] + g_lane[j]);
+      for (int j = 0; j < PB; ++j) {
+        const uint4 got = *reinterpret_cast<const uint4*>(g_ptr[j] + base[run] + slot[run] * g_mul[j] + g_lane[j]);
+        regs[run * PB + j] = uint4{got.x & keep[run], got.y & keep[run], got.z & keep[run], got.w & keep[run]};
+      }
   };
   auto stash = [&](int stage, const uint4 (&regs)[PER]) {
 #pragma unroll

@@ -259,3 +259,47 @@ extern "C" int pyre_reduce_partials(const void* in, int in_dt, int n_partials, l
                      out_dt, total, width);
   return check_launch("reduce_partials");
 }
+
+// ---------------------------------------------------------------------------
+// Fill utility: sets whole rows of a [outer, rows, row_elems] tensor to one bit pattern.
+// It zeroes a request's state slot at admission and, in the debug mode that poisons freed
+// memory, writes NaN over pages and slots that went back to their pool. The row ids come
+// from the host by value, so no upload is needed.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr int kFillIds = 64;
+struct FillIds { int v[kFillIds]; };
+
+template <typename U>
+__global__ __launch_bounds__(256) void fill_rows_kernel(U* __restrict__ base, size_t outer_stride, size_t row_elems,
+                                                        FillIds ids, U pattern) {
+  U* row = base + blockIdx.z * outer_stride + static_cast<size_t>(ids.v[blockIdx.y]) * row_elems;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < row_elems;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x)
+    row[i] = pattern;
+}
+}  // namespace
+
+extern "C" int pyre_fill_rows(void* base, int elem_bytes, long outer_stride, int n_outer, int n_rows, long row_elems,
+                              const int* ids_host, int n_ids, unsigned pattern, hipStream_t stream) {
+  PYRE_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "fill_rows: elements of %d bytes", elem_bytes);
+  PYRE_REQUIRE(n_outer >= 1 && n_outer <= 65535 && row_elems >= 1 && outer_stride >= static_cast<long>(n_rows) * row_elems,
+               "fill_rows: bad sizes");
+  for (int i = 0; i < n_ids; ++i)
+    PYRE_REQUIRE(ids_host[i] >= 0 && ids_host[i] < n_rows, "fill_rows: row %d is outside 0..%d", ids_host[i], n_rows - 1);
+  const unsigned bx = static_cast<unsigned>(row_elems / 256 < 1 ? 1 : (row_elems / 256 > 64 ? 64 : row_elems / 256));
+  for (int done = 0; done < n_ids; done += kFillIds) {
+    FillIds ids;
+    const int now = n_ids - done < kFillIds ? n_ids - done : kFillIds;
+    for (int i = 0; i < kFillIds; ++i) ids.v[i] = ids_host[done + (i < now ? i : 0)];
+    const dim3 grid(bx, now, n_outer);
+    if (elem_bytes == 4)
+      hipLaunchKernelGGL(fill_rows_kernel<uint32_t>, grid, dim3(256), 0, stream, static_cast<uint32_t*>(base),
+                         static_cast<size_t>(outer_stride), static_cast<size_t>(row_elems), ids, pattern);
+    else
+      hipLaunchKernelGGL(fill_rows_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<uint16_t*>(base),
+                         static_cast<size_t>(outer_stride), static_cast<size_t>(row_elems), ids,
+                         static_cast<uint16_t>(pattern));
+  }
+  return check_launch("fill_rows");
+}

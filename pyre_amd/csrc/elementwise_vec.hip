@@ -43,7 +43,14 @@ constexpr int kNormMaxVec = 8;  // float4 per thread
 // THREADS = 256 keeps up to 8192 elements of a row in registers and suits many rows;
 // THREADS = 1024 gives a short row one float4 per thread, so that all loads of a
 // decode step's few rows are in flight at once.
-template <typename TD, typename TG, typename TO, int THREADS>
+//
+// The sum of squares is added up in an order that the row's width alone fixes, whichever
+// variant runs: a row wider than 1024 elements is summed as 1024 threads would (thread t
+// adds its pieces t, t + 1024, ... in ascending order; every 64 consecutive threads are
+// reduced by the butterfly of wave_sum; the 16 results are added in ascending order).
+// The 256-thread variant then plays VIRT = 4 of those threads per thread: t = thread +
+// 256 j. A position's result therefore does not depend on how many rows share the step.
+template <typename TD, typename TG, typename TO, int THREADS, int VIRT>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, int n_partials, size_t partial_stride,
     const TG* __restrict__ gain, TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
@@ -52,7 +59,9 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
   const size_t in_off = static_cast<size_t>(r_in) * hidden;
   const int nvec = hidden / 4;
   float4 v[kNormMaxVec];
-  float ss = 0.f;
+  float ss[VIRT];
+#pragma unroll
+  for (int j = 0; j < VIRT; ++j) ss[j] = 0.f;
 #pragma unroll
   for (int i = 0; i < kNormMaxVec; ++i) {
     const int c = threadIdx.x + i * THREADS;
@@ -74,10 +83,25 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
       if (!rows) Vec4<float>::store(resid + in_off + 4 * c, x);
     }
     v[i] = x;
-    ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    // explicit fused multiply-adds: the same roundings in every variant of the kernel
+    ss[i % VIRT] = fmaf(x.w, x.w, fmaf(x.z, x.z, fmaf(x.y, x.y, fmaf(x.x, x.x, ss[i % VIRT]))));
   }
-  ss = block_sum(ss, scratch);
-  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+  float total;
+  if (VIRT == 1) {
+    total = block_sum(ss[0], scratch);
+  } else {
+    // the waves of the threads this thread stands for are wave + (THREADS / 64) j
+    const int w = threadIdx.x / kWave;
+#pragma unroll
+    for (int j = 0; j < VIRT; ++j) {
+      const float s = wave_sum(ss[j]);
+      if ((threadIdx.x & (kWave - 1)) == 0) scratch[w + (THREADS / kWave) * j] = s;
+    }
+    __syncthreads();
+    total = 0.f;
+    for (int i = 0; i < VIRT * THREADS / kWave; ++i) total += scratch[i];
+  }
+  const float inv = rsqrtf(total / static_cast<float>(hidden) + eps);
   const size_t out_off = static_cast<size_t>(r_out) * hidden;
 #pragma unroll
   for (int i = 0; i < kNormMaxVec; ++i) {
@@ -207,17 +231,19 @@ bool add_rmsnorm_vec(float* resid, const void* delta, int delta_dt, int n_partia
                      const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
                      int hidden, float eps, hipStream_t stream) {
   if (hidden % 4 || hidden > 4 * 256 * kNormMaxVec || (delta && partial_stride % 4)) return false;
-  const bool few = n <= 128 && hidden > 1024;  // a decode step: spread each row over more threads
+  // Which variant runs depends on the number of rows; what it computes does not (see the kernel).
+  const bool wide = hidden > 1024;
+  const bool few = n <= 128 && wide;  // a decode step: spread each row over more threads
+#define PYRE_NORM_LAUNCH(THREADS, VIRT)                                                                     \
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, THREADS, VIRT>), dim3(n), dim3(THREADS), 0, stream, \
+                     resid, static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),  \
+                     static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps)
   PYRE_DISPATCH(delta_dt, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO, {
-    if (few)
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, 1024>), dim3(n), dim3(1024), 0, stream, resid,
-                         static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),
-                         static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps);
-    else
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, 256>), dim3(n), dim3(256), 0, stream, resid,
-                         static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),
-                         static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps);
+    if (few) PYRE_NORM_LAUNCH(1024, 1);
+    else if (wide) PYRE_NORM_LAUNCH(256, 4);
+    else PYRE_NORM_LAUNCH(256, 1);
   })));
+#undef PYRE_NORM_LAUNCH
   return true;
 }
 

@@ -40,6 +40,12 @@ int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, cons
                       int w_dt, long ldw, const void* bias, int bias_dt, void* out, int out_dt,
                       long ldo, int M, int N, int K, hipStream_t stream);
 
+// base[o][ids[i]][0 .. row_elems) = pattern for every o < n_outer: rows of a contiguous
+// [n_outer, n_rows, row_elems] tensor of 2- or 4-byte elements (outer_stride in elements).
+// ids_host is HOST memory. Zeroes state slots; poisons freed pages in the debug mode.
+int pyre_fill_rows(void* base, int elem_bytes, long outer_stride, int n_outer, int n_rows, long row_elems,
+                   const int* ids_host, int n_ids, unsigned pattern, hipStream_t stream);
+
 // bfloat16 products with 1..64 rows (decode): 1 if the kernel takes the shape.
 int pyre_gemm_skinny_supports(int M, int N, int K, long ldx, long ldw);
 

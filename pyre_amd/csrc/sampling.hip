@@ -68,17 +68,25 @@ __global__ __launch_bounds__(kWave) void argmax_final_kernel(const float* __rest
 }
 
 // p_i = exp((x_i - max) / T) / sum;  token = first i with cumsum(p)_i > u, u in [0, 1).
-// Thread t owns the contiguous slice [t * per, (t + 1) * per) of the vocabulary,
-// so that the cumulative sum runs in vocabulary order.
+// Thread t owns the contiguous slice [t * per, (t + 1) * per) of the vocabulary, so that the
+// cumulative sum runs in vocabulary order: the sum before slice t is (sum of the slices of the
+// waves before t's, added wave by wave) + (sum of the slices before t in its wave), which never
+// decreases with t. A thread whose slice may hold the target walks it element by element from
+// that sum; the lowest token at which a walk passes the target is the result. If rounding lets
+// every walk end at or below the target, the result is the last token of non-zero probability
+// of the last slice that was walked.
 __global__ __launch_bounds__(kThreads) void sample_kernel(const float* __restrict__ logits,
                                                           size_t row_stride,
                                                           const float* __restrict__ temperature,
                                                           const float* __restrict__ uniform,
                                                           int* __restrict__ out, int vocab) {
+  constexpr int kWaves = kThreads / kWave;
   __shared__ float scratch[16];
   __shared__ float slice_sum[kThreads];
-  __shared__ int chosen;
-  const int r = blockIdx.x, tid = threadIdx.x;
+  __shared__ float slice_before[kThreads];  // sum of the slices before this one in its wave
+  __shared__ float wave_before[kWaves + 1]; // sum of the waves before this one; [kWaves]: the total
+  __shared__ int passed, missed;
+  const int r = blockIdx.x, tid = threadIdx.x, w = tid / kWave;
   if (!(temperature[r] > 0.f)) return;  // greedy rows keep the argmax already in out[r]
   const float* row = logits + r * row_stride;
   const float inv_t = 1.f / temperature[r];
@@ -92,34 +100,46 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(const float* __restric
   float s = 0.f;
   for (int i = begin; i < end; ++i) s += expf((row[i] - mx) * inv_t);
   slice_sum[tid] = s;
-  if (tid == 0) chosen = -1;
+  if (tid == 0) { passed = 0x7fffffff; missed = -1; }
   __syncthreads();
-
-  if (tid == 0) {
-    float total = 0.f;
-    for (int t = 0; t < kThreads; ++t) total += slice_sum[t];
-    const float target = uniform[r] * total;
-    // Find the slice in which the running sum passes the target, then the element.
+  if ((tid & (kWave - 1)) == 0) {
     float run = 0.f;
-    int t = 0;
-    for (; t < kThreads - 1; ++t) {
-      if (run + slice_sum[t] > target) break;
-      run += slice_sum[t];
+    for (int j = 0; j < kWave; ++j) { slice_before[tid + j] = run; run += slice_sum[tid + j]; }
+    scratch[w] = run;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float run = 0.f;
+    for (int j = 0; j < kWaves; ++j) { wave_before[j] = run; run += scratch[j]; }
+    wave_before[kWaves] = run;
+  }
+  __syncthreads();
+  const float target = uniform[r] * wave_before[kWaves];
+  const float before = wave_before[w] + slice_before[tid];
+  // The slice that holds the target starts at or below it and ends above it; the ends are
+  // taken a little generously, since a walk's sum and the slice's own differ by rounding.
+  if (s > 0.f && before <= target && (before + s) >= target * (1.f - 1e-5f)) {
+    float run = before;
+    int pick = -1, last = -1;
+    for (int i = begin; i < end; ++i) {
+      const float p = expf((row[i] - mx) * inv_t);
+      run += p;
+      if (p > 0.f) {
+        last = i;
+        if (run > target) { pick = i; break; }
+      }
     }
-    int b = min(vocab, t * per), e = min(vocab, b + per);
-    // Rounding may leave the target just beyond the last slice's sum: fall back
-    // to the last token with non-zero probability.
-    int pick = -1;
-    for (int i = b; i < e; ++i) {
-      run += expf((row[i] - mx) * inv_t);
-      if (run > target) { pick = i; break; }
+    if (pick >= 0) atomicMin(&passed, pick);
+    else atomicMax(&missed, last);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pick = passed != 0x7fffffff ? passed : missed;
+    if (pick < 0) {  // nobody walked: the last token that can be drawn at all
+      for (int i = vocab - 1; i >= 0 && pick < 0; --i)
+        if (expf((row[i] - mx) * inv_t) > 0.f) pick = i;
     }
-    if (pick < 0) {
-      for (int i = vocab - 1; i >= 0; --i)
-        if (expf((row[i] - mx) * inv_t) > 0.f) { pick = i; break; }
-    }
-    chosen = pick < 0 ? 0 : pick;
-    out[r] = chosen;
+    out[r] = pick < 0 ? 0 : pick;
   }
 }
 

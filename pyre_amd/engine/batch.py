@@ -14,8 +14,21 @@ from dataclasses import dataclass, field
 
 import numpy as np
 
+#: sizes (requests) at which decode steps are captured in HIP graphs
+DECODE_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64)
+MIN_TABLE_WIDTH = 8
 
-TILE = 32  #: tokens of one request that the prompt-portion attention kernel takes at a time
+
+def round_decode_shape(n_rows: int, n_pages: int) -> tuple[int, int]:
+    """The fixed sizes at which a step's single-token requests are run: the number of
+    requests rounded up to a bucket (beyond the largest bucket: as it is), the block
+    table's width to a power of two of pages. A captured step is replayed at these
+    sizes, and whoever chooses a launch shape that changes the order of a sum (how the
+    keys of a request are split) chooses it from these, so that an eager step and a
+    replayed one give the same bits. This function is the only place that rounds."""
+    rows = next((b for b in DECODE_ROW_BUCKETS if b >= n_rows), n_rows)
+    width = max(MIN_TABLE_WIDTH, 1 << (max(1, n_pages) - 1).bit_length())
+    return rows, width
 
 
 @dataclass
@@ -45,11 +58,13 @@ class HostBatch:
     logit_rows: np.ndarray      #: [M] token indices whose logits are wanted, in entry order
     slots: list[np.ndarray]     #: per page group [N]: cache slot of each token
     tables: list[np.ndarray]    #: per page group [S, P]: block tables (-1: released or unused)
+    page_size: int = 0
     max_q_len: int = 0
-    decode_tokens: np.ndarray = None   #: token indices of requests that bring one token
-    prefill_tiles: np.ndarray = None   #: [T, 2] (first token, count <= TILE) of the others, longest context first
-    max_decode_ctx: int = 0            #: longest context among the single-token requests
+    n_single: int = 0                  #: requests that bring one token
+    max_single_ctx: int = 0            #: longest context among them
     token_src: np.ndarray = None       #: [N] row of the device-side ids that a token comes from, or -1
+    #: what the parts asked for beside the above (:class:`~pyre_amd.parts.base.StepArraySpec`)
+    arrays: dict = field(default_factory=dict)
 
     @property
     def decode_only(self) -> bool:
@@ -58,6 +73,18 @@ class HostBatch:
     @property
     def feeds(self) -> bool:
         return self.token_src is not None and bool((self.token_src >= 0).any())
+
+    def decode_shape(self) -> tuple[int, int]:
+        """(requests, context in tokens) at which the single-token requests are to be
+        launched: their number and longest context, rounded by :func:`round_decode_shape`."""
+        ps = max(1, self.page_size)
+        rows, width = round_decode_shape(self.n_single, -(-self.max_single_ctx // ps))
+        return rows, width * ps
+
+    def attach(self, specs) -> "HostBatch":
+        """Build the arrays that the parts asked for."""
+        self.arrays = {s.name: np.ascontiguousarray(s.build(self), dtype=np.int32) for s in specs}
+        return self
 
 
 def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: int | None = None) -> HostBatch:
@@ -125,28 +152,72 @@ def build_host_batch(entries: list[Entry], cache, vocab_size: int, table_width: 
                                "lies in a released page")
         slots.append((pages * ps + positions % ps).astype(np.int32))
     single = counts == 1
-    decode_tokens = q_start_a[:-1][single]
-    max_decode_ctx = int(ctx_len[single].max()) if single.any() else 0
-    tiles = []
-    for s in np.nonzero(~single)[0]:
-        a, b = q_start[s], q_start[s + 1]
-        tiles.extend((int(positions[t0]) + min(TILE, b - t0), t0, min(TILE, b - t0)) for t0 in range(a, b, TILE))
-    tiles.sort(key=lambda t: -t[0])  # the tiles with the most keys start first
     return HostBatch(
-        decode_tokens=i32(decode_tokens), prefill_tiles=i32([t[1:] for t in tiles]).reshape(-1, 2),
-        max_decode_ctx=max_decode_ctx,
+        page_size=ps, n_single=int(single.sum()), max_single_ctx=int(ctx_len[single].max()) if single.any() else 0,
         n_tokens=n_tokens, n_seqs=n_seqs, rids=[e.rid for e in entries], tokens=tok.astype(np.int32),
         positions=positions.astype(np.int32), seq_of_token=seq_of_token, q_start=q_start_a,
         ctx_len=ctx_len.astype(np.int32), state_slots=i32(state_slots), logit_rows=i32(logit_rows),
         slots=slots, tables=tables, max_q_len=max_q, token_src=i32(token_src))
 
 
+def prepare_step(entries: list[Entry], cache, vocab_size: int, graph_max_rows: int = 0,
+                 has_fed_ids: bool = False) -> tuple[HostBatch, tuple[int, int] | None]:
+    """Everything of a step that can fail, all or nothing: admit the requests not seen
+    before, reserve pages for every entry's tokens, lay the batch out. If any of it
+    fails (no pages, no slot, a token outside the vocabulary, a request named twice, a
+    request past the longest length) the error is raised with this call's admissions
+    and reservations undone: the cache is as it was.
+
+    Returns the batch and, for a step of single tokens of at most ``graph_max_rows``
+    requests that each want their logits, the fixed sizes (rows, table width) at which
+    it can be captured and replayed; else None."""
+    from pyre_amd.cache.allocator import OutOfPages
+
+    admitted, reserved = [], []
+    try:
+        seen = set()
+        for e in entries:
+            if e.rid in seen:
+                raise ValueError(f"request {e.rid!r} appears twice in one step")
+            seen.add(e.rid)
+        # all pages or none: checked for the whole step before the first one is taken
+        if cache.page_groups:
+            need = sum(cache.pages_needed(e.rid if e.rid in cache else None, len(e.tokens)) for e in entries)
+            if need > cache.free_pages():
+                raise OutOfPages(f"the step needs {need} pages, {cache.free_pages()} are free")
+        for e in entries:
+            if e.rid not in cache:
+                cache.add_request(e.rid)
+                admitted.append(e.rid)
+        for e in entries:
+            cache.reserve(e.rid, len(e.tokens))
+            reserved.append(e.rid)
+        n_tokens = sum(len(e.tokens) for e in entries)
+        pages = max((len(cache.block_table(e.rid, 0)) for e in entries), default=0) if cache.page_groups else 0
+        graphable = (n_tokens == len(entries) and n_tokens <= graph_max_rows and all(len(e.want) == 1 for e in entries))
+        if graphable:
+            rows, width = round_decode_shape(n_tokens, pages)
+        else:
+            width = max(MIN_TABLE_WIDTH, -(-pages // 8) * 8)
+        hb = build_host_batch(entries, cache, vocab_size, table_width=width)
+        if hb.feeds and not has_fed_ids:
+            raise ValueError("an entry takes its token from the device, but no ids were given")
+        return hb, ((rows, width) if graphable else None)
+    except BaseException:
+        for rid in admitted:
+            cache.free_request(rid)
+        for rid in reserved:
+            if rid not in admitted:
+                cache.unreserve(rid)
+        raise
+
+
 def pad_decode_batch(hb: HostBatch, n_rows: int, scratch_slot: int, max_ctx: int) -> HostBatch:
     """A decode-only batch widened to ``n_rows`` requests with rows that do nothing:
     token 0 at position 0, no cache slot to write to, an empty block table (every key
     hidden), the scratch state slot. A captured step is replayed at a fixed size;
-    the rows beyond the live requests are these. ``max_ctx`` (the longest context
-    the step's table can hold) fixes how the keys are split."""
+    the rows beyond the live requests are these. ``max_ctx`` is the longest context
+    the step's table can hold."""
     pad = n_rows - hb.n_seqs
     if pad < 0 or not hb.decode_only:
         raise ValueError("only decode batches can be padded, and only upwards")
@@ -162,5 +233,5 @@ def pad_decode_batch(hb: HostBatch, n_rows: int, scratch_slot: int, max_ctx: int
         logit_rows=i32(range(n_rows)),
         slots=[cat(s, [-1] * pad) for s in hb.slots],
         tables=[np.concatenate([t, np.full((pad, t.shape[1]), -1, dtype=np.int32)]) for t in hb.tables],
-        max_q_len=1, decode_tokens=i32(range(n_rows)), prefill_tiles=i32([]).reshape(-1, 2),
-        max_decode_ctx=max_ctx, token_src=cat(hb.token_src, [-1] * pad))
+        max_q_len=1, page_size=hb.page_size, n_single=n_rows, max_single_ctx=max_ctx,
+        token_src=cat(hb.token_src, [-1] * pad))

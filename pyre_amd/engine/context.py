@@ -72,9 +72,10 @@ class Runtime:
         return self.dtype == torch.float32
 
 
-def meta_layout(n_cap: int, s_cap: int, table_widths: list[int]) -> tuple[dict, int]:
+def meta_layout(n_cap: int, s_cap: int, table_widths: list[int], extra=()) -> tuple[dict, int]:
     """Offsets (in int32 elements) of the step arrays inside the metadata buffer
-    for a step of up to ``n_cap`` tokens and ``s_cap`` requests."""
+    for a step of up to ``n_cap`` tokens and ``s_cap`` requests. ``extra``: the arrays
+    that parts asked for (:class:`~pyre_amd.parts.base.StepArraySpec`)."""
     off = 0
     lay = {}
 
@@ -83,9 +84,10 @@ def meta_layout(n_cap: int, s_cap: int, table_widths: list[int]) -> tuple[dict, 
         lay[name] = (off, n)
         off += (n + 3) // 4 * 4
 
-    for name in ("tokens", "positions", "seq_of_token", "logit_rows", "decode_tokens", "token_src"):
+    for name in ("tokens", "positions", "seq_of_token", "logit_rows", "token_src"):
         put(name, n_cap)
-    put("prefill_tiles", 2 * (n_cap // 32 + s_cap))
+    for spec in extra:
+        put("x:" + spec.name, int(spec.capacity(n_cap, s_cap)))
     put("q_start", s_cap + 1)
     put("ctx_len", s_cap)
     put("state_slots", s_cap)
@@ -98,10 +100,12 @@ def meta_layout(n_cap: int, s_cap: int, table_widths: list[int]) -> tuple[dict, 
 class MetaBuffers:
     """Pinned host staging and the device copy of a step's int32 arrays."""
 
-    def __init__(self, device: torch.device, max_tokens: int, max_seqs: int, table_widths: list[int]):
-        """``table_widths``: the widest block table of each page group."""
+    def __init__(self, device: torch.device, max_tokens: int, max_seqs: int, table_widths: list[int], extra=()):
+        """``table_widths``: the widest block table of each page group; ``extra``: the
+        arrays that parts asked for."""
         self.max_widths = table_widths
-        _, size = meta_layout(max_tokens, max_seqs, table_widths)
+        self.extra = list(extra)
+        _, size = meta_layout(max_tokens, max_seqs, table_widths, self.extra)
         self.capacity = size
         self.host = torch.empty(size, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
@@ -113,7 +117,7 @@ class MetaBuffers:
         n_cap = n_cap or hb.n_tokens
         s_cap = s_cap or hb.n_seqs
         widths = [t.shape[1] for t in hb.tables]
-        lay, used = meta_layout(n_cap, s_cap, widths)
+        lay, used = meta_layout(n_cap, s_cap, widths, self.extra)
         if used > self.capacity:
             raise RuntimeError(f"step of {n_cap} tokens / {s_cap} requests exceeds the engine's limits")
         if self._pending:
@@ -128,7 +132,12 @@ class MetaBuffers:
         fill("tokens", hb.tokens), fill("positions", hb.positions), fill("seq_of_token", hb.seq_of_token)
         fill("logit_rows", hb.logit_rows), fill("q_start", hb.q_start), fill("ctx_len", hb.ctx_len)
         fill("state_slots", hb.state_slots)
-        fill("decode_tokens", hb.decode_tokens), fill("prefill_tiles", hb.prefill_tiles)
+        for spec in self.extra:
+            arr = hb.arrays[spec.name]
+            if arr.size > lay["x:" + spec.name][1]:
+                raise RuntimeError(f"step array {spec.name!r} has {arr.size} entries, its stated capacity is "
+                                   f"{lay['x:' + spec.name][1]}")
+            fill("x:" + spec.name, arr)
         o, n = lay["token_src"]
         h[o:o + n] = -1
         if hb.token_src is not None:
@@ -152,16 +161,18 @@ class MetaBuffers:
 
 
 @dataclass
-class KVLayerView:
-    """One layer's keys and values and the step's addressing for its group."""
+class PagedLayerView:
+    """One layer's paged tensors and the step's addressing for its group."""
 
-    k: torch.Tensor                  #: [pages, nkv, page_size, hd]
-    v: torch.Tensor                  #: [pages, nkv, hd, page_size]
+    tensors: dict                    #: name -> [pages, *page_shape], as the mixer's description laid them out
     table: torch.Tensor              #: [S, P] int32, this step's block tables
-    slots: torch.Tensor              #: [N] int32, where this step's tokens go
+    slots: torch.Tensor              #: [N] int32, where this step's tokens go (page * page_size + offset)
     page_size: int
     window: int
     writes: bool = True              #: False: the layer reads a cache another layer wrote
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self.tensors[name]
 
 
 @dataclass
@@ -186,8 +197,7 @@ class StepContext:
     q_start: torch.Tensor
     ctx_len: torch.Tensor
     state_slots: torch.Tensor
-    decode_tokens: torch.Tensor = None   #: flat indices of the single-token requests' tokens
-    prefill_tiles: torch.Tensor = None   #: (first token, count) of the other requests' tiles
+    arrays: dict = field(default_factory=dict)  #: name -> int32 device array that a part asked for
 
     @property
     def workspace(self) -> Workspace:

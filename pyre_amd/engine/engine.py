@@ -16,10 +16,9 @@ import torch
 from pyre_amd.cache import CacheManager
 from pyre_amd.config.engine import EngineConfig
 from pyre_amd.config.model import ModelConfig
-from pyre_amd.engine.batch import Entry, build_host_batch, pad_decode_batch
-from pyre_amd.engine.context import (TORCH_DTYPES, KVLayerView, MetaBuffers, Runtime, StateLayerView,
+from pyre_amd.engine.batch import DECODE_ROW_BUCKETS, Entry, pad_decode_batch, prepare_step, round_decode_shape
+from pyre_amd.engine.context import (TORCH_DTYPES, MetaBuffers, PagedLayerView, Runtime, StateLayerView,
                                      StepContext)
-from pyre_amd.parts.fast import DECODE_ROW_BUCKETS
 from pyre_amd.parts.model import LayeredModel
 from pyre_amd.registry import get_architecture, load_config
 from pyre_amd.weights.loader import adopt_state, load_weights
@@ -53,11 +52,18 @@ class Engine:
         specs = model.cache_specs()
         probe = CacheManager(specs, ec.page_size, 1, ec.max_num_seqs, self.max_model_len)
         num_pages = self._choose_num_pages(probe)
-        self.cache = CacheManager(specs, ec.page_size, num_pages, ec.max_num_seqs, self.max_model_len)
-        self.cache.materialize(self.device, self.dtype)
-        # captured steps round their tables up to a power of two of pages
-        widths = [max(8, 1 << (self.cache.max_pages_per_seq - 1).bit_length()) for _ in self.cache.page_groups]
-        self.meta = MetaBuffers(self.device, max(ec.max_num_batched_tokens, ec.max_num_seqs), ec.max_num_seqs, widths)
+        from pyre_amd.hip import ops
+
+        with torch.cuda.device(self.device):
+            self.cache = CacheManager(specs, ec.page_size, num_pages, ec.max_num_seqs, self.max_model_len,
+                                      fill=ops.fill_rows, poison=ec.debug_poison)
+            self.cache.materialize(self.device, self.dtype)
+        # A captured step runs at rounded sizes: its rows may exceed max_num_seqs (49 requests
+        # run as 64), its tables are a power of two of pages wide.
+        seq_cap, width = round_decode_shape(ec.max_num_seqs, self.cache.max_pages_per_seq)
+        self.step_arrays = model.step_arrays()
+        self.meta = MetaBuffers(self.device, max(ec.max_num_batched_tokens, seq_cap), seq_cap,
+                                [width for _ in self.cache.page_groups], self.step_arrays)
         self.steps_run = 0
         #: captured decode steps: (rows, table width) -> "warm" (ran eagerly once) or (graph, logits)
         self._graphs: dict[tuple[int, int], object] = {}
@@ -119,23 +125,11 @@ class Engine:
         import torch.cuda.tunable as tunable
 
         from pyre_amd.parts.fast import SKINNY_MAX_ROWS
-        from pyre_amd.parts.linear import Linear
 
         shapes = {}
-
-        def walk(obj, depth=0):
-            if isinstance(obj, Linear):
-                if obj.weight is not None and obj.weight.dtype == torch.bfloat16:
-                    shapes.setdefault((obj.out_features, obj.in_features), obj)
-                return
-            if depth > 4 or not hasattr(obj, "__dict__"):
-                return
-            for v in vars(obj).values():
-                for item in (v if isinstance(v, (list, tuple)) else [v]):
-                    if hasattr(item, "__dict__") and type(item).__module__.startswith(("pyre_amd", "test", "tests")):
-                        walk(item, depth + 1)
-
-        walk(self.model)
+        for lin in self.model.linears():
+            if lin.weight is not None and lin.weight.dtype == torch.bfloat16:
+                shapes.setdefault((lin.out_features, lin.in_features), lin)
         tunable.enable(True)
         if hasattr(tunable, "write_file_on_exit"):
             tunable.write_file_on_exit(False)
@@ -175,6 +169,16 @@ class Engine:
         device, rows in the order of the entries and of each ``want`` (None if no
         logits are wanted).
 
+        The step is all or nothing: if it cannot be prepared (no pages, no slot, a token
+        outside the vocabulary, a request named twice) the error is raised with every
+        admission and reservation of this call undone, so that the caller sees the cache
+        it had and may try again with another batch.
+
+        The returned tensor is a view of scratch memory that belongs to the engine: the
+        next ``step`` overwrites it (work put on the same stream before that, a sampler's
+        kernels or a copy to the host, reads it in order and is safe). Copy it if it has
+        to outlive the next step.
+
         An entry with ``feed = i`` takes its one token from ``fed_ids[i]`` (int32 on
         the device, for instance the ids a sampler has just written) when the step
         runs on the device: the host can put the step on the stream without waiting
@@ -186,32 +190,15 @@ class Engine:
             raise ValueError(f"step of {n_tokens} tokens exceeds max_num_batched_tokens={ec.max_num_batched_tokens}")
         if len(entries) > ec.max_num_seqs:
             raise ValueError(f"step of {len(entries)} requests exceeds max_num_seqs={ec.max_num_seqs}")
-        cache = self.cache
-        for e in entries:
-            if e.rid not in cache:
-                cache.add_request(e.rid)
-        for e in entries:
-            cache.reserve(e.rid, len(e.tokens))
-        pages = max((len(cache.block_table(e.rid, 0)) for e in entries), default=0) if cache.page_groups else 0
-        graphable = (ec.use_graphs and n_tokens == len(entries) and n_tokens <= GRAPH_MAX_ROWS
-                     and all(len(e.want) == 1 for e in entries))
-        if graphable:
-            # Fixed sizes, so that the step can be captured once and replayed:
-            # the table as wide as a power of two of pages, the rows up to a bucket.
-            width = max(8, 1 << (pages - 1).bit_length())
-            rows = next(b for b in GRAPH_ROW_BUCKETS if b >= n_tokens)
-        else:
-            width = max(8, -(-pages // 8) * 8)
-        hb = build_host_batch(entries, cache, self.vocab_size, table_width=width)
-        if hb.feeds and fed_ids is None:
-            raise ValueError("an entry takes its token from the device, but no ids were given")
+        hb, graph_shape = prepare_step(entries, self.cache, self.vocab_size, GRAPH_MAX_ROWS if ec.use_graphs else 0,
+                                       fed_ids is not None)
         with torch.cuda.device(self.device):
-            if graphable:
-                logits = self._step_captured(hb, rows, width, fed_ids)
+            if graph_shape is not None:
+                logits = self._step_captured(hb, *graph_shape, fed_ids)
             else:
                 logits = self._run(hb, fed_ids)
         for e in entries:
-            cache.commit(e.rid, len(e.tokens))
+            self.cache.commit(e.rid, len(e.tokens))
         self.steps_run += 1
         return logits
 
@@ -232,7 +219,7 @@ class Engine:
             n_logits=len(hb.logit_rows), tokens=views["tokens"], positions=views["positions"],
             seq_of_token=views["seq_of_token"], logit_rows=views["logit_rows"][:len(hb.logit_rows)],
             q_start=views["q_start"], ctx_len=views["ctx_len"], state_slots=views["state_slots"],
-            decode_tokens=views["decode_tokens"], prefill_tiles=views["prefill_tiles"])
+            arrays={spec.name: views["x:" + spec.name] for spec in self.step_arrays})
         return ctx, self._layer_views(views)
 
     def _forward(self, ctx, caches):
@@ -246,7 +233,7 @@ class Engine:
             ops.use_stream(None)
 
     def _run(self, hb, fed_ids=None):
-        ctx, caches = self._context(hb, fed_ids)
+        ctx, caches = self._context(hb.attach(self.step_arrays), fed_ids)
         return self._forward(ctx, caches)
 
     def _step_captured(self, hb, rows: int, width: int, fed_ids=None):
@@ -256,6 +243,7 @@ class Engine:
         live = hb.n_seqs
         key = (rows, width)
         padded = pad_decode_batch(hb, rows, self.cache.max_num_seqs, width * self.cache.page_size)
+        padded.attach(self.step_arrays)
         state = self._graphs.get(key)
         if state is None:
             ctx, caches = self._context(padded, fed_ids)
@@ -291,11 +279,12 @@ class Engine:
                 out.append(None)
                 continue
             kind, gi = where
-            if kind == "kv":
+            if kind == "paged":
                 g = cache.page_groups[gi]
                 li = g.layer_index(src)
-                out.append(KVLayerView(g.k[li], g.v[li], views[f"table{gi}"], views[f"slots{gi}"],
-                                       g.page_size, g.spec.window, writes=call.cache_from is None))
+                out.append(PagedLayerView({name: t[li] for name, t in g.tensors.items()}, views[f"table{gi}"],
+                                          views[f"slots{gi}"], g.page_size, g.spec.window,
+                                          writes=call.cache_from is None))
             else:
                 g = cache.state_groups[gi]
                 out.append(StateLayerView(g.tensor[g.layer_index(src)], views["state_slots"]))

@@ -20,7 +20,6 @@ import json
 import sys
 from pathlib import Path
 
-PAGE_SIZE = 16
 TOKEN_ROUNDING = 64
 
 
@@ -31,8 +30,14 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (a divisor of 64)")
+    ap.add_argument("--max-seqs", type=int, default=8, help="most requests that are live at a time")
+    ap.add_argument("--poison", action="store_true",
+                    help="debugging aid: freed cache pages and state slots are filled with NaN")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
+    if args.page_size <= 0 or TOKEN_ROUNDING % args.page_size:
+        ap.error(f"--page-size must divide {TOKEN_ROUNDING}")
 
     def note(msg: str) -> None:
         print(f"[trace_run] {msg}", file=sys.stderr, flush=True)
@@ -54,15 +59,19 @@ def main(argv: list[str] | None = None) -> int:
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     max_tokens = -(-max(args.max_tokens, TOKEN_ROUNDING) // TOKEN_ROUNDING) * TOKEN_ROUNDING
-    from pyre_amd.registry import load_config
+    from pyre_amd.registry import get_architecture, load_config
 
-    model_limit = getattr(load_config(args.model), "max_position_embeddings", 0) or 0
-    ec = EngineConfig(dtype=args.dtype, device=args.device, page_size=PAGE_SIZE,
-                      max_cached_tokens=max_tokens, max_num_seqs=8, max_model_len=max(model_limit, max_tokens),
-                      max_num_batched_tokens=max(max_tokens, 4096), use_graphs=False)
+    # the longest request: what the model's description says, or the pool if that is more
+    config = load_config(args.model)
+    model_limit = get_architecture(config.architecture).build(config).max_positions
+    ec = EngineConfig(dtype=args.dtype, device=args.device, page_size=args.page_size,
+                      max_cached_tokens=max_tokens, max_num_seqs=args.max_seqs,
+                      max_model_len=max(model_limit, max_tokens),
+                      max_num_batched_tokens=max(max_tokens, 4096), use_graphs=False, debug_poison=args.poison)
     note(f"loading {args.model} ({args.dtype}) ...")
     engine = Engine.from_folder(args.model, ec)
-    note(f"ready: {engine.cache.page_groups[0].num_pages if engine.cache.page_groups else 0} pages of {PAGE_SIZE} tokens")
+    note(f"ready: {engine.cache.page_groups[0].num_pages if engine.cache.page_groups else 0} pages of "
+         f"{args.page_size} tokens")
 
     for line in sys.stdin:
         line = line.strip()

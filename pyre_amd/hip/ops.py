@@ -197,6 +197,33 @@ def reduce_partials(p: Partials, out: torch.Tensor, n: int) -> None:
     call("pyre_reduce_partials", *p._args(p.width), out.data_ptr(), dtype_code(out), n, p.width, _stream())
 
 
+_FILL_PATTERNS = {(4, "zero"): 0, (2, "zero"): 0, (4, "nan"): 0x7FC00000, (2, "nan"): 0x7FC0}
+
+
+def fill_rows(tensor: torch.Tensor, ids: list[int], value: float) -> None:
+    """tensor[:, id] = value for every listed id; ``tensor`` is contiguous ``[outer, rows, ...]``
+    of float32 or bfloat16, ``value`` is 0.0 or NaN (state slots are zeroed with it, freed pages
+    poisoned)."""
+    import ctypes
+    import math
+
+    _dev(tensor)
+    _contig("tensor", tensor)
+    if tensor.dim() < 2 or tensor.dtype not in _DT:
+        raise KernelError("fill_rows: a float32 or bfloat16 tensor [outer, rows, ...] expected")
+    if not ids:
+        return
+    kind = "nan" if math.isnan(value) else "zero" if value == 0.0 else None
+    if kind is None:
+        raise KernelError("fill_rows: the value must be 0 or NaN")
+    outer, rows = tensor.shape[0], tensor.shape[1]
+    row_elems = tensor.stride(1)
+    arr = (ctypes.c_int * len(ids))(*[int(i) for i in ids])
+    with torch.cuda.device(tensor.device):
+        call("pyre_fill_rows", tensor.data_ptr(), tensor.element_size(), tensor.stride(0), outer, rows, row_elems,
+             ctypes.cast(arr, ctypes.c_void_p), len(ids), _FILL_PATTERNS[(tensor.element_size(), kind)], _stream())
+
+
 def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
                  m: int, a_rows: torch.Tensor | None = None) -> None:
     """out[0:m] = a[0:m] (or a[a_rows]) @ w.T (+ bias), fp32 accumulation in ascending k."""

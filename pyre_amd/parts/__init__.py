@@ -1,9 +1,9 @@
-from pyre_amd.parts.base import (AttentionSpec, BlockSpec, EmbeddingSpec, FeedForward, KVCacheSpec,
+from pyre_amd.parts.base import (AttentionSpec, BlockSpec, EmbeddingSpec, FeedForward,
                                  LayerCall, LMHeadSpec, Mixer, ModelSpec, Norm, NoPositionSpec, Part,
-                                 PositionEncoding, RMSNormSpec, RotarySpec, StateCacheSpec, SwiGLUSpec,
+                                 PagedCacheSpec, PagedTensorSpec, PositionEncoding, RMSNormSpec, RotarySpec, StateCacheSpec, SwiGLUSpec,
                                  TensorSpec, make_part, register_part)
 
-__all__ = ["AttentionSpec", "BlockSpec", "EmbeddingSpec", "FeedForward", "KVCacheSpec", "LayerCall",
-           "LMHeadSpec", "Mixer", "ModelSpec", "Norm", "NoPositionSpec", "Part", "PositionEncoding",
+__all__ = ["AttentionSpec", "BlockSpec", "EmbeddingSpec", "FeedForward", "LayerCall",
+           "LMHeadSpec", "Mixer", "ModelSpec", "Norm", "NoPositionSpec", "PagedCacheSpec", "PagedTensorSpec", "Part", "PositionEncoding",
            "RMSNormSpec", "RotarySpec", "StateCacheSpec", "SwiGLUSpec", "TensorSpec", "make_part",
            "register_part"]

@@ -4,10 +4,50 @@ from __future__ import annotations
 
 import torch
 
+import numpy as np
+
 from pyre_amd.hip import ops
 from pyre_amd.parts import fast
-from pyre_amd.parts.base import AttentionSpec, KVCacheSpec, Mixer, TensorSpec, make_part
+from pyre_amd.parts.base import (AttentionSpec, Mixer, PagedCacheSpec, PagedTensorSpec, StepArraySpec, TensorSpec,
+                                 make_part)
 from pyre_amd.parts.linear import Linear, linear_specs
+
+
+def KVCacheSpec(num_kv_heads: int, head_dim: int, window: int = 0) -> PagedCacheSpec:
+    """What this attention keeps per token, laid out for its kernels: the rotated key as
+    ``k [pages, kv_heads, page_size, head_dim]`` (a head's keys of a page lie together, one
+    key is one contiguous run) and the value transposed, ``v [pages, kv_heads, head_dim,
+    page_size]``, so that the MFMA kernels read runs of tokens for one feature."""
+    return PagedCacheSpec((PagedTensorSpec("k", (num_kv_heads, head_dim), token_axis=1),
+                           PagedTensorSpec("v", (num_kv_heads, head_dim), token_axis=2)), window)
+
+
+#: tokens of one request that the prompt-portion attention kernel takes at a time
+TILE = 32
+
+
+def _decode_tokens(hb) -> np.ndarray:
+    """Flat indices of the tokens of requests that bring a single token."""
+    counts = hb.q_start[1:] - hb.q_start[:-1]
+    return hb.q_start[:-1][counts == 1]
+
+
+def _prefill_tiles(hb) -> np.ndarray:
+    """[T, 2] (first token, count <= TILE) of the requests that bring more than one token,
+    the tiles that see the most keys first."""
+    counts = hb.q_start[1:] - hb.q_start[:-1]
+    tiles = []
+    for s in np.nonzero(counts != 1)[0]:
+        a, b = int(hb.q_start[s]), int(hb.q_start[s + 1])
+        tiles.extend((int(hb.positions[t0]) + min(TILE, b - t0), t0, min(TILE, b - t0)) for t0 in range(a, b, TILE))
+    tiles.sort(key=lambda t: -t[0])
+    return np.asarray([t[1:] for t in tiles], dtype=np.int32).reshape(-1, 2)
+
+
+STEP_ARRAYS = (
+    StepArraySpec("attention.decode_tokens", lambda n_cap, s_cap: n_cap, _decode_tokens),
+    StepArraySpec("attention.prefill_tiles", lambda n_cap, s_cap: 2 * (n_cap // TILE + s_cap), _prefill_tiles),
+)
 
 
 class Attention(Mixer):
@@ -33,6 +73,12 @@ class Attention(Mixer):
         s = self.spec
         return KVCacheSpec(s.num_kv_heads, s.head_dim, s.window)
 
+    def step_arrays(self):
+        return list(STEP_ARRAYS)
+
+    def linears(self) -> list:
+        return [self.qkv, self.out]
+
     def tensor_specs(self) -> list[TensorSpec]:
         s, p = self.spec, self.spec.prefix
         return (linear_specs(f"{p}.q_proj", self.q_dim, s.hidden_size, s.qkv_bias)
@@ -54,12 +100,13 @@ class Attention(Mixer):
         qkv = self.qkv.forward(ctx, h, n)
         q = ws.get("attn.q", (n, self.q_dim), ctx.dtype)
         cos, sin, rot = self.position.rotary(ctx.runtime)
-        ops.rope_kv_write(qkv, q, cache.k if cache.writes else None, cache.v if cache.writes else None,
+        k_pages, v_pages = cache["k"], cache["v"]
+        ops.rope_kv_write(qkv, q, k_pages if cache.writes else None, v_pages if cache.writes else None,
                           cos, sin, rot, ctx.positions, cache.slots, n, s.num_heads, s.num_kv_heads,
                           s.head_dim, cache.page_size)
         o = ws.get("attn.o", (n, self.q_dim), ctx.dtype)
         if not fast.attention(self, ctx, q, o, cache):
-            ops.attn_generic(q, o, cache.k, cache.v, ctx.positions, ctx.seq_of_token, cache.table, n,
+            ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, n,
                              s.num_heads, s.num_kv_heads, s.head_dim, cache.page_size, self.scale,
                              cache.window)
         return self.out.forward(ctx, o, n)

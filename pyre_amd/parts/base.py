@@ -12,9 +12,10 @@ Interfaces (duck-typed; the base classes document them):
 
 ``Part``          ``tensor_specs()`` names the checkpoint tensors it needs;
                   ``bind(tensors, runtime)`` takes them (already on the device).
-``Mixer``         ``cache_spec()`` says what it keeps per token (pages of keys and
-                  values, all or a window) or per request (fixed-size state), or
-                  nothing; ``forward(ctx, h, cache) -> Partials`` turns the normed
+``Mixer``         ``cache_spec()`` says what it keeps per token (tensors in pages, in a
+                  layout of its own choice, all tokens or a window) or per request
+                  (fixed-size state), or nothing; ``step_arrays()`` names the work
+                  lists its kernels want of every step; ``forward(ctx, h, cache) -> Partials`` turns the normed
                   hidden rows into the term to be added to the residual stream.
 ``FeedForward``   ``forward(ctx, h) -> Partials``.
 ``Norm``          ``forward(ctx, resid, delta, out, rows=None)``: adds ``delta`` to the
@@ -55,15 +56,60 @@ class TensorSpec:
 
 
 @dataclass(frozen=True)
-class KVCacheSpec:
-    """Keys and values per token, in pages. ``window`` = 0 keeps every key;
-    ``window`` = W keeps the last W (a query at position p sees p-W+1 .. p)."""
+class PagedTensorSpec:
+    """One tensor that a mixer keeps per token, in pages.
 
-    num_kv_heads: int
-    head_dim: int
+    ``token_shape`` is what one token owns, for instance ``(kv_heads, head_dim)`` for a
+    key. A page of ``page_size`` tokens has the token axis inserted at ``token_axis``:
+    ``token_axis = 1`` on ``(kv_heads, head_dim)`` gives pages of ``(kv_heads, page_size,
+    head_dim)`` (every head's keys of a page lie together), ``token_axis = 2`` gives
+    ``(kv_heads, head_dim, page_size)`` (transposed: runs of tokens), ``token_axis = 0``
+    gives ``(page_size, ...)`` (one record per token). The layout is the mixer's choice,
+    made for its kernels; the cache manager only allocates what it is told.
+    ``dtype`` is "model" (the engine's element type) or "float32".
+    """
+
+    name: str
+    token_shape: tuple[int, ...]
+    token_axis: int = 0
+    dtype: str = "model"
+
+    def __post_init__(self) -> None:
+        if not (0 <= self.token_axis <= len(self.token_shape)):
+            raise ValueError(f"paged tensor {self.name!r}: token_axis {self.token_axis} does not fit "
+                             f"token_shape {self.token_shape}")
+        if self.dtype not in ("model", "float32"):
+            raise ValueError(f"paged tensor {self.name!r}: dtype must be 'model' or 'float32'")
+
+    def page_shape(self, page_size: int) -> tuple[int, ...]:
+        s = list(self.token_shape)
+        s.insert(self.token_axis, page_size)
+        return tuple(s)
+
+    def elements_per_token(self) -> int:
+        n = 1
+        for d in self.token_shape:
+            n *= d
+        return n
+
+
+@dataclass(frozen=True)
+class PagedCacheSpec:
+    """What a mixer keeps per token: one or more tensors in pages that share a block
+    table. ``window`` = 0 keeps every token; ``window`` = W keeps the last W (a query at
+    position p sees p-W+1 .. p), and pages that no later query can see are given back."""
+
+    tensors: tuple[PagedTensorSpec, ...]
     window: int = 0
 
-    kind: ClassVar[str] = "kv"
+    kind: ClassVar[str] = "paged"
+
+    def __post_init__(self) -> None:
+        names = [t.name for t in self.tensors]
+        if not names or len(names) != len(set(names)):
+            raise ValueError("a paged cache needs at least one tensor, each with a name of its own")
+        if self.window < 0:
+            raise ValueError("window must not be negative")
 
 
 @dataclass(frozen=True)
@@ -80,10 +126,31 @@ class StateCacheSpec:
 # --------------------------------------------------------------------------- part classes
 
 
+@dataclass(frozen=True)
+class StepArraySpec:
+    """An int32 array that a part's kernels need of every step beside the common ones
+    (tokens, positions, block tables, ...): work lists, tiles, anything that follows from
+    the step's batch. ``build(host_batch)`` returns it (numpy int32, any shape);
+    ``capacity(max_tokens, max_seqs)`` bounds its number of elements. The engine builds it
+    on the host, uploads it in the step's one copy and hands it to the parts as
+    ``ctx.arrays[name]`` (device) and ``ctx.host.arrays[name]`` (host). Parts that name the
+    same array share it."""
+
+    name: str
+    capacity: Any = field(compare=False)
+    build: Any = field(compare=False)
+
+
 class Part:
     """Base of everything that owns tensors."""
 
     def tensor_specs(self) -> list[TensorSpec]:
+        return []
+
+    def linears(self) -> list:
+        """The matrix products (:class:`~pyre_amd.parts.linear.Linear`) this part owns,
+        for whoever wants to prepare them (the engine lets the BLAS library time its
+        kernels for their shapes)."""
         return []
 
     def bind(self, tensors: dict[str, Any], runtime: Any) -> None:
@@ -91,8 +158,12 @@ class Part:
 
 
 class Mixer(Part):
-    def cache_spec(self) -> KVCacheSpec | StateCacheSpec | None:
+    def cache_spec(self) -> PagedCacheSpec | StateCacheSpec | None:
         return None
+
+    def step_arrays(self) -> list[StepArraySpec]:
+        """Arrays that this mixer's kernels want of every step beside the common ones."""
+        return []
 
     def forward(self, ctx, h, cache):
         raise NotImplementedError

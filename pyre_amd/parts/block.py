@@ -39,6 +39,9 @@ class PreNormBlock(Part):
         for p in self.parts():
             p.bind(tensors, runtime)
 
+    def linears(self) -> list:
+        return [lin for p in self.parts() for lin in p.linears()]
+
     def forward(self, ctx, state: Hidden, cache) -> None:
         h = ctx.workspace.get("block.h", (ctx.n_tokens, state.resid.shape[1]), ctx.dtype)
         self.mixer_norm.forward(ctx, state.resid, state.pending, h)

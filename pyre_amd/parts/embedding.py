@@ -40,6 +40,9 @@ class LMHead(Part):
     def bind(self, tensors, runtime) -> None:
         self.linear.set(tensors[self.spec.name])
 
+    def linears(self) -> list:
+        return [self.linear]
+
     def forward(self, ctx, h: torch.Tensor, m: int) -> torch.Tensor:
         out = ctx.workspace.get("head.logits", (m, self.spec.vocab_size), torch.float32)
         p = self.linear.forward(ctx, h, m, out=out)

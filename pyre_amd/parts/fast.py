@@ -113,8 +113,6 @@ DECODE_TARGET_WAVES = 1024
 #: a split takes at least this many keys (two chunks)
 DECODE_MIN_KEYS_PER_SPLIT = 64
 DECODE_MAX_SPLITS = 128
-#: sizes (requests) at which decode steps are captured in HIP graphs
-DECODE_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64)
 
 
 def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
@@ -133,31 +131,30 @@ def attention(mixer, ctx, q, o, cache) -> bool:
     from pyre_amd.hip import ops
 
     s = mixer.spec
-    if ctx.dtype != torch.bfloat16 or cache.k.dtype != torch.bfloat16:
+    k_pages, v_pages = cache["k"], cache["v"]
+    if ctx.dtype != torch.bfloat16 or k_pages.dtype != torch.bfloat16:
         return False
     if not ctx.runtime.options.get("mfma_attention", True):
         return False
     if not ops.attn_mfma_supports(s.head_dim, cache.page_size, s.num_heads, s.num_kv_heads):
         return False
     hb = ctx.host
-    n_dec, n_tiles = len(hb.decode_tokens), len(hb.prefill_tiles)
+    dec, tiles = hb.arrays["attention.decode_tokens"], hb.arrays["attention.prefill_tiles"]
+    n_dec, n_tiles = len(dec), len(tiles)
     if n_dec:
-        # The split is chosen from rounded-up sizes (requests to the next captured-step
-        # size, context to a power of two of pages), so that a step gives bit for bit the
-        # same result whether it runs eagerly or as a replayed graph at those sizes.
-        rows = next((b for b in DECODE_ROW_BUCKETS if b >= n_dec), n_dec)
-        pages = max(1, -(-hb.max_decode_ctx // cache.page_size))
-        span = max(8, 1 << (pages - 1).bit_length()) * cache.page_size
+        # The split is chosen from the step's rounded sizes, so that a step gives bit for bit
+        # the same result whether it runs eagerly or as a replayed graph at those sizes.
+        rows, span = hb.decode_shape()
         nsplits = ctx.runtime.options.get("decode_splits") or decode_splits(
             rows, s.num_heads, s.num_kv_heads, span, cache.window,
             ctx.runtime.options.get("decode_target_waves", DECODE_TARGET_WAVES))
         acc = ctx.workspace.get("attn.part_acc", (n_dec, s.num_heads, nsplits, s.head_dim), torch.float32)
         ml = ctx.workspace.get("attn.part_ml", (n_dec, s.num_heads, nsplits, 2), torch.float32)
-        ops.attn_decode_bf16(q, o, cache.k, cache.v, ctx.decode_tokens, n_dec, ctx.positions,
+        ops.attn_decode_bf16(q, o, k_pages, v_pages, ctx.arrays["attention.decode_tokens"], n_dec, ctx.positions,
                              ctx.seq_of_token, cache.table, acc, ml, nsplits, s.num_heads, s.num_kv_heads,
                              s.head_dim, cache.page_size, mixer.scale, cache.window)
     if n_tiles:
-        ops.attn_prefill_bf16(q, o, cache.k, cache.v, ctx.prefill_tiles, n_tiles, ctx.positions,
+        ops.attn_prefill_bf16(q, o, k_pages, v_pages, ctx.arrays["attention.prefill_tiles"], n_tiles, ctx.positions,
                               ctx.seq_of_token, cache.table, s.num_heads, s.num_kv_heads, s.head_dim,
                               cache.page_size, mixer.scale, cache.window)
     return True

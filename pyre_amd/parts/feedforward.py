@@ -29,6 +29,9 @@ class SwiGLU(FeedForward):
         self.gate_up.set(torch.cat([tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]], dim=0))
         self.down.set(tensors[f"{p}.down_proj.weight"])
 
+    def linears(self) -> list:
+        return [self.gate_up, self.down]
+
     def forward(self, ctx, h):
         n = ctx.n_tokens
         act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)

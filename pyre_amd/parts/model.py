@@ -40,6 +40,18 @@ class LayeredModel(Part):
                 seen.setdefault(s.name, s)
         return list(seen.values())
 
+    def linears(self) -> list:
+        return [lin for p in self.parts() for lin in p.linears()]
+
+    def step_arrays(self) -> list:
+        """The arrays that the mixers ask of every step, each name once."""
+        seen = {}
+        for layer in self.layers:
+            mixer = getattr(layer, "mixer", None)
+            for spec in (mixer.step_arrays() if mixer is not None else []):
+                seen.setdefault(spec.name, spec)
+        return list(seen.values())
+
     def cache_specs(self) -> list:
         """What each entry of the order keeps; None for an entry that keeps nothing
         or reads another entry's cache."""

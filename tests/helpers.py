@@ -28,6 +28,17 @@ def make_engine(folder, dtype: str, **kw):
     return Engine.from_folder(folder, EngineConfig(**args))
 
 
+def make_engine_from_state(config, state, dtype: str, **kw):
+    """The same for tensors that are already on the device (shapes too large for a file)."""
+    from pyre_amd.config.engine import EngineConfig
+    from pyre_amd.engine.engine import Engine
+
+    args = dict(dtype=dtype, page_size=16, max_cached_tokens=1024, max_num_seqs=8,
+                max_num_batched_tokens=1024, use_graphs=False)
+    args.update(kw)
+    return Engine.from_state(config, dict(state), EngineConfig(**args))
+
+
 def replay(engine, steps) -> dict:
     """steps: [(entries, end)] with entries = [(rid, tokens, want)].
     Returns {(rid, position): logits row (CPU float32)}."""
@@ -57,7 +68,7 @@ def replay(engine, steps) -> dict:
 
 def plain_logits(plain, ids, rounding=None) -> torch.Tensor:
     cfg, w = plain
-    return P.forward(w, cfg, ids, rounding=rounding).float()
+    return P.forward(w, cfg, ids, rounding=rounding).float().cpu()
 
 
 def first_bad(got: dict, want: dict[object, torch.Tensor], tol: float):

@@ -1,9 +1,11 @@
 """A plain, slow Qwen2 forward pass: whole sequences, no cache, one function per
-part, written from the reference's formulas (each function cites file:line of
-/root/reference). It shares no code with ``pyre_amd``: it reads ``config.json``
-with ``json`` and the weights with ``safetensors`` itself.
+part, written from the reference's formulas (each function cites file:line of the
+reference repository, pyre/model.py and its neighbours). It shares no code with
+``pyre_amd``: it reads ``config.json`` with ``json`` and the weights with
+``safetensors`` itself.
 
-Everything runs on the CPU in ``dtype`` (float64 by default: the engine's float32
+Everything runs where the weights lie (the CPU, unless a test moves them: the shapes of
+real models are too slow there) in ``dtype`` (float64 by default: the engine's float32
 path is then compared with something more exact than itself). ``rounding`` emulates
 a 16-bit engine: the values that such an engine stores in 16 bits (normed rows,
 rotated queries and keys, values, attention output, gated activations) are rounded
@@ -103,8 +105,8 @@ def causal_attention(q, k, v, scale: float, window: int = 0) -> torch.Tensor:
     than window-1 positions back."""
     S = q.shape[1]
     scores = torch.matmul(q, k.transpose(-1, -2)) * scale
-    i = torch.arange(S).unsqueeze(1)
-    j = torch.arange(S).unsqueeze(0)
+    i = torch.arange(S, device=q.device).unsqueeze(1)
+    j = torch.arange(S, device=q.device).unsqueeze(0)
     hidden = j > i
     if window > 0:
         hidden = hidden | (j < i - window + 1)
@@ -152,10 +154,12 @@ def decoder_layer(x, w: dict, i: int, cfg: dict, cos, sin, rnd) -> torch.Tensor:
 
 def forward(w: dict, cfg: dict, ids, rounding=None, return_hidden: bool = False):
     """pyre/model.py:188-201 without a cache: token ids (S,) -> logits (S, vocab)."""
-    ids = torch.as_tensor(ids, dtype=torch.long)
+    table = w["model.embed_tokens.weight"]
+    ids = torch.as_tensor(ids, dtype=torch.long, device=table.device)
     rnd = _rounder(rounding)
-    x = embed(ids, w["model.embed_tokens.weight"])
+    x = embed(ids, table)
     cos, sin = rope_tables(len(ids), cfg["head_dim"], cfg["rope_theta"], x.dtype)
+    cos, sin = cos.to(x.device), sin.to(x.device)
     hidden = []
     for i in range(cfg["num_hidden_layers"]):
         x = decoder_layer(x, w, i, cfg, cos, sin, rnd)

@@ -8,7 +8,12 @@ import random
 import pytest
 
 from pyre_amd.cache import RELEASED, CacheManager, OutOfPages, PageAllocator
-from pyre_amd.parts.base import KVCacheSpec, StateCacheSpec
+from pyre_amd.parts.base import PagedCacheSpec, PagedTensorSpec, StateCacheSpec
+
+
+def KVCacheSpec(nkv, hd, window=0):
+    return PagedCacheSpec((PagedTensorSpec("k", (nkv, hd), 1), PagedTensorSpec("v", (nkv, hd), 2)), window)
+
 
 FULL = KVCacheSpec(2, 16)
 WIN = KVCacheSpec(2, 16, window=40)
@@ -132,7 +137,8 @@ def test_layers_with_the_same_needs_share_a_group():
     m = CacheManager(specs, 16, 10, 4, 512)
     assert [g.entries for g in m.page_groups] == [[0, 2], [1, 5]]
     assert [g.entries for g in m.state_groups] == [[4, 6]]
-    assert m.group_of_entry == {0: ("kv", 0), 2: ("kv", 0), 1: ("kv", 1), 5: ("kv", 1), 4: ("state", 0), 6: ("state", 0)}
+    assert m.group_of_entry == {0: ("paged", 0), 2: ("paged", 0), 1: ("paged", 1), 5: ("paged", 1), 4: ("state", 0),
+                                6: ("state", 0)}
     assert m.page_groups[1].layer_index(5) == 1
     assert m.bytes_per_page(2) == 2 * (2 * 2 * 16 * 16 * 2) * 2
 
@@ -217,3 +223,154 @@ def test_no_page_lost_held_twice_or_freed_twice(seed):
     for rid in list(live):
         m.free_request(rid)
     assert all(g.allocator.num_used == 0 for g in m.page_groups) and m.slots.num_used == 0
+
+
+# --- what a page holds is the mixer's business ------------------------------------------
+
+def test_a_page_holds_whatever_the_description_says():
+    import torch
+
+    latent = PagedCacheSpec((PagedTensorSpec("latent", (24,)), PagedTensorSpec("gate", (3, 2), token_axis=2, dtype="float32")))
+    assert PagedTensorSpec("k", (2, 16), 1).page_shape(8) == (2, 8, 16)
+    assert PagedTensorSpec("v", (2, 16), 2).page_shape(8) == (2, 16, 8)
+    assert PagedTensorSpec("latent", (24,)).page_shape(8) == (8, 24)
+    m = CacheManager([latent, FULL, latent], 8, 5, 2, 64)
+    assert [g.entries for g in m.page_groups] == [[0, 2], [1]]
+    m.materialize("cpu", torch.bfloat16)
+    g = m.page_groups[0]
+    assert g.tensors["latent"].shape == (2, 5, 8, 24) and g.tensors["latent"].dtype == torch.bfloat16
+    assert g.tensors["gate"].shape == (2, 5, 3, 2, 8) and g.tensors["gate"].dtype == torch.float32
+    assert set(m.page_groups[1].tensors) == {"k", "v"}
+    assert m.bytes_per_page(2) == 2 * 8 * (24 * 2 + 6 * 4) + 2 * (2 * 16 * 8 * 2)
+    with pytest.raises(ValueError, match="name of its own"):
+        PagedCacheSpec((PagedTensorSpec("x", (4,)), PagedTensorSpec("x", (4,))))
+    with pytest.raises(ValueError, match="token_axis"):
+        PagedTensorSpec("x", (4,), token_axis=2)
+
+
+def test_unreserve_gives_back_what_a_step_that_did_not_run_had_taken():
+    m = CacheManager([FULL, WIN], 16, 12, 2, 512)
+    m.add_request("a")
+    m.reserve("a", 20)
+    m.commit("a", 20)
+    before = [list(m.block_table("a", g)) for g in range(2)]
+    m.reserve("a", 70)                 # four more pages in each group
+    assert m.page_groups[0].allocator.num_used == 6
+    m.unreserve("a")
+    assert [list(m.block_table("a", g)) for g in range(2)] == before
+    assert m.page_groups[0].allocator.num_used == 2 and m.length("a") == 20
+    assert (m.block_table_array("a", 0)[2:] == RELEASED).all()
+    m.check_invariants()
+    m.reserve("a", 70)
+    m.commit("a", 70)                  # and the request goes on as if nothing had happened
+    m.check_invariants()
+    m.free_request("a")
+    assert m.page_groups[0].allocator.num_used == 0 and m.page_groups[1].allocator.num_used == 0
+
+
+def test_poison_mode_marks_what_nobody_holds():
+    """NaN wherever no live request holds the memory, zero in a page just taken, under a
+    random sequence of requests with a window (on the CPU: torch does the filling)."""
+    import torch
+
+    rng = random.Random(5)
+    m = CacheManager([FULL, WIN, StateCacheSpec((3,))], 16, 14, 3, 400, poison=True)
+    m.materialize("cpu", torch.float32)
+    assert all(torch.isnan(t).all() for g in m.page_groups for t in g.tensors.values())
+    assert torch.isnan(m.state_groups[0].tensor[:, :3]).all()
+    live = {}
+    for step in range(300):
+        if live and rng.random() < 0.25:
+            rid = rng.choice(list(live))
+            m.free_request(rid)
+            del live[rid]
+        elif len(live) < 3 and rng.random() < 0.5:
+            rid = step
+            slot = m.add_request(rid)
+            assert (m.state_groups[0].tensor[:, slot] == 0).all()
+            live[rid] = 0
+        elif live:
+            rid = rng.choice(list(live))
+            n = rng.randrange(1, 40)
+            try:
+                m.reserve(rid, n)
+            except (OutOfPages, ValueError):
+                continue
+            # the request writes its tokens (here: ones) and commits
+            for gi, g in enumerate(m.page_groups):
+                for pos in range(live[rid], live[rid] + n):
+                    page = m.block_table(rid, gi)[pos // 16]
+                    g.tensors["k"][:, page, :, pos % 16] = 1.0
+            m.commit(rid, n)
+            live[rid] += n
+        m.check_invariants()
+        for gi, g in enumerate(m.page_groups):
+            held = {p for r in live for p in m.block_table(r, gi) if p != RELEASED}
+            for p in range(g.num_pages):
+                nan = torch.isnan(g.tensors["k"][:, p])
+                assert (not nan.any()) if p in held else nan.all(), (step, gi, p)
+        free_slots = set(range(3)) - {m.slot(r) for r in live}
+        for sl in free_slots:
+            assert torch.isnan(m.state_groups[0].tensor[:, sl]).all()
+
+
+# --- a step is prepared all or nothing ---------------------------------------------------
+
+def _snapshot(m):
+    return ({r: (m.slot(r), m.length(r), [list(m.block_table(r, g)) for g in range(len(m.page_groups))])
+             for r in m.live_requests},
+            [g.allocator.num_free for g in m.page_groups], m.slots.num_free)
+
+
+def test_a_step_that_cannot_be_prepared_leaves_the_cache_as_it_was():
+    from pyre_amd.engine.batch import Entry, prepare_step
+
+    m = CacheManager([FULL, WIN], 16, 8, 3, 256)
+    hb, shape = prepare_step([Entry("a", [1] * 40, [39])], m, 100)
+    assert shape is None and hb.n_tokens == 40
+    m.commit("a", 40)
+    before = _snapshot(m)
+    # the second entry runs out of pages: "a" keeps no reservation, "b" and "c" are not admitted
+    with pytest.raises(OutOfPages):
+        prepare_step([Entry("a", [1] * 20, []), Entry("b", [2] * 60, []), Entry("c", [3] * 30, [])], m, 100)
+    assert _snapshot(m) == before
+    m.check_invariants()
+    # reserve itself fails (the longest length) after others were reserved
+    roomy = CacheManager([FULL], 16, 40, 3, 100)
+    prepare_step([Entry("a", [1] * 40, [])], roomy, 100)
+    roomy.commit("a", 40)
+    was = _snapshot(roomy)
+    with pytest.raises(ValueError, match="limit"):
+        prepare_step([Entry("b", [2] * 10, []), Entry("a", [1] * 70, [])], roomy, 100)
+    assert _snapshot(roomy) == was
+    # laying out fails after everything was reserved: a token outside the vocabulary
+    with pytest.raises(ValueError, match="vocabulary"):
+        prepare_step([Entry("a", [1, 2], []), Entry("b", [5, 100], [])], m, 100)
+    assert _snapshot(m) == before
+    with pytest.raises(ValueError, match="twice"):
+        prepare_step([Entry("b", [1], []), Entry("b", [2], [])], m, 100)
+    with pytest.raises(ValueError, match="wanted place"):
+        prepare_step([Entry("b", [1, 2], [2])], m, 100)
+    # no slot for a fourth request
+    for r in "bc":
+        prepare_step([Entry(r, [1], [])], m, 100)
+        m.commit(r, 1)
+    before = _snapshot(m)
+    with pytest.raises(OutOfPages, match="slot"):
+        prepare_step([Entry("a", [1], []), Entry("d", [1], [])], m, 100)
+    assert _snapshot(m) == before
+    m.check_invariants()
+    # and a retry with a batch that fits goes through
+    hb, shape = prepare_step([Entry("a", [7], [0]), Entry("b", [8], [0])], m, 100, graph_max_rows=64)
+    assert shape == (2, 8) and hb.n_single == 2 and hb.decode_shape() == (2, 8 * 16)
+
+
+def test_rounding_of_decode_steps_is_idempotent():
+    from pyre_amd.engine.batch import DECODE_ROW_BUCKETS, round_decode_shape
+
+    for n in range(1, 70):
+        for pages in (1, 7, 8, 9, 200, 256, 257):
+            rows, width = round_decode_shape(n, pages)
+            assert rows >= n and width >= pages and width & (width - 1) == 0
+            assert round_decode_shape(rows, width) == (rows, width)
+            assert rows in DECODE_ROW_BUCKETS or n > DECODE_ROW_BUCKETS[-1]

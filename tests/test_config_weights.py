@@ -174,6 +174,52 @@ def test_one_error_lists_everything_that_is_wrong(tmp_path):
         adopt_state(state, specs, "cpu", torch.float32)
 
 
+def test_wrong_class_of_element_type_is_named(tmp_path):
+    """Integers under a weight's name are refused at load, by name, in the same one error
+    as everything else that is wrong (not later, inside a kernel call)."""
+    from safetensors.torch import save_file
+
+    cfg = preset("tiny-b")
+    specs = model_tensor_specs(cfg)
+    state = random_state(specs, 0)
+    state["model.layers.2.mlp.down_proj.weight"] = torch.zeros(96, 256, dtype=torch.int64)
+    state["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(96, dtype=torch.int8)
+    state["model.norm.weight"] = torch.zeros(95)
+    cfg.save(tmp_path)
+    save_file(state, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_weights(tmp_path, specs, "cpu", torch.bfloat16)
+    assert {n for n, _, _ in e.value.wrong_dtype} == {"model.layers.2.mlp.down_proj.weight",
+                                                      "model.layers.0.self_attn.q_proj.bias"}
+    assert [n for n, _, _ in e.value.wrong_shape] == ["model.norm.weight"]
+    assert "wrong element type" in str(e.value) and "I64" in str(e.value) and "floating-point" in str(e.value)
+    with pytest.raises(WeightsError) as e2:
+        adopt_state(state, specs, "cpu", torch.float32)
+    assert len(e2.value.wrong_dtype) == 2
+
+
+def test_tied_head_that_the_file_also_holds_must_equal_the_embedding(tmp_path):
+    from safetensors.torch import save_file
+
+    cfg = preset("tiny-a")                                       # tie_word_embeddings
+    specs = model_tensor_specs(cfg)
+    state = random_state(specs, 0)
+    assert "lm_head.weight" not in state
+    state["lm_head.weight"] = state["model.embed_tokens.weight"].clone()
+    cfg.save(tmp_path)
+    save_file(state, str(tmp_path / "model.safetensors"))
+    w = load_weights(tmp_path, specs, "cpu", torch.bfloat16)      # equal: accepted, and one memory
+    assert w["lm_head.weight"].data_ptr() == w["model.embed_tokens.weight"].data_ptr()
+    state["lm_head.weight"][3, 5] += 1.0
+    save_file(state, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_weights(tmp_path, specs, "cpu", torch.bfloat16)
+    assert e.value.tied_mismatch == [("lm_head.weight", "model.embed_tokens.weight")]
+    assert "tied but different" in str(e.value)
+    with pytest.raises(WeightsError):
+        adopt_state(state, specs, "cpu", torch.float32)
+
+
 def test_no_safetensors(tmp_path):
     preset("tiny-a").save(tmp_path)
     with pytest.raises(FileNotFoundError, match="safetensors"):      # pyre/loader.py:47-48

@@ -120,6 +120,101 @@ def test_sampling_does_not_depend_on_batch_mates(model_dirs):
     assert sched.run()[sid] != together[1]
 
 
+def _check_against_plain_sampler(plain, prompt, tokens, temperature, seed, seq_id, tol):
+    """Every token of a generated sequence against the plain implementation, given the
+    engine's own tokens before it: the plain logits of prompt + tokens[:k], the plain
+    sampler with the same uniform number. A token may differ only where that number lies
+    within ``tol`` of an edge of the chosen token's interval of the cumulative distribution
+    (greedy: where the two largest logits are within ``tol`` of the logit scale). Returns
+    how many did."""
+    from pyre_amd.sampling.rng import uniform
+
+    cfg, w = plain
+    ids, near = list(prompt), 0
+    for k, tok in enumerate(tokens):
+        row = P.forward(w, cfg, ids)[-1]
+        if temperature > 0:
+            u = uniform(seed, seq_id, k)
+            twin = P.sample_inverse_cdf(row, temperature, u)
+            if twin != tok:
+                c = torch.cumsum(torch.softmax(row.double() / temperature, -1), -1)
+                lo, hi = (float(c[tok - 1]) if tok > 0 else 0.0), float(c[tok])
+                margin = 0.0 if lo <= u < hi else min(abs(u - lo), abs(u - hi))
+                assert margin < tol, f"token {k}: {tok} drawn, the plain sampler draws {twin}; u={u} is {margin:.2e} outside [{lo}, {hi})"
+                near += 1
+        else:
+            twin = int(row.argmax())
+            if twin != tok:
+                margin = float((row[twin] - row[tok]) / row.abs().max())
+                assert margin < tol, f"token {k}: {tok} chosen, plain argmax is {twin}, margin {margin:.2e}"
+                near += 1
+        ids.append(tok)
+    return near
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_config_b_workload_against_the_plain_sampler(dtype, model_dirs, plain_models):
+    """Six prompts of 3 to 120 tokens arrive one every other step, so that prompt portions
+    of 32 share steps with decoding requests; temperature 0.8 with a seeded stream, 24 new
+    tokens each, pages of 8 tokens. Every token is the plain sampler's on the plain logits
+    with the same uniform number (`tests/test_scheduler.py:20-64` of the reference compares
+    batched with alone; here both are compared with the trusted path)."""
+    import random
+
+    from pyre_amd.api import Scheduler
+
+    plain = plain_models["tiny-b"]
+    rng = random.Random(1)
+    prompts = [random_ids(1000, rng.randint(3, 120), seed=10 + i) for i in range(6)]
+    eng = _load(model_dirs["tiny-b"], dtype, page_size=8, max_cached_tokens=1024, prefill_chunk=32,
+                max_num_batched_tokens=40)
+    sched = Scheduler(eng, max_batch=4)
+    ids = []
+    mixed = 0
+    for p in prompts:
+        ids.append(sched.add_request(p, 24, temperature=0.8, seed=1))
+        for _ in range(2):
+            plan_before = len(sched.running)
+            sched.step()
+            mixed += plan_before > 0
+    out = sched.run()
+    assert mixed > 0 and eng.cache.page_groups[0].allocator.num_used == 0
+    assert all(len(out[i]) == 24 for i in ids)
+    tol = 1e-5 if dtype == "float32" else 4e-2
+    near = sum(_check_against_plain_sampler(plain, p, out[i], 0.8, 1, i, tol) for p, i in zip(prompts, ids))
+    assert near <= (1 if dtype == "float32" else 8), f"{near} of 144 tokens were decided by rounding"
+
+
+@pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
+                                                ("tiny-b", "float32", True), ("tiny-c", "float32", True)])
+def test_many_live_requests_generate_the_plain_tokens(model, dtype, graphs, model_dirs, plain_models):
+    """20 and then 50 requests of unequal lengths decode together (steps of 17 to 64 rows,
+    padded to their captured sizes), some greedy, some sampled; every token against the
+    plain implementation."""
+    from pyre_amd.api import Scheduler
+
+    plain = plain_models[model]
+    vocab = plain[0]["vocab_size"]
+    eng = _load(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=64, max_cached_tokens=64 * 96,
+                max_num_batched_tokens=512, prefill_chunk=64)
+    tol = 1e-5 if dtype == "float32" else 4e-2
+    for count in (20, 50):
+        prompts = [random_ids(vocab, 3 + (11 * i) % 47, seed=count + i) for i in range(count)]
+        new = [6 + (5 * i) % 9 for i in range(count)]         # they end at different steps: the batch shrinks
+        sched = Scheduler(eng, max_batch=64)
+        ids = [sched.add_request(p, n, temperature=0.7 if i % 3 == 0 else 0.0, seed=9) for i, (p, n) in
+               enumerate(zip(prompts, new))]
+        out = sched.run()
+        assert eng.cache.page_groups[0].allocator.num_used == 0
+        near = 0
+        for i, (p, sid) in enumerate(zip(prompts, ids)):
+            assert len(out[sid]) == new[i]
+            near += _check_against_plain_sampler(plain, p, out[sid], 0.7 if i % 3 == 0 else 0.0, 9, sid, tol)
+        assert near <= (1 if dtype == "float32" else count), f"{near} tokens were decided by rounding"
+    if graphs:
+        assert eng.graph_replays > 0
+
+
 def test_preemption_recomputes_and_gives_the_same_tokens(model_dirs):
     """With so few pages that running requests cannot all grow, the latest one is
     preempted and recomputed; tokens equal those of a roomy pool."""

@@ -76,6 +76,37 @@ def test_add_rmsnorm(dtype, hidden):
     assert torch.allclose(o2.double(), want[[6, 2]], atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [1028, 1536, 3584, 5120, 8192])
+def test_add_rmsnorm_row_does_not_depend_on_row_count(dtype, hidden):
+    """A wide row normed in a step of few rows (the 1024-thread form) and in a step of many
+    (the 256-thread form) gives the same bits: the sum of squares is added in one order."""
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+
+    many, few, eps = 200, 5, 1e-6
+    resid = rnd(many, hidden, seed=1, scale=3.0)
+    delta = rnd(2, many, hidden, seed=2)
+    gain = rnd(hidden, seed=4, dtype=DT[dtype]) + 1
+    pick = [0, 77, 128, 150, 199][:few]
+    out_many = torch.empty(many, hidden, device=DEV, dtype=DT[dtype])
+    r_many = resid.clone()
+    ops.add_rmsnorm(r_many, Partials(delta), gain, eps, out_many)
+    r_few = resid[pick].clone()
+    out_few = torch.empty(few, hidden, device=DEV, dtype=DT[dtype])
+    ops.add_rmsnorm(r_few, Partials(delta[:, pick].contiguous()), gain, eps, out_few)
+    assert torch.equal(r_few, r_many[pick])
+    assert torch.equal(out_few, out_many[pick])
+    # the final norm's gather form: few listed rows of a long residual, and many of them
+    rows_few, rows_many = i32(pick), i32(list(range(many - 1, -1, -1)))
+    g_few = torch.empty(few, hidden, device=DEV, dtype=DT[dtype])
+    g_many = torch.empty(many, hidden, device=DEV, dtype=DT[dtype])
+    ops.add_rmsnorm(resid.clone(), Partials(delta), gain, eps, g_few, rows=rows_few)
+    ops.add_rmsnorm(resid.clone(), Partials(delta), gain, eps, g_many, rows=rows_many)
+    assert torch.equal(g_few, out_many[pick])
+    assert torch.equal(g_many, out_many.flip(0))
+
+
 @pytest.mark.parametrize("adt,wdt", [("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")])
 @pytest.mark.parametrize("m,n,k", [(1, 37, 50), (5, 130, 257), (77, 200, 64), (130, 65, 1000)])
 def test_gemm_generic(adt, wdt, m, n, k):
@@ -286,7 +317,7 @@ def test_attn_decode_mfma(nq, nkv, hd, page, window, nsplits):
 @pytest.mark.parametrize("window", [0, 50])
 def test_attn_prefill_mfma(nq, nkv, hd, page, window, form):
     ops = _ops()
-    from pyre_amd.engine.batch import TILE
+    from pyre_amd.parts.attention import TILE
 
     ctx_lens, q_lens = [2, 40, 97, 700, 1100], [2, 40, 33, 3, 600]
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=4)
@@ -371,6 +402,44 @@ def test_sample_inverse_cdf():
     flat = torch.zeros(1, v, device=DEV)
     ops.sample(flat, torch.tensor([1.0], device=DEV), torch.tensor([0.5], device=DEV), out2)
     assert abs(int(out2[0]) - v // 2) <= 1
+
+
+def test_sample_at_slice_edges_and_against_the_plain_sampler():
+    """Targets on and beside the edges of the threads' slices (all sums exact: equal logits,
+    2 tokens per slice), then many random rows against the float64 twin wherever the drawn
+    number is not within rounding of an edge of the chosen token's interval."""
+    import plain_qwen2 as P
+
+    ops = _ops()
+    v = 2048
+    us = [0.5, (1024 - 0.5) / v, (1024 + 0.5) / v, 0.0, (v - 0.25) / v, 1 / v, 63.5 / v, 64 / v, 128 / v]
+    want = [1024, 1023, 1024, 0, v - 1, 1, 63, 64, 128]
+    flat = torch.zeros(len(us), v, device=DEV)
+    out = torch.zeros(len(us), dtype=torch.int32, device=DEV)
+    ops.sample(flat, torch.ones(len(us), device=DEV), torch.tensor(us, device=DEV), out)
+    assert out.tolist() == want
+    assert [P.sample_inverse_cdf(flat[0].cpu(), 1.0, u) for u in us] == want
+    # only a few tokens can be drawn at all, the rest underflow to zero probability
+    spiky = torch.full((3, 5000), -1e4, device=DEV)
+    spiky[:, 17] = spiky[:, 3000] = spiky[:, 4999] = 0.0
+    out3 = torch.zeros(3, dtype=torch.int32, device=DEV)
+    ops.sample(spiky, torch.ones(3, device=DEV), torch.tensor([0.2, 0.5, 0.99], device=DEV), out3)
+    assert out3.tolist() == [17, 3000, 4999]
+    m, v = 256, 15013
+    logits = rnd(m, v, seed=21, scale=3.0)
+    temps = [0.3 + 0.005 * i for i in range(m)]
+    draws = [random.Random(1000 + i).random() for i in range(m)]
+    out = torch.zeros(m, dtype=torch.int32, device=DEV)
+    ops.sample(logits, torch.tensor(temps, device=DEV), torch.tensor(draws, device=DEV), out)
+    got, rows, close = out.tolist(), logits.cpu(), 0
+    for i in range(m):
+        c = torch.cumsum(torch.softmax(rows[i].double() / temps[i], -1), -1)
+        twin = P.sample_inverse_cdf(rows[i], temps[i], draws[i])
+        if got[i] != twin:
+            edge = c[min(got[i], twin)].item()
+            assert abs(got[i] - twin) == 1 and abs(edge - draws[i]) < 1e-5, (i, got[i], twin, draws[i], edge)
+            close += 1
+    assert close <= 3
 
 
 # ----------------------------------------------------------------------------- weight-streaming products

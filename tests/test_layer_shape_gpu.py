@@ -1,44 +1,61 @@
-"""One layer with the sizes of the Qwen2.5-7B shape (width 3584, 28 query / 4
-key-value heads of 128, feed-forward 18944; a small vocabulary so that the plain
-implementation stays quick) against the plain implementation. The tiny models never
-reach the code that only real sizes take: weight-streaming products with many column
-tiles and eight-way splits along k, the library products of a long portion, attention
-with seven query heads per key/value head, decode steps replayed from HIP graphs."""
+"""Two layers with the sizes of the Qwen2.5-7B shape (width 3584, 28 query / 4 key-value
+heads of 128, feed-forward 18944) and its whole vocabulary of 152,064 against the plain
+implementation. The tiny models never reach the code that only real sizes take:
+weight-streaming products with many column tiles and splits along k, the head's product
+over 152,064 rows in slices of 64 requests, the library products of a long portion,
+attention with seven query heads per key/value head, decode steps of 17 to 64 requests
+replayed from HIP graphs at their padded sizes.
+
+The weights are drawn on the device (a file of this shape would take 3 GB) and the plain
+implementation runs there too, in float64 (on the CPU it would take minutes)."""
 
 from __future__ import annotations
 
 import pytest
 import torch
 
-from helpers import TOL, first_bad, make_engine, plain_logits, random_ids, replay
+import plain_qwen2 as P
+from helpers import TOL, first_bad, make_engine_from_state, plain_logits, random_ids, replay
 
 pytestmark = pytest.mark.gpu
 
+DEV = "cuda:0"
+
 
 @pytest.fixture(scope="module")
-def layer_model(tmp_path_factory):
-    import plain_qwen2 as P
+def layers_7b():
     from pyre_amd.config import preset
-    from pyre_amd.weights import write_random_model
+    from pyre_amd.weights import model_tensor_specs, random_state
 
-    cfg = preset("qwen2.5-7b", num_hidden_layers=1, vocab_size=1536)
-    d = tmp_path_factory.mktemp("layer7b")
-    write_random_model(d, cfg, seed=5, std=0.02, gain_std=0.1)
-    return d, (P.read_config(d), P.read_weights(d))
+    cfg = preset("qwen2.5-7b", num_hidden_layers=2)
+    assert cfg.vocab_size == 152064 and cfg.hidden_size == 3584 and cfg.intermediate_size == 18944
+    state = random_state(model_tensor_specs(cfg), seed=5, std=0.02, gain_std=0.1, dtype="bfloat16", device=DEV)
+    plain_cfg = {k: getattr(cfg, k) for k in ("hidden_size", "intermediate_size", "num_hidden_layers",
+                                              "num_attention_heads", "num_key_value_heads", "vocab_size",
+                                              "rms_norm_eps", "rope_theta", "tie_word_embeddings", "head_dim")}
+    weights = {n: t.to(torch.float64) for n, t in state.items()}
+    yield cfg, state, (plain_cfg, weights)
+    weights.clear()
+    state.clear()
+    torch.cuda.empty_cache()
+
+
+def _want(plain, reqs, dtype):
+    rounding = torch.bfloat16 if dtype == "bfloat16" else None
+    return {r: plain_logits(plain, ids, rounding) for r, ids in reqs.items()}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_one_layer_of_the_7b_shape(dtype, layer_model):
-    folder, plain = layer_model
-    vocab = plain[0]["vocab_size"]
+def test_two_layers_of_the_7b_shape_with_the_whole_vocabulary(dtype, layers_7b):
+    cfg, state, plain = layers_7b
+    vocab = cfg.vocab_size
     reqs = {"a": random_ids(vocab, 150, 1), "b": random_ids(vocab, 90, 2), "c": random_ids(vocab, 41, 3)}
-    rounding = torch.bfloat16 if dtype == "bfloat16" else None
-    want = {r: plain_logits(plain, ids, rounding) for r, ids in reqs.items()}
-    eng = make_engine(folder, dtype, use_graphs=True, max_cached_tokens=512, max_num_seqs=4)
+    want = _want(plain, reqs, dtype)
+    eng = make_engine_from_state(cfg, state, dtype, use_graphs=True, max_cached_tokens=512, max_num_seqs=4)
     a, b, c = reqs["a"], reqs["b"], reqs["c"]
     steps = [
         ([("a", a[:100], [0, 63, 99])], []),                       # a long portion: library products in 16 bits
-        ([("a", a[100:130], [29]), ("b", b[:70], [69])], []),      # two portions in one step
+        ([("a", a[100:130], [29]), ("b", b[:70], list(range(70)))], []),   # two portions; 71 rows of logits at once
     ]
     # decode a and b token by token beside portions of c, then c alone
     for i in range(20):
@@ -52,3 +69,37 @@ def test_one_layer_of_the_7b_shape(dtype, layer_model):
     assert bad is None, bad
     assert eng.graph_replays > 0
     assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_many_requests_at_the_7b_shape(dtype, layers_7b):
+    """64, then 33, then 17 live requests, one token each per step, from HIP graphs: the
+    weight-streaming products with two to four tiles of rows, the fused SiLU-gate product of
+    17 to 64 rows, the decode attention's split rule at large batches, the head in slices."""
+    cfg, state, plain = layers_7b
+    vocab = cfg.vocab_size
+    lengths = [5 + (7 * i) % 29 for i in range(64)]              # contexts that cross page ends at different steps
+    reqs = {i: random_ids(vocab, n + 4, 100 + i) for i, n in enumerate(lengths)}
+    want = _want(plain, reqs, dtype)
+    eng = make_engine_from_state(cfg, state, dtype, use_graphs=True, max_cached_tokens=64 * 48, max_num_seqs=64,
+                                 max_num_batched_tokens=2048)
+    # prompts in two mixed steps, no logits; then four decode steps with fewer and fewer requests
+    steps = [([(i, reqs[i][:lengths[i]], []) for i in range(0, 40)], []),
+             ([(i, reqs[i][:lengths[i]], []) for i in range(40, 64)], [])]
+    live = list(range(64))
+    for k, keep in enumerate((64, 64, 33, 17)):
+        live = live[:keep]
+        steps.append(([(i, [reqs[i][lengths[i] + k]], [0]) for i in live], []))
+    got = replay(eng, steps)
+    assert len(got) == 64 + 64 + 33 + 17
+    bad, worst = first_bad(got, want, TOL[dtype])
+    assert bad is None, bad
+    # the same again: steps that ran eagerly at their padded sizes (64, 48 for 33, 24 for 17) are now replayed
+    for i in range(64):
+        eng.finish(i)
+    got2 = replay(eng, steps)
+    assert eng.graph_replays > 0
+    bad, worst = first_bad(got2, want, TOL[dtype])
+    assert bad is None, bad
+    for k in got:
+        assert torch.equal(got[k], got2[k]), f"{k}: a replayed step differs from the eager one"

@@ -27,26 +27,30 @@ class Rig:
         from pyre_amd.engine.context import MetaBuffers, Runtime
 
         self.dtype = DT[dtype]
+        from pyre_amd.parts.attention import STEP_ARRAYS
+
         self.cache = CacheManager(cache_specs, page_size, pages, seqs, max_len)
         self.cache.materialize(DEV, self.dtype)
-        self.meta = MetaBuffers(DEV, 512, seqs, [32 for _ in self.cache.page_groups])
+        self.arrays = list(STEP_ARRAYS)
+        self.meta = MetaBuffers(DEV, 512, seqs, [32 for _ in self.cache.page_groups], self.arrays)
         self.runtime = Runtime(DEV, self.dtype, max_len)
 
     def context(self, entries, vocab=1000):
         from pyre_amd.engine.batch import Entry, build_host_batch
-        from pyre_amd.engine.context import KVLayerView, StepContext
+        from pyre_amd.engine.context import PagedLayerView, StepContext
 
         es = [Entry(r, list(t), list(w)) for r, t, w in entries]
         for e in es:
             if e.rid not in self.cache:
                 self.cache.add_request(e.rid)
             self.cache.reserve(e.rid, len(e.tokens))
-        hb = build_host_batch(es, self.cache, vocab, table_width=32)
+        hb = build_host_batch(es, self.cache, vocab, table_width=32).attach(self.arrays)
         v = self.meta.upload(hb)
         ctx = StepContext(self.runtime, hb, hb.n_tokens, hb.n_seqs, len(hb.logit_rows), v["tokens"], v["positions"],
                           v["seq_of_token"], v["logit_rows"][:len(hb.logit_rows)], v["q_start"], v["ctx_len"],
-                          v["state_slots"], v["decode_tokens"], v["prefill_tiles"])
-        views = [KVLayerView(g.k[0], g.v[0], v[f"table{i}"], v[f"slots{i}"], g.page_size, g.spec.window)
+                          v["state_slots"], {a.name: v["x:" + a.name] for a in self.arrays})
+        views = [PagedLayerView({n: t[0] for n, t in g.tensors.items()}, v[f"table{i}"], v[f"slots{i}"], g.page_size,
+                                g.spec.window)
                  for i, g in enumerate(self.cache.page_groups)]
         return ctx, views, es
 
@@ -107,7 +111,8 @@ def attention_weights(H, nq, nkv, hd, seed):
 def test_attention_part(dtype, nq, nkv, hd, window):
     """Two requests, each fed in two portions and a single token, against the plain
     attention block over the whole sequences."""
-    from pyre_amd.parts.base import AttentionSpec, KVCacheSpec, RotarySpec, make_part
+    from pyre_amd.parts.attention import KVCacheSpec
+    from pyre_amd.parts.base import AttentionSpec, RotarySpec, make_part
 
     H, theta = 56, 1e4
     spec = AttentionSpec(H, nq, nkv, hd, RotarySpec(hd, theta, 256), "a", window=window)

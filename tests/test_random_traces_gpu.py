@@ -48,17 +48,25 @@ def random_trace(vocab: int, seed: int, max_live: int = 4, n_requests: int = 9):
 @pytest.mark.parametrize("seed", [0, 1, 2])
 @pytest.mark.parametrize("model,dtype", [("tiny-a", "float32"), ("tiny-c", "bfloat16"), ("tiny-b", "bfloat16"),
                                          ("tiny-d", "float32")])
-def test_random_trace(model, dtype, seed, model_dirs, plain_models):
+def test_random_trace(model, dtype, seed, model_dirs, plain_models, poison=False, page=16):
     plain = plain_models[model]
     reqs, steps = random_trace(plain[0]["vocab_size"], seed)
     rounding = torch.bfloat16 if dtype == "bfloat16" else None
     want = {r: plain_logits(plain, ids, rounding) for r, ids in reqs.items()}
     # four live requests of at most 160 tokens: 4 * 10 pages of 16, and not one more
-    eng = make_engine(model_dirs[model], dtype, num_pages=40, max_cached_tokens=None, max_num_seqs=4,
-                      max_num_batched_tokens=512, use_graphs=seed == 1)
+    eng = make_engine(model_dirs[model], dtype, num_pages=40 * 16 // page, page_size=page, max_cached_tokens=None,
+                      max_num_seqs=4, max_num_batched_tokens=512, use_graphs=seed == 1, debug_poison=poison)
     got = replay(eng, steps)
     assert got, "the trace asked for no logits"
     bad, worst = first_bad(got, want, TOL[dtype])
     assert bad is None, f"seed {seed}: {bad}"
     eng.cache.check_invariants()
     assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+@pytest.mark.parametrize("model,dtype,seed,page", [("tiny-c", "bfloat16", 1, 16), ("tiny-b", "float32", 0, 8),
+                                                   ("tiny-c", "bfloat16", 2, 32), ("tiny-d", "float32", 2, 16)])
+def test_random_trace_on_poisoned_pages(model, dtype, seed, page, model_dirs, plain_models):
+    """The same with every freed page and slot filled with NaN (and other page sizes): what a
+    request reads of memory it does not hold would show as NaN in its logits."""
+    test_random_trace(model, dtype, seed, model_dirs, plain_models, poison=True, page=page)

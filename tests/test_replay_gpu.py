@@ -11,7 +11,10 @@ from helpers import TOL, cut, first_bad, make_engine, plain_logits, random_ids, 
 
 pytestmark = pytest.mark.gpu
 
-CASES = [(m, d) for m in ("tiny-a", "tiny-b", "tiny-c", "tiny-d") for d in ("float32", "bfloat16")]
+#: (model, element type, page size): every shape on 16-token pages, and the shape whose workload
+#: is defined on 8-token pages (and a tied one) on those
+CASES = [(m, d, 16) for m in ("tiny-a", "tiny-b", "tiny-c", "tiny-d") for d in ("float32", "bfloat16")]
+CASES += [("tiny-b", "float32", 8), ("tiny-b", "bfloat16", 8), ("tiny-a", "float32", 8), ("tiny-c", "bfloat16", 32)]
 LENGTHS = {"a": 97, "b": 64, "c": 33, "d": 150}
 
 
@@ -37,11 +40,11 @@ def engines(model_dirs):
     return get
 
 
-@pytest.mark.parametrize("model,dtype", CASES)
-def test_whole(model, dtype, engines, plain_models):
+@pytest.mark.parametrize("model,dtype,page", CASES)
+def test_whole(model, dtype, page, engines, plain_models):
     plain = plain_models[model]
     reqs = _requests(plain[0]["vocab_size"])
-    eng = engines(model, dtype)
+    eng = engines(model, dtype, page_size=page)
     steps = [([(r, ids, list(range(len(ids))))], [r]) for r, ids in reqs.items()]
     got = replay(eng, steps)
     assert len(got) == sum(LENGTHS.values())
@@ -51,11 +54,11 @@ def test_whole(model, dtype, engines, plain_models):
     assert eng.cache.page_groups[0].allocator.num_used == 0
 
 
-@pytest.mark.parametrize("model,dtype", CASES)
-def test_tail_token_by_token(model, dtype, engines, plain_models):
+@pytest.mark.parametrize("model,dtype,page", CASES)
+def test_tail_token_by_token(model, dtype, page, engines, plain_models):
     plain = plain_models[model]
     reqs = _requests(plain[0]["vocab_size"])
-    eng = engines(model, dtype)
+    eng = engines(model, dtype, page_size=page)
     steps = []
     for r, ids in reqs.items():
         head = len(ids) - 32
@@ -68,11 +71,11 @@ def test_tail_token_by_token(model, dtype, engines, plain_models):
     assert eng.cache.page_groups[0].allocator.num_used == 0
 
 
-@pytest.mark.parametrize("model,dtype", CASES)
-def test_ragged_portions(model, dtype, engines, plain_models):
+@pytest.mark.parametrize("model,dtype,page", CASES)
+def test_ragged_portions(model, dtype, page, engines, plain_models):
     plain = plain_models[model]
     reqs = _requests(plain[0]["vocab_size"])
-    eng = engines(model, dtype)
+    eng = engines(model, dtype, page_size=page)
     steps = []
     for r, ids in reqs.items():
         pos = 0
@@ -86,28 +89,27 @@ def test_ragged_portions(model, dtype, engines, plain_models):
     assert bad is None, bad
 
 
-@pytest.mark.parametrize("model,dtype", CASES)
-def test_mixed_with_page_reuse(model, dtype, engines, plain_models):
+@pytest.mark.parametrize("model,dtype,page", CASES)
+def test_mixed_with_page_reuse(model, dtype, page, engines, plain_models):
     """Up to four live requests; portions of some beside decoded tokens of others.
-    The pool holds 20 pages (320 tokens) while the requests need 24 in total, so
-    later requests get pages that earlier ones gave back."""
+    The pool holds 320 tokens (20 pages of 16) while the requests need 24 pages of 16 in
+    total, so later requests get pages that earlier ones gave back."""
     plain = plain_models[model]
     vocab = plain[0]["vocab_size"]
     lengths = {"p": 70, "q": 45, "r": 100, "s": 38, "t": 66, "u": 51}
     reqs = {r: random_ids(vocab, n, seed=n) for r, n in lengths.items()}
-    eng = engines(model, dtype, max_cached_tokens=320)
+    eng = engines(model, dtype, max_cached_tokens=320, page_size=page)
+    pool = 320 // page
     order = list(reqs)
     fed = {r: 0 for r in reqs}
     prefill_until = {r: lengths[r] - 12 for r in reqs}   # then one token at a time
     live, waiting, steps = [], order[:], []
     k = 0
     while live or waiting:
-        def pages(r, extra):
-            return -(-(fed[r] + extra) // 16)
         while waiting and len(live) < 4:
             # admit only if the whole request fits beside the live ones
-            need = sum(-(-lengths[r] // 16) for r in live) + -(-lengths[waiting[0]] // 16)
-            if need > 20:
+            need = sum(-(-lengths[r] // page) for r in live) + -(-lengths[waiting[0]] // page)
+            if need > pool:
                 break
             live.append(waiting.pop(0))
         entries, end = [], []
@@ -132,6 +134,47 @@ def test_mixed_with_page_reuse(model, dtype, engines, plain_models):
     assert bad is None, bad
     eng.cache.check_invariants()
     assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+@pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
+                                                ("tiny-c", "float32", True), ("tiny-b", "bfloat16", True),
+                                                ("tiny-d", "float32", True)])
+def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_models):
+    """64 live requests, one token each per step, shrinking to 49, 33, 24 and 17 as requests
+    end: every row of every step against the plain implementation. Captured steps run at
+    padded sizes (49 as 64, 33 as 48, 17 as 24); their padding rows must change nothing."""
+    plain = plain_models[model]
+    vocab = plain[0]["vocab_size"]
+    prompt = [2 + (13 * i) % 61 for i in range(64)]                 # 2 to 62 tokens: page ends fall everywhere
+    reqs = {i: random_ids(vocab, n + 10, 500 + i) for i, n in enumerate(prompt)}
+    want = _expected(plain, reqs, dtype)
+    eng = make_engine(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=64, max_cached_tokens=64 * 80,
+                      max_num_batched_tokens=1024)
+    steps = [([(i, reqs[i][:prompt[i]], [prompt[i] - 1]) for i in range(lo, min(lo + 16, 64))], []) for lo in range(0, 64, 16)]
+    live = list(range(64))
+    for k, keep in enumerate((64, 64, 64, 49, 49, 33, 33, 24, 17, 17)):
+        end = live[keep:]
+        if end:                                                     # they leave before this step
+            steps[-1] = (steps[-1][0], end)
+        live = live[:keep]
+        steps.append(([(i, [reqs[i][prompt[i] + k]], [0]) for i in live], []))
+    steps[-1] = (steps[-1][0], list(live))
+    got = replay(eng, steps)
+    assert len(got) == 64 + 3 * 64 + 2 * 49 + 2 * 33 + 24 + 2 * 17
+    bad, worst = first_bad(got, want, TOL[dtype])
+    assert bad is None, bad
+    eng.cache.check_invariants()
+    assert eng.cache.page_groups[0].allocator.num_used == 0
+    if graphs:
+        assert eng.graph_replays >= 4
+
+
+@pytest.mark.parametrize("model,dtype,page", [("tiny-b", "float32", 8), ("tiny-c", "bfloat16", 16), ("tiny-a", "bfloat16", 16)])
+def test_mixed_with_page_reuse_on_poisoned_pages(model, dtype, page, model_dirs, plain_models):
+    """The mixed trace again with the debug mode that fills every freed page with NaN: a
+    kernel that read a page its request does not hold would put NaN into the logits."""
+    test_mixed_with_page_reuse(model, dtype, page, lambda m, d, **kw: make_engine(model_dirs[m], d, debug_poison=True, **kw),
+                               plain_models)
 
 
 def test_weights_stored_in_32_bits_run_in_either_mode(tmp_path, plain_models):

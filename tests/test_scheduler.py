@@ -9,7 +9,9 @@ import pytest
 
 from pyre_amd.cache import CacheManager
 from pyre_amd.engine.scheduler import Scheduler
-from pyre_amd.parts.base import KVCacheSpec
+from pyre_amd.parts.base import PagedCacheSpec, PagedTensorSpec
+
+ONE_RECORD = PagedCacheSpec((PagedTensorSpec("record", (8,)),))
 
 
 @dataclass
@@ -26,7 +28,7 @@ class FakeEngine:
 
     def __init__(self, pages=64, page_size=16, max_len=512, **cfg):
         self.engine_config = FakeConfig(**cfg)
-        self.cache = CacheManager([KVCacheSpec(1, 8)], page_size, pages, self.engine_config.max_num_seqs, max_len)
+        self.cache = CacheManager([ONE_RECORD], page_size, pages, self.engine_config.max_num_seqs, max_len)
         self.max_model_len = max_len
         self.steps = []
 
