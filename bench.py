@@ -1,17 +1,26 @@
-"""Decode and prefill throughput of the Qwen2.5-7B shape with random weights on one MI355X.
+"""Decode and prefill throughput of a Qwen2.5 shape with random weights on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--model qwen2.5-7b]
+    python bench.py --workload serve [--model qwen2.5-1.5b] [--requests 256] [--max-batch 64]
 
 A step is one decode step of the scheduler: every running request gets one new
 token (plan, one engine step over the paged cache, greedy sampling, token fed
 back). ``value`` is decoded tokens per second at ``--batch`` requests whose
 context reaches ``--context`` at the last timed step. The same line carries the
-prefill of a 2,048-token prompt, the decode step's memory roofline, and decode
-throughput at batch 1 and 64. Timing follows the reference's harness
-(`bench/harness.py:95-120`): fenced by device synchronisation, warm-up first;
-decode excludes prefill (`bench/harness.py:10-12`). Synthetic token ids (uniform
-over the vocabulary), random weights ~ N(0, 0.02): there is no tokenizer and no
-checkpoint here.
+prefill of a 2,048-token prompt, the decode step's memory roofline, decode
+throughput, step time and roofline at batch 1 and 64, and where and when it ran
+(device, ROCm and torch versions, git revision, time: `bench/harness.py:49-67`).
+Timing follows the reference's harness (`bench/harness.py:95-120`): fenced by device
+synchronisation, warm-up first, the median of three timed blocks of ``--steps`` steps;
+decode excludes prefill (`bench/harness.py:10-12`).
+
+``--workload serve`` is continuous batching as in `bench/bench_batch.py:29-46` (one
+scheduler run, all tokens over the wall clock): by default 256 requests on the
+Qwen2.5-1.5B shape, prompt lengths log-uniform in [16, 2048], outputs uniform in
+[16, 512], prompt portions of 512, contexts of at most 4,096, seeded.
+
+Synthetic token ids (uniform over the vocabulary), random weights ~ N(0, 0.02): there is
+no tokenizer and no checkpoint here.
 """
 
 from __future__ import annotations
@@ -44,6 +53,109 @@ def model_numbers(cfg, n_layers: int, dtype_bytes: int):
     return weight_bytes, kv_bytes_per_token, prefill_flops
 
 
+def environment() -> dict:
+    """Where and when: device, library versions, the revision of this tree."""
+    import datetime
+    import os
+    import subprocess
+
+    import torch
+
+    try:
+        sha = subprocess.run(["git", "rev-parse", "--short", "HEAD"], capture_output=True, text=True, timeout=10,
+                             cwd=os.path.dirname(os.path.abspath(__file__))).stdout.strip() or None
+    except (OSError, subprocess.SubprocessError):
+        sha = None
+    return {"device": torch.cuda.get_device_name(0), "torch": torch.__version__, "rocm": torch.version.hip,
+            "git": sha, "time": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ")}
+
+
+def serve(args) -> int:
+    """Continuous batching of many requests of unequal lengths through the scheduler."""
+    import math
+
+    import torch
+
+    from pyre_amd.api import Scheduler
+    from pyre_amd.config import EngineConfig, preset
+    from pyre_amd.engine.context import TORCH_DTYPES
+    from pyre_amd.engine.engine import Engine
+    from pyre_amd.weights import model_tensor_specs, random_state
+
+    model = args.model or "qwen2.5-1.5b"
+    cfg = preset(model)
+    dev, max_context, chunk = "cuda:0", 4096, 512
+    rng = random.Random(args.seed)
+    prompts, outputs = [], []
+    for _ in range(args.requests):
+        n = int(round(math.exp(rng.uniform(math.log(16), math.log(2048)))))
+        prompts.append([rng.randrange(cfg.vocab_size) for _ in range(n)])
+        outputs.append(rng.randint(16, 512))
+    t0 = time.perf_counter()
+    budget = chunk + args.max_batch
+    ec = EngineConfig(dtype=args.dtype, device=dev, page_size=16, max_num_seqs=args.max_batch,
+                      max_cached_tokens=args.max_batch * max_context, max_model_len=max_context,
+                      max_num_batched_tokens=budget, prefill_chunk=chunk, use_graphs=not args.no_graphs,
+                      tune_gemm_rows=())
+    state = random_state(model_tensor_specs(cfg), 0, 0.02, 0.0, TORCH_DTYPES[ec.dtype], device=dev)
+    engine = Engine.from_state(cfg, state, ec)
+    del state
+    print(f"[bench] engine ready in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    def run(n_requests: int) -> dict:
+        sched = Scheduler(engine, max_batch=args.max_batch)
+        for p, n in zip(prompts[:n_requests], outputs[:n_requests]):
+            sched.add_request(p, max_new_tokens=n)
+        replays0, captured_s, eager_s, captured, eager = engine.graph_replays, 0.0, 0.0, 0, 0
+        torch.cuda.synchronize()
+        t_start = t_note = time.perf_counter()
+        while sched.has_work:
+            before = engine.graph_replays
+            t = time.perf_counter()
+            sched.step()
+            dt = time.perf_counter() - t
+            if engine.graph_replays > before:
+                captured, captured_s = captured + 1, captured_s + dt
+            else:
+                eager, eager_s = eager + 1, eager_s + dt
+            if time.perf_counter() - t_note > 30:
+                t_note = time.perf_counter()
+                print(f"[bench] {len(sched.finished)} of {n_requests} requests done ...", file=sys.stderr, flush=True)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t_start
+        gen = sum(len(r.generated) for r in sched.finished.values())
+        assert len(sched.finished) == n_requests and engine.cache.page_groups[0].allocator.num_used == 0
+        pre = sum(len(p) for p in prompts[:n_requests])
+        return {"wall_s": round(wall, 3), "prompt_tokens": pre, "generated_tokens": gen,
+                "total_tok_s": round((pre + gen) / wall, 1), "decode_tok_s": round(gen / wall, 1),
+                "steps": captured + eager, "captured_steps": captured,
+                "captured_share": round(captured / max(1, captured + eager), 4),
+                "ms_per_captured_step": round(captured_s / max(1, captured) * 1e3, 3),
+                "ms_per_uncaptured_step": round(eager_s / max(1, eager) * 1e3, 3),
+                "preemptions": sum(r.preemptions for r in sched.finished.values()),
+                "graph_replays": engine.graph_replays - replays0}
+
+    run(min(args.requests, 2 * args.max_batch))      # warm-up: buffers grown, decode steps captured
+    res = run(args.requests)
+    line = {
+        "metric": "serving tok/s (%s shape, %d requests, continuous batching)" % (model, args.requests),
+        "value": res["total_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": res["steps"], "warmup": 0,
+        "ms_per_step": round(res["wall_s"] / res["steps"] * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic token ids, random weights N(0, 0.02) seed 0; prompts log-uniform [16, 2048], "
+                "outputs uniform [16, 512], seed %d" % args.seed,
+        "config": {"model": model, "requests": args.requests, "max_batch": args.max_batch, "prefill_chunk": chunk,
+                   "max_num_batched_tokens": budget, "max_context": max_context, "page_size": 16,
+                   "parallelism": "single GPU", "layers": cfg.num_hidden_layers, "hidden_size": cfg.hidden_size,
+                   "intermediate_size": cfg.intermediate_size, "num_attention_heads": cfg.num_attention_heads,
+                   "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "vocab_size": cfg.vocab_size, "graphs": bool(ec.use_graphs)},
+        "serve": res, "env": environment(),
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -51,7 +163,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--model", default="qwen2.5-7b", help="preset shape")
+    ap.add_argument("--model", default=None, help="preset shape (qwen2.5-7b; for --workload serve qwen2.5-1.5b)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve"])
+    ap.add_argument("--requests", type=int, default=256, help="serve: number of requests")
+    ap.add_argument("--max-batch", type=int, default=64, help="serve: requests that run at a time")
+    ap.add_argument("--seed", type=int, default=0, help="serve: seed of the lengths and token ids")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has")
     ap.add_argument("--points", default="1,64", help="further decode batch sizes ('' for none)")
@@ -65,6 +181,9 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.workload == "serve":
+        return serve(args)
+    args.model = args.model or "qwen2.5-7b"
 
     import torch
 
@@ -102,13 +221,16 @@ def main() -> int:
     def sync() -> None:
         torch.cuda.synchronize()
 
-    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        """(tokens per second, ms per step) of `steps` decode steps at `batch`."""
+    BLOCKS = 3
+
+    def decode(batch: int, steps: int, warmup: int) -> dict:
+        """Three timed blocks of `steps` decode steps at `batch`; the block of median time counts.
+        The last block ends at the full context."""
         sched = Scheduler(engine, max_batch=batch)
         # Requests whose prompt is done decode while the others are still being
         # prefilled (one step per portion of a prompt), so leave room for those tokens too.
         portions = -(-args.context // PREFILL_TOKENS)
-        start_ctx = args.context - (steps + warmup) - portions * batch - 2
+        start_ctx = args.context - (BLOCKS * steps + warmup) - portions * batch - 2
         for _ in range(batch):
             sched.add_request(prompt(start_ctx), max_new_tokens=args.context - start_ctx)
         t_fill = time.perf_counter()
@@ -119,16 +241,22 @@ def main() -> int:
                 print(f"[bench] filling caches for batch {batch} ...", file=sys.stderr, flush=True)
         for _ in range(warmup):
             sched.step()
-        sync()
-        t = time.perf_counter()
-        for _ in range(steps):
-            out = sched.step()
-            assert len(out) == batch
-        sync()
-        dt = time.perf_counter() - t
+        blocks = []
+        for _ in range(BLOCKS):
+            ctx0 = sum(r.num_computed for r in sched.running) / batch
+            sync()
+            t = time.perf_counter()
+            for _ in range(steps):
+                out = sched.step()
+                assert len(out) == batch
+            sync()
+            blocks.append((time.perf_counter() - t, ctx0 + steps / 2))
         for r in list(sched.running):
             engine.finish(r.seq_id)
-        return batch * steps / dt, dt / steps * 1e3
+        dt, mean_ctx = sorted(blocks)[BLOCKS // 2]
+        ms = dt / steps * 1e3
+        achieved = (weight_bytes + batch * mean_ctx * kv_per_token) / (ms / 1e3) / 1e9
+        return {"tok_s": batch * steps / dt, "ms": ms, "gbs": achieved, "frac": achieved / HBM_PEAK_GBS}
 
     prefill = None
     if not args.no_prefill:
@@ -152,17 +280,19 @@ def main() -> int:
         print(json.dumps({"metric": "prefill tok/s (%s shape, %d tokens)" % (args.model, PREFILL_TOKENS),
                           "prefill": prefill, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32"}))
         return 0
-    value, ms_per_step = decode(args.batch, args.steps, args.warmup)
-    mean_ctx = args.context - args.steps / 2
-    step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token
-    achieved = step_bytes / (ms_per_step / 1e3) / 1e9
-    pts = {}
+    main_point = decode(args.batch, args.steps, args.warmup)
+    value, ms_per_step, achieved = main_point["tok_s"], main_point["ms"], main_point["gbs"]
+    pts, pts_ms, pts_frac = {}, {}, {}
     for b in points:
-        pts[f"decode_b{b}"] = round(decode(b, args.steps, args.warmup)[0], 1)
-        print(f"[bench] decode_b{b} {pts[f'decode_b{b}']}", file=sys.stderr, flush=True)
+        pt = decode(b, args.steps, args.warmup)
+        pts[f"decode_b{b}"], pts_ms[f"decode_b{b}"] = round(pt["tok_s"], 1), round(pt["ms"], 4)
+        pts_frac[f"decode_b{b}"] = round(pt["frac"], 4)
+        print(f"[bench] decode_b{b} {pts[f'decode_b{b}']} tok/s, {pts_ms[f'decode_b{b}']} ms, "
+              f"{pts_frac[f'decode_b{b}']} of the HBM peak", file=sys.stderr, flush=True)
+    pts_ms[f"decode_b{args.batch}"], pts_frac[f"decode_b{args.batch}"] = round(ms_per_step, 4), round(achieved / HBM_PEAK_GBS, 4)
 
     line = {
-        "metric": "decode tok/s (Qwen2.5-7B shape, batch %d, context %d)" % (args.batch, args.context),
+        "metric": "decode tok/s (%s shape, batch %d, context %d)" % (args.model, args.batch, args.context),
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
@@ -177,7 +307,8 @@ def main() -> int:
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
-        "points": pts,
+        "points": pts, "points_ms_per_step": pts_ms, "points_hbm_frac": pts_frac,
+        "timing": "median of %d timed blocks of %d steps" % (BLOCKS, args.steps), "env": environment(),
     }
     print(json.dumps(line))
     return 0
