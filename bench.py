@@ -1,7 +1,7 @@
 """Decode and prefill throughput of a Qwen2.5 shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--model qwen2.5-7b]
-    python bench.py --workload serve [--model qwen2.5-1.5b] [--requests 256] [--max-batch 64]
+    python bench.py --workload serve [--model qwen2.5-1.5b] [--requests 256] [--max-batch 256]
 
 A step is one decode step of the scheduler: every running request gets one new
 token (plan, one engine step over the paged cache, greedy sampling, token fed
@@ -92,7 +92,7 @@ def serve(args) -> int:
         prompts.append([rng.randrange(cfg.vocab_size) for _ in range(n)])
         outputs.append(rng.randint(16, 512))
     t0 = time.perf_counter()
-    budget = chunk + args.max_batch
+    budget = args.token_budget or 4 * chunk + args.max_batch
     ec = EngineConfig(dtype=args.dtype, device=dev, page_size=16, max_num_seqs=args.max_batch,
                       max_cached_tokens=args.max_batch * max_context, max_model_len=max_context,
                       max_num_batched_tokens=budget, prefill_chunk=chunk, use_graphs=not args.no_graphs,
@@ -166,8 +166,10 @@ def main() -> int:
     ap.add_argument("--model", default=None, help="preset shape (qwen2.5-7b; for --workload serve qwen2.5-1.5b)")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve"])
     ap.add_argument("--requests", type=int, default=256, help="serve: number of requests")
-    ap.add_argument("--max-batch", type=int, default=64, help="serve: requests that run at a time")
+    ap.add_argument("--max-batch", type=int, default=256, help="serve: requests that run at a time")
     ap.add_argument("--seed", type=int, default=0, help="serve: seed of the lengths and token ids")
+    ap.add_argument("--token-budget", type=int, default=0,
+                    help="serve: tokens in one step (0: four prompt portions beside a token of every running request)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has")
     ap.add_argument("--points", default="1,64", help="further decode batch sizes ('' for none)")

@@ -14,8 +14,9 @@ from dataclasses import dataclass, field
 
 import numpy as np
 
-#: sizes (requests) at which decode steps are captured in HIP graphs
-DECODE_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64)
+#: sizes (requests) at which decode steps are captured in HIP graphs: up to 64 rows the
+#: weight-streaming products' own sizes, beyond that the BLAS library's products
+DECODE_ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 MIN_TABLE_WIDTH = 8
 
 

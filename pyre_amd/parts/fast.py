@@ -70,7 +70,8 @@ def linear(lin, ctx, x, n, out):
     k, n_out = lin.in_features, lin.out_features
     skinny = rt.options.get("skinny_gemm", True) and ops.gemm_skinny_supports(
         min(n, SKINNY_MAX_ROWS), n_out, k, x.stride(0), lin.weight.stride(0))
-    if skinny and (n <= SKINNY_MAX_ROWS or out is not None):
+    library = rt.options.get("library_gemm", True)
+    if skinny and (n <= SKINNY_MAX_ROWS or (out is not None and not library)):
         if out is not None:
             # float32 results wanted in place (the head's logits): no split, 64 rows at a time
             for r0 in range(0, n, SKINNY_MAX_ROWS):
@@ -81,8 +82,13 @@ def linear(lin, ctx, x, n, out):
         buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
         ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
         return Partials(buf, lin.bias)
-    if out is not None or not rt.options.get("library_gemm", True):
+    if not library:
         return None
+    if out is not None:
+        # many rows of float32 results in place (the head's logits of a large decode step, or of
+        # every row of a portion): one pass over the weights in the library
+        torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out_dtype=torch.float32, out=out)
+        return Partials(out.view(1, n, n_out), lin.bias)
     if lin.role in rt.options.get("library_f32_roles", LIBRARY_F32_ROLES):
         buf = ctx.workspace.get(f"linear32.{lin.role}", (n, n_out), torch.float32)
         torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out_dtype=torch.float32, out=buf)

@@ -103,3 +103,22 @@ def test_decode_steps_of_many_requests_at_the_7b_shape(dtype, layers_7b):
     assert bad is None, bad
     for k in got:
         assert torch.equal(got[k], got2[k]), f"{k}: a replayed step differs from the eager one"
+
+
+def test_captured_decode_steps_with_library_products_at_the_7b_shape(layers_7b):
+    """100 live requests: a decode step of 128 rows, whose products are the BLAS library's,
+    captured and replayed four times; every replay against the plain implementation."""
+    cfg, state, plain = layers_7b
+    vocab = cfg.vocab_size
+    lengths = [3 + (5 * i) % 23 for i in range(100)]
+    reqs = {i: random_ids(vocab, n + 6, 300 + i) for i, n in enumerate(lengths)}
+    want = _want(plain, reqs, "bfloat16")
+    eng = make_engine_from_state(cfg, state, "bfloat16", use_graphs=True, max_cached_tokens=100 * 48, max_num_seqs=100,
+                                 max_num_batched_tokens=2048)
+    steps = [([(i, reqs[i][:lengths[i]], []) for i in range(lo, lo + 50)], []) for lo in (0, 50)]
+    for k in range(6):
+        steps.append(([(i, [reqs[i][lengths[i] + k]], [0]) for i in range(100)], []))
+    got = replay(eng, steps)
+    assert len(got) == 600 and eng.graph_replays == 5
+    bad, worst = first_bad(got, want, TOL["bfloat16"])
+    assert bad is None, bad

@@ -169,6 +169,38 @@ def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_m
         assert eng.graph_replays >= 4
 
 
+@pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
+                                                ("tiny-b", "float32", True)])
+def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, model_dirs, plain_models):
+    """200, 150, 100 and 70 live requests: decode steps whose products go to the BLAS library
+    (more than 64 rows), captured at 256, 192, 128 and 96 rows and replayed several times,
+    each replay against the plain implementation (a library call that records a clearing of
+    memory into the graph would be right once and wrong afterwards)."""
+    plain = plain_models[model]
+    vocab = plain[0]["vocab_size"]
+    prompt = [2 + (13 * i) % 37 for i in range(200)]
+    reqs = {i: random_ids(vocab, n + 12, 900 + i) for i, n in enumerate(prompt)}
+    want = _expected(plain, reqs, dtype)
+    eng = make_engine(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=200, max_cached_tokens=200 * 64,
+                      max_num_batched_tokens=2048)
+    steps = [([(i, reqs[i][:prompt[i]], []) for i in range(lo, lo + 50)], []) for lo in range(0, 200, 50)]
+    live, counts = list(range(200)), (200, 200, 200, 150, 150, 150, 100, 100, 100, 70, 70, 70)
+    for k, keep in enumerate(counts):
+        end = live[keep:]
+        if end:
+            steps[-1] = (steps[-1][0], end)
+        live = live[:keep]
+        steps.append(([(i, [reqs[i][prompt[i] + k]], [0]) for i in live], []))
+    steps[-1] = (steps[-1][0], list(live))
+    got = replay(eng, steps)
+    assert len(got) == sum(counts)
+    bad, worst = first_bad(got, want, TOL[dtype])
+    assert bad is None, bad
+    assert eng.cache.page_groups[0].allocator.num_used == 0
+    if graphs:
+        assert eng.graph_replays == 8      # of each size: once eagerly, then captured and replayed twice
+
+
 @pytest.mark.parametrize("model,dtype,page", [("tiny-b", "float32", 8), ("tiny-c", "bfloat16", 16), ("tiny-a", "bfloat16", 16)])
 def test_mixed_with_page_reuse_on_poisoned_pages(model, dtype, page, model_dirs, plain_models):
     """The mixed trace again with the debug mode that fills every freed page with NaN: a
