@@ -290,7 +290,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
   const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
   const int head0 = kvh * n_rep + qt * 16, nheads = min(16, n_rep - qt * 16);
-  const int idx = blockIdx.z, tok = tokens[idx];
+  const int idx = blockIdx.z, tok = tokens ? tokens[idx] : idx;  // no list: the batch holds single tokens only
   const int pos = positions[tok];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
 
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(128) void attn_decode_reduce(const float* __restric
   const float ws = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
   if (tid < nsplits) w[tid] = ws;
   const float L = block_sum(ls * ws, scratch);  // its barriers publish w[]
-  const int tok = tokens[idx];
+  const int tok = tokens ? tokens[idx] : idx;
   for (int d = tid; d < HD; d += 128) {
     float acc = 0.f;
 #pragma unroll 8

@@ -35,6 +35,24 @@ template <> struct Vec4<bf16> {
 
 __device__ inline float4 add4(float4 a, float4 b) { return float4{a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w}; }
 
+// p[0] + p[1] + ... + p[n - 1] (in that order) of the float4 at `src` in each of n partial sums that
+// lie `stride` elements apart. Up to kAtOnce loads are in flight together: a kernel that only
+// passes a few rows on spends its time waiting for loads, one round trip after the other.
+constexpr int kAtOnce = 12;
+template <typename T>
+__device__ inline float4 sum_partials4(const T* src, size_t stride, int n) {
+  float4 v[kAtOnce];
+#pragma unroll
+  for (int p = 0; p < kAtOnce; ++p)
+    if (p < n) v[p] = Vec4<T>::load(src + p * stride);
+  float4 s = v[0];
+#pragma unroll
+  for (int p = 1; p < kAtOnce; ++p)
+    if (p < n) s = add4(s, v[p]);
+  for (int p = kAtOnce; p < n; ++p) s = add4(s, Vec4<T>::load(src + p * stride));
+  return s;
+}
+
 // ---------------------------------------------------------------------------
 // add + RMSNorm, one block per row, the row kept in registers between the passes.
 // ---------------------------------------------------------------------------
@@ -68,17 +86,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
     if (c >= nvec) break;
     float4 x = Vec4<float>::load(resid + in_off + 4 * c);
     if (delta) {
-      const TD* dp = delta + in_off + 4 * c;
-      float4 d = Vec4<TD>::load(dp);
-      int p = 1;
-      for (; p + 3 < n_partials; p += 4) {  // four loads in flight, added in the order p, p+1, ...
-        const float4 d0 = Vec4<TD>::load(dp + p * partial_stride);
-        const float4 d1 = Vec4<TD>::load(dp + (p + 1) * partial_stride);
-        const float4 d2 = Vec4<TD>::load(dp + (p + 2) * partial_stride);
-        const float4 d3 = Vec4<TD>::load(dp + (p + 3) * partial_stride);
-        d = add4(add4(add4(add4(d, d0), d1), d2), d3);
-      }
-      for (; p < n_partials; ++p) d = add4(d, Vec4<TD>::load(dp + p * partial_stride));
+      const float4 d = sum_partials4<TD>(delta + in_off + 4 * c, partial_stride, n_partials);
       x = add4(x, d);
       if (!rows) Vec4<float>::store(resid + in_off + 4 * c, x);
     }
@@ -133,17 +141,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
 
   auto value4 = [&](int col) {
-    const TI* src = qkv + in_row + col;
-    float4 v = Vec4<TI>::load(src);
-    int p = 1;
-    for (; p + 3 < n_partials; p += 4) {  // four loads in flight, added in the order p, p+1, ...
-      const float4 d0 = Vec4<TI>::load(src + p * partial_stride);
-      const float4 d1 = Vec4<TI>::load(src + (p + 1) * partial_stride);
-      const float4 d2 = Vec4<TI>::load(src + (p + 2) * partial_stride);
-      const float4 d3 = Vec4<TI>::load(src + (p + 3) * partial_stride);
-      v = add4(add4(add4(add4(v, d0), d1), d2), d3);
-    }
-    for (; p < n_partials; ++p) v = add4(v, Vec4<TI>::load(src + p * partial_stride));
+    float4 v = sum_partials4<TI>(qkv + in_row + col, partial_stride, n_partials);
     if (bias) {  // col is a multiple of 4: one load of four
       v = add4(v, bias_dt == kF32 ? Vec4<float>::load(static_cast<const float*>(bias) + col)
                                   : Vec4<bf16>::load(static_cast<const bf16*>(bias) + col));

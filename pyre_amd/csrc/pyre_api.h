@@ -66,7 +66,8 @@ int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
 // 1 if the MFMA attention kernels take this geometry (else use pyre_attn_generic).
 int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv);
 
-// One new token per request. tokens[i] indexes the flat batch; part_acc is
+// One new token per request. tokens[i] indexes the flat batch (null: token i itself, a batch
+// of single tokens only, which saves every wave a dependent load); part_acc is
 // [n_tokens, nq, nsplits, hd] floats and part_ml [n_tokens, nq, nsplits, 2] of scratch.
 int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
                           const int* tokens, int n_tokens, const int* positions,

@@ -347,15 +347,17 @@ def _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table,
 def attn_decode_bf16(q, out, k_cache, v_cache, tokens, n_tokens, positions, seq_of_token, block_table,
                      part_acc, part_ml, nsplits, nq, nkv, hd, page_size, scale, window=0) -> None:
     """Attention of ``n_tokens`` single new tokens (``tokens`` indexes the flat
-    batch) over the paged cache, keys split ``nsplits`` ways."""
+    batch; None: the batch is these tokens, in order) over the paged cache, keys split
+    ``nsplits`` ways."""
     _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
-    _i32("tokens", tokens, n_tokens)
+    if tokens is not None:
+        _i32("tokens", tokens, n_tokens)
     if part_acc.dtype != torch.float32 or part_acc.numel() < n_tokens * nq * nsplits * hd:
         raise KernelError("attn_decode: partial accumulators too small")
     if part_ml.dtype != torch.float32 or part_ml.numel() < n_tokens * nq * nsplits * 2:
         raise KernelError("attn_decode: partial max/sum buffer too small")
     call("pyre_attn_decode_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-         tokens.data_ptr(), n_tokens, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+         _ptr(tokens), n_tokens, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
          block_table.stride(0), part_acc.data_ptr(), part_ml.data_ptr(), nsplits, nq, nkv, hd, page_size,
          float(scale), int(window), _stream())
 

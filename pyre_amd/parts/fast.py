@@ -156,7 +156,9 @@ def attention(mixer, ctx, q, o, cache) -> bool:
             ctx.runtime.options.get("decode_target_waves", DECODE_TARGET_WAVES))
         acc = ctx.workspace.get("attn.part_acc", (n_dec, s.num_heads, nsplits, s.head_dim), torch.float32)
         ml = ctx.workspace.get("attn.part_ml", (n_dec, s.num_heads, nsplits, 2), torch.float32)
-        ops.attn_decode_bf16(q, o, k_pages, v_pages, ctx.arrays["attention.decode_tokens"], n_dec, ctx.positions,
+        # a batch of single tokens only needs no list of them
+        which = None if n_dec == ctx.n_tokens else ctx.arrays["attention.decode_tokens"]
+        ops.attn_decode_bf16(q, o, k_pages, v_pages, which, n_dec, ctx.positions,
                              ctx.seq_of_token, cache.table, acc, ml, nsplits, s.num_heads, s.num_kv_heads,
                              s.head_dim, cache.page_size, mixer.scale, cache.window)
     if n_tiles:
