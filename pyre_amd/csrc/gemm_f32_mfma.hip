@@ -1,0 +1,176 @@
+// out[m, n] = sum_k A[m, k] * W[n, k] (+ bias[n]) with all three in float32, on the matrix
+// cores' true 32-bit instruction (v_mfma_f32_32x32x2_f32: float32 operands, float32 products
+// and sums; no reduced-precision mode is involved). This is the product of the 32-bit path
+// of the model (`pyre/model.py:92-94,125,139,201` are the products it stands for); operands
+// of mixed element types stay with gemm_generic.hip.
+//
+// As in the weight-streaming kernels the product is computed transposed, out^T = W A^T: the
+// 32 rows of an MFMA tile are output columns n, its 32 columns are rows m, so that a lane
+// holds runs of four consecutive n of one row m and stores them as one float4.
+//
+// k is walked in stages of 16 through LDS; within a stage, MFMA step s (0..7) multiplies k = s
+// in lanes 0..31 and k = 8 + s in lanes 32..63, so that every lane reads its eight values of a
+// stage as two 16-byte LDS loads. The order in which the products of an output element are
+// added is therefore (0, 8), (1, 9), ..., (7, 15), (16, 24), ...: a function of k alone. Both
+// tile shapes below walk k the same way, so an element's value does not depend on the shape,
+// on the number of rows in the step or on where the row lies in it, bit for bit.
+//
+// k may be split into `ksplit` parts (grid.z), each writing a partial sum out[s] that the
+// consumer adds in the order 0..ksplit-1: products with few output columns and a long k would
+// otherwise leave most of the chip idle. The caller chooses ksplit from N and K alone.
+#include "pyre_api.h"
+#include "pyre_common.h"
+
+using namespace pyre;
+
+namespace {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int BK = 16;      // k per stage
+constexpr int LD = BK + 4;  // floats per LDS row: 80 bytes, so that eight rows' 16-byte pieces fall on distinct banks
+
+// Four consecutive k of one row; zero where the row or the k is not there.
+__device__ inline f32x4 load_k4(const float* base, size_t ld, int row, int rows, int k, int K, bool vec_ok) {
+  if (row >= rows || k >= K) return f32x4{0.f, 0.f, 0.f, 0.f};
+  const float* p = base + static_cast<size_t>(row) * ld + k;
+  if (vec_ok && k + 3 < K) return *reinterpret_cast<const f32x4*>(p);
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 4 && k + j < K; ++j) v[j] = p[j];
+  return v;
+}
+
+// WN x WM waves (along n and along m), each on TN x TM tiles of 32 x 32.
+template <int WN, int WM, int TN, int TM>
+__global__ __launch_bounds__(64 * WN * WM) void gemm_f32_mfma_kernel(
+    const float* __restrict__ A, size_t lda, const float* __restrict__ W, size_t ldw,
+    const void* __restrict__ bias, int bias_dt, float* __restrict__ out, size_t ldo, size_t part_stride, int M,
+    int N, int K, int kper, int vec_ok) {
+  constexpr int NT = 64 * WN * WM, BN = WN * TN * 32, BM = WM * TM * 32;
+  constexpr int WP = (BN * 4 + NT - 1) / NT, AP = (BM * 4 + NT - 1) / NT;  // 16-byte pieces per thread and stage
+  __shared__ __attribute__((aligned(16))) float Ws[BN][LD];
+  __shared__ __attribute__((aligned(16))) float As[BM][LD];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, c = lane & 31;
+  const int wn = wave % WN, wm = wave / WN;
+  const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+  const int kbeg = blockIdx.z * kper;
+  K = min(K, kbeg + kper);  // this part's end
+  out += blockIdx.z * part_stride;
+  if (blockIdx.z) bias = nullptr;  // the bias belongs to one part only
+
+  f32x4 wr[WP], ar[AP];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < WP; ++i) {
+      const int p = tid + NT * i;
+      wr[i] = p < BN * 4 ? load_k4(W, ldw, n0 + p / 4, N, k0 + 4 * (p % 4), K, vec_ok) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int i = 0; i < AP; ++i) {
+      const int p = tid + NT * i;
+      ar[i] = p < BM * 4 ? load_k4(A, lda, m0 + p / 4, M, k0 + 4 * (p % 4), K, vec_ok) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < WP; ++i) {
+      const int p = tid + NT * i;
+      if (p < BN * 4) *reinterpret_cast<f32x4*>(&Ws[p / 4][4 * (p % 4)]) = wr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < AP; ++i) {
+      const int p = tid + NT * i;
+      if (p < BM * 4) *reinterpret_cast<f32x4*>(&As[p / 4][4 * (p % 4)]) = ar[i];
+    }
+  };
+
+  f32x16 acc[TN][TM];
+#pragma unroll
+  for (int t = 0; t < TN; ++t)
+#pragma unroll
+    for (int u = 0; u < TM; ++u)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[t][u][i] = 0.f;
+
+  fetch(kbeg);
+  for (int k0 = kbeg; k0 < K; k0 += BK) {
+    stash();
+    __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);  // in flight while this stage is multiplied
+    f32x4 a[TN][2], b[TM][2];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) a[t][h] = *reinterpret_cast<const f32x4*>(&Ws[(wn * TN + t) * 32 + c][8 * half + 4 * h]);
+#pragma unroll
+    for (int u = 0; u < TM; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) b[u][h] = *reinterpret_cast<const f32x4*>(&As[(wm * TM + u) * 32 + c][8 * half + 4 * h]);
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int u = 0; u < TM; ++u)
+          acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s >> 2][s & 3], b[u][s >> 2][s & 3], acc[t][u], 0, 0, 0);
+    __syncthreads();
+  }
+
+  // acc[t][u][4 i + j]: output column n = tile row 8 i + 4 half + j, output row m = tile column c.
+#pragma unroll
+  for (int u = 0; u < TM; ++u) {
+    const int m = m0 + (wm * TM + u) * 32 + c;
+    if (m >= M) continue;
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + (wn * TN + t) * 32 + 8 * i + 4 * half;
+        if (n >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[j] = acc[t][u][4 * i + j];
+          if (bias && n + j < N) v[j] += load_as_float(bias, bias_dt, n + j);
+        }
+        float* dst = out + static_cast<size_t>(m) * ldo + n;
+        if (n + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+          *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+          for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = v[j];
+        }
+      }
+  }
+}
+
+}  // namespace
+
+extern "C" int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw, const void* bias, int bias_dt,
+                             float* out, long ldo, long part_stride, int M, int N, int K, int ksplit,
+                             hipStream_t stream) {
+  PYRE_REQUIRE(!bias || known_dtype(bias_dt), "gemm_f32: unknown bias dtype");
+  PYRE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
+  PYRE_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_f32: a leading dimension is too small");
+  PYRE_REQUIRE(ksplit >= 1 && ksplit <= 64 && (ksplit == 1 || part_stride >= static_cast<long>(M) * ldo),
+               "gemm_f32: ksplit=%d, partial sums %ld apart", ksplit, part_stride);
+  if (M == 0) return 0;
+  const int kper = ((K + ksplit - 1) / ksplit + BK - 1) / BK * BK;
+  PYRE_REQUIRE(static_cast<long>(ksplit - 1) * kper < K, "gemm_f32: a part of k would be empty (K=%d, ksplit=%d)", K, ksplit);
+  // 16-byte loads along k need rows that start on 16 bytes
+  const int vec_ok = lda % 4 == 0 && ldw % 4 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(W) % 16 == 0;
+  if (M <= 32) {  // a decode step's few rows: four waves side by side along n
+    const dim3 grid((N + 127) / 128, (M + 31) / 32, ksplit);
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<4, 1, 1, 1>), grid, dim3(256), 0, stream, A, static_cast<size_t>(lda), W,
+                       static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),
+                       static_cast<size_t>(part_stride), M, N, K, kper, vec_ok);
+  } else {
+    const dim3 grid((N + 127) / 128, (M + 127) / 128, ksplit);
+    PYRE_REQUIRE(grid.y <= 65535, "gemm_f32: M=%d too large for one launch", M);
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<2, 2, 2, 2>), grid, dim3(256), 0, stream, A, static_cast<size_t>(lda), W,
+                       static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),
+                       static_cast<size_t>(part_stride), M, N, K, kper, vec_ok);
+  }
+  return check_launch("gemm_f32");
+}

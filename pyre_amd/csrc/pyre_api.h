@@ -46,6 +46,14 @@ int pyre_gemm_generic(const void* A, int a_dt, long lda, const int* a_rows, cons
 int pyre_fill_rows(void* base, int elem_bytes, long outer_stride, int n_outer, int n_rows, long row_elems,
                    const int* ids_host, int n_ids, unsigned pattern, hipStream_t stream);
 
+// The same for float32 operands and results only, on the matrix cores' float32 instruction:
+// the product of the true 32-bit path. The order of an element's additions depends on k alone.
+// ksplit > 1: partial sums out[s] (part_stride elements apart) over ksplit parts of k, the bias
+// in part 0; the consumer adds them in the order 0..ksplit-1.
+int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw, const void* bias, int bias_dt,
+                  float* out, long ldo, long part_stride, int M, int N, int K, int ksplit,
+                  hipStream_t stream);
+
 // bfloat16 products with 1..64 rows (decode): 1 if the kernel takes the shape.
 int pyre_gemm_skinny_supports(int M, int N, int K, long ldx, long ldw);
 

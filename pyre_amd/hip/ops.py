@@ -244,6 +244,39 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, ou
          out.data_ptr(), dtype_code(out), out.stride(0), m, n_out, k, _stream())
 
 
+F32_KSPLIT_MAX = 8
+
+
+def gemm_f32_ksplit(n_out: int, k: int) -> int:
+    """Into how many parts of k the float32 product is split: enough blocks of 128 output
+    columns for the 256 compute units, parts of at least 512. A function of the weight's
+    shape alone, never of the rows, so that a row's result does not depend on its step."""
+    blocks = -(-n_out // 128)
+    return max(1, min(F32_KSPLIT_MAX, 256 // blocks, k // 512))
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, m: int,
+             ksplit: int = 1) -> None:
+    """out[0:m] = a[0:m] @ w.T (+ bias) with float32 operands and result, on the matrix cores'
+    float32 instruction; the order of an element's additions depends on k alone. With
+    ``ksplit`` > 1, ``out`` is [ksplit, m, N]: partial sums over parts of k (the bias in part 0)."""
+    _dev(a, w, bias, out)
+    n_out, k = w.shape
+    if a.dtype != torch.float32 or w.dtype != torch.float32 or out.dtype != torch.float32:
+        raise KernelError("gemm_f32: float32 operands and result expected")
+    if a.dim() != 2 or a.shape[1] != k or out.shape[-1] != n_out or out.dim() != (2 if ksplit == 1 else 3):
+        raise KernelError(f"gemm_f32: a {tuple(a.shape)} @ w {tuple(w.shape)}.T -> out {tuple(out.shape)} do not fit")
+    if a.stride(1) != 1 or w.stride(1) != 1 or out.stride(-1) != 1:
+        raise KernelError("gemm_f32: rows must be contiguous")
+    if out.shape[-2] < m or a.shape[0] < m or (ksplit > 1 and (out.shape[0] != ksplit or out.shape[1] != m)):
+        raise KernelError("gemm_f32: fewer rows than m, or partial sums that are not [ksplit, m, N]")
+    if bias is not None and bias.numel() != n_out:
+        raise KernelError("gemm_f32: bias length")
+    call("pyre_gemm_f32", a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), _ptr(bias),
+         dtype_code(bias) if bias is not None else 0, out.data_ptr(), out.stride(-2),
+         out.stride(0) if ksplit > 1 else 0, m, n_out, k, ksplit, _stream())
+
+
 def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                  n: int, nq: int, nkv: int, hd: int, page_size: int, scale: float,

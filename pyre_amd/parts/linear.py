@@ -38,9 +38,19 @@ class Linear:
         done = fast.linear(self, ctx, x, n, out)
         if done is not None:
             return done
+        f32 = x.dtype == torch.float32 and self.weight.dtype == torch.float32
+        if f32 and out is None:
+            # the true 32-bit path: the matrix cores' float32 instruction, k split by the weight's shape alone
+            ks = ops.gemm_f32_ksplit(self.out_features, self.in_features)
+            buf = ctx.workspace.get(f"linear.{self.role}", (ks, n, self.out_features), torch.float32)
+            ops.gemm_f32(x, self.weight, None, buf if ks > 1 else buf[0], n, ks)
+            return Partials(buf, self.bias)
         if out is None:
             out = ctx.workspace.get(f"linear.{self.role}", (n, self.out_features), torch.float32)
-        ops.gemm_generic(x, self.weight, None, out, n)
+        if f32 and out.dtype == torch.float32:
+            ops.gemm_f32(x, self.weight, None, out, n)
+        else:
+            ops.gemm_generic(x, self.weight, None, out, n)  # mixed element types, any sizes
         return Partials(out.view(1, n, self.out_features), self.bias)
 
 

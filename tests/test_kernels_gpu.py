@@ -124,6 +124,51 @@ def test_gemm_generic(adt, wdt, m, n, k):
     assert torch.allclose(out0, bias.expand(m, n))
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 37, 50), (5, 130, 257), (32, 128, 16), (33, 129, 17), (77, 200, 64), (130, 65, 1000),
+                                   (300, 3584, 3584), (8, 1000, 18944)])
+def test_gemm_f32_on_the_matrix_cores(m, n, k):
+    """float32 in, float32 products and sums (the result is as close to a float64 product as
+    plain float32 FMAs are), and a row's result bit for bit the same whatever rows share
+    the call and wherever it lies among them."""
+    ops = _ops()
+    a = rnd(m, k, seed=1)
+    w = rnd(n, k, seed=2)
+    bias = rnd(n, seed=3)
+    out = torch.full((m, n), float("nan"), device=DEV)
+    ops.gemm_f32(a, w, bias, out, m)
+    want = a.double() @ w.double().T + bias.double()
+    assert torch.allclose(out.double(), want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
+    fma = torch.empty(m, n, device=DEV)
+    ops.gemm_generic(a, w, bias, fma, m)
+    err_mfma, err_fma = (out.double() - want).abs().max().item(), (fma.double() - want).abs().max().item()
+    assert err_mfma <= 4 * err_fma + 1e-6, (err_mfma, err_fma)      # no reduced-precision mode
+    # rows alone, in another order, in a strided view, without a bias: the same bits
+    for rows in ([0], [m - 1], list(range(m - 1, -1, -1)), list(range(0, m, 3))):
+        sub = a[rows].contiguous()
+        o = torch.empty(len(rows), n, device=DEV)
+        ops.gemm_f32(sub, w, bias, o, len(rows))
+        assert torch.equal(o, out[rows]), rows
+    wide = torch.zeros(m, k + 5, device=DEV)
+    wide[:, 1:k + 1] = a                                            # rows that do not start on 16 bytes
+    o = torch.empty(m, n, device=DEV)
+    ops.gemm_f32(wide[:, 1:k + 1], w, None, o, m)
+    assert torch.allclose(o + bias, out, atol=1e-6, rtol=1e-6)
+    # linearity: a zero input gives the bias
+    ops.gemm_f32(torch.zeros_like(a), w, bias, o, m)
+    assert torch.equal(o, bias.expand(m, n))
+    # k in parts: the parts add up to the product, the bias is in the first, no part is empty
+    for ks in {2, 3, ops.gemm_f32_ksplit(n, k)}:
+        kper = -(-(-(-k // ks)) // 16) * 16      # a part's length, as the kernel rounds it
+        if (ks - 1) * kper >= k:
+            continue
+        parts = torch.full((ks, m, n), float("nan"), device=DEV)
+        ops.gemm_f32(a, w, bias, parts if ks > 1 else parts[0], m, ks)
+        assert torch.allclose(parts.double().sum(0), want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
+        one = torch.empty(ks, 1, n, device=DEV)
+        ops.gemm_f32(a[m // 2:m // 2 + 1], w, bias, one if ks > 1 else one[0], 1, ks)
+        assert torch.equal(one[:, 0], parts[:, m // 2])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_silu_mul(dtype):
     ops = _ops()
