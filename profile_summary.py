@@ -1,6 +1,6 @@
 """Per-kernel totals of a rocprofv3 kernel trace.
 
-    python -m pyre_amd.profile_summary RESULTS.db [TOP] [--match TEXT] [--tail-ms MS]
+    python profile_summary.py RESULTS.db [TOP] [--match TEXT] [--tail-ms MS]
 
 reads the ``kernels`` view of the rocpd SQLite file that
 ``rocprofv3 --kernel-trace --stats -d DIR -o NAME -- <program>`` writes
@@ -8,7 +8,7 @@ reads the ``kernels`` view of the rocpd SQLite file that
 kernel name, longest total first. ``--tail-ms MS`` keeps only the launches of the
 last MS milliseconds of the trace (the timed steps of a benchmark, without its set-up).
 
-    python -m pyre_amd.profile_summary --counters COUNTERS.csv [--match TEXT]
+    python profile_summary.py --counters COUNTERS.csv [--match TEXT]
 
 reads the ``*_counter_collection.csv`` of ``rocprofv3 --pmc ... --output-format csv`` and
 prints, per kernel name, the mean of each counter over the kernel's launches.

@@ -6,6 +6,7 @@
 //   probs     = softmax(scores)                               (pyre/model.py:122)
 //   out       = sum_j probs[j] v_j                            (pyre/model.py:123)
 //
+// `tokens` (or null: all of them) lists the n tokens of the flat batch to attend for.
 // A token at position `pos` sees the keys lo..pos of its request, all read from
 // the cache (this step's keys were written before the call), so prompt portions
 // and single decoded tokens are the same case. lo = max(0, pos - window + 1) for
@@ -28,15 +29,15 @@ constexpr int kMaxHead = 256;
 template <typename TQ, typename TC>
 __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
-    TQ* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
-    const int* __restrict__ block_table, int table_stride, int nq, int nkv, int hd, int page_size,
-    float scale, int window) {
+    TQ* __restrict__ out, const int* __restrict__ tokens, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride, int nq, int nkv,
+    int hd, int page_size, float scale, int window) {
   __shared__ float qs[kMaxHead];
   __shared__ float sc[kChunk];
   __shared__ float accs[kThreads];
   __shared__ float scratch[16];
 
-  const int n = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int kvh = h / (nq / nkv);
   const int pos = positions[n];
   const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
 }  // namespace
 
 extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
-                                 const void* v_cache, int cache_dt, const int* positions,
+                                 const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                                  const int* seq_of_token, const int* block_table, int table_stride,
                                  int n, int nq, int nkv, int hd, int page_size, float scale,
                                  int window, hipStream_t stream) {
@@ -117,7 +118,7 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
   PYRE_DISPATCH(q_dt, TQ, PYRE_DISPATCH(cache_dt, TC,
       hipLaunchKernelGGL((attn_generic_kernel<TQ, TC>), dim3(n, nq), dim3(kThreads), 0, stream,
                          static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),
-                         static_cast<const TC*>(v_cache), static_cast<TQ*>(out), positions,
+                         static_cast<const TC*>(v_cache), static_cast<TQ*>(out), tokens, positions,
                          seq_of_token, block_table, table_stride, nq, nkv, hd, page_size, scale,
                          window)));
   return check_launch("attn_generic");

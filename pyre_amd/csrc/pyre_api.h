@@ -65,11 +65,20 @@ int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, floa
 int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
                                int two_i, int K, hipStream_t stream);
 
+// tokens: the n tokens of the flat batch to attend for, or null for tokens 0..n-1.
 int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
-                      const void* v_cache, int cache_dt, const int* positions,
+                      const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                       const int* seq_of_token, const int* block_table, int table_stride, int n,
                       int nq, int nkv, int hd, int page_size, float scale, int window,
                       hipStream_t stream);
+
+// Prompt portions in true float32 on the matrix cores' float32 instruction: tiles as for
+// pyre_attn_prefill_bf16, float32 queries, caches and output, any head size up to 256, any
+// page size. The order of a token's sums depends on its own bounds alone.
+int pyre_attn_prefill_f32(const float* q, float* out, const float* k_cache, const float* v_cache,
+                          const int* tiles, int n_tiles, const int* positions, const int* seq_of_token,
+                          const int* block_table, int table_stride, int nq, int nkv, int hd, int page_size,
+                          float scale, int window, hipStream_t stream);
 
 // 1 if the MFMA attention kernels take this geometry (else use pyre_attn_generic).
 int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv);

@@ -280,9 +280,10 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: t
 def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                  n: int, nq: int, nkv: int, hd: int, page_size: int, scale: float,
-                 window: int = 0) -> None:
-    """Causal attention of n tokens over the paged cache; see attention_generic.hip."""
-    _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table)
+                 window: int = 0, tokens: torch.Tensor | None = None) -> None:
+    """Causal attention of n tokens over the paged cache (``tokens``: which of the flat batch,
+    else the first n); see attention_generic.hip."""
+    _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table, tokens)
     if q.dtype != out.dtype or q.numel() < n * nq * hd or out.numel() < n * nq * hd:
         raise KernelError("attn: q/out buffers do not fit")
     if tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
@@ -291,12 +292,33 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_ca
         raise KernelError("attn: k and v caches differ in element type")
     _contig("q", q), _contig("out", out), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
     _i32("positions", positions, n), _i32("seq_of_token", seq_of_token, n)
+    if tokens is not None:
+        _i32("tokens", tokens, n)
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
         raise KernelError("attn: block table must be int32 [rows, pages]")
     call("pyre_attn_generic", q.data_ptr(), out.data_ptr(), dtype_code(q), k_cache.data_ptr(),
-         v_cache.data_ptr(), dtype_code(k_cache), positions.data_ptr(), seq_of_token.data_ptr(),
+         v_cache.data_ptr(), dtype_code(k_cache), _ptr(tokens), positions.data_ptr(), seq_of_token.data_ptr(),
          block_table.data_ptr(), block_table.stride(0), n, nq, nkv, hd, page_size, float(scale),
          int(window), _stream())
+
+
+def attn_prefill_f32(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,
+                     nq, nkv, hd, page_size, scale, window=0) -> None:
+    """Attention of prompt portions in true float32 on the matrix cores; ``tiles`` is int32
+    [n_tiles, 2] = (first token, count <= 32)."""
+    _dev(q, out, k_cache, v_cache, tiles, positions, seq_of_token, block_table)
+    for name, t in (("q", q), ("out", out), ("k_cache", k_cache), ("v_cache", v_cache)):
+        if t.dtype != torch.float32:
+            raise KernelError(f"attn_prefill_f32: {name} must be float32")
+        _contig(name, t)
+    if tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
+        raise KernelError("attn_prefill_f32: cache shapes do not fit the head geometry")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("attn_prefill_f32: block table must be int32 [rows, pages]")
+    _i32("positions", positions), _i32("seq_of_token", seq_of_token), _i32("tiles", tiles, 2 * n_tiles)
+    call("pyre_attn_prefill_f32", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         tiles.data_ptr(), n_tiles, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+         block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), _stream())
 
 
 ARGMAX_SCRATCH_PER_ROW = 128  #: 4-byte words of scratch per row of logits

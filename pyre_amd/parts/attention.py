@@ -106,7 +106,22 @@ class Attention(Mixer):
                           s.head_dim, cache.page_size)
         o = ws.get("attn.o", (n, self.q_dim), ctx.dtype)
         if not fast.attention(self, ctx, q, o, cache):
-            ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, n,
-                             s.num_heads, s.num_kv_heads, s.head_dim, cache.page_size, self.scale,
-                             cache.window)
+            self._attend_plainly(ctx, q, o, cache)
         return self.out.forward(ctx, o, n)
+
+    def _attend_plainly(self, ctx, q, o, cache) -> None:
+        """The kernels that take every geometry and element type; the whole of the 32-bit path."""
+        s, n = self.spec, ctx.n_tokens
+        k_pages, v_pages = cache["k"], cache["v"]
+        geometry = (s.num_heads, s.num_kv_heads, s.head_dim, cache.page_size, self.scale, cache.window)
+        tiles = ctx.host.arrays["attention.prefill_tiles"]
+        if len(tiles) and q.dtype == torch.float32 and k_pages.dtype == torch.float32:
+            # prompt portions on the matrix cores' float32 instruction, single tokens one by one
+            ops.attn_prefill_f32(q, o, k_pages, v_pages, ctx.arrays["attention.prefill_tiles"], len(tiles),
+                                 ctx.positions, ctx.seq_of_token, cache.table, *geometry)
+            singles = ctx.host.arrays["attention.decode_tokens"]
+            if len(singles):
+                ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, len(singles),
+                                 *geometry, tokens=ctx.arrays["attention.decode_tokens"])
+        else:
+            ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, n, *geometry)

@@ -377,15 +377,54 @@ def test_attn_prefill_mfma(nq, nkv, hd, page, window, form):
     assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("kernel", ["generic32", "generic16", "decode", "prefill"])
+@pytest.mark.parametrize("nq,nkv,hd,page", GENERIC_SHAPES + [(3, 1, 10, 8), (7, 1, 72, 16), (12, 2, 128, 48)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attn_prefill_f32_on_the_matrix_cores(nq, nkv, hd, page, window):
+    """Prompt portions in true float32: any head size and page size, scrambled pages, windows;
+    as close to a float64 result as the one-block-per-token kernel is; a token's result bit for
+    bit the same however its request's tokens are cut into tiles; NaN in pages that the
+    request does not hold changes nothing; generic kernel for listed single tokens."""
+    ops = _ops()
+    ctx_lens, q_lens = [2, 40, 97, 700, 1100], [2, 40, 33, 3, 600]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.float32, seed=6)
+    held = set(table[table >= 0].tolist())
+    for p in range(kc.shape[0]):
+        if p not in held:
+            kc[p], vc[p] = float("nan"), float("nan")
+    scale = hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    ref = torch.empty_like(q)
+    ops.attn_generic(q, ref, kc, vc, pos, seq_of, table, q.shape[0], nq, nkv, hd, page, scale, window)
+    outs = []
+    for width in (32, 7, 19):                                    # tiles of up to `width` tokens
+        tiles, base = [], 0
+        for ql in q_lens:
+            tiles += [(t0, min(width, base + ql - t0)) for t0 in range(base, base + ql, width)]
+            base += ql
+        tiles.append((0, 0))                                     # an empty tile does nothing
+        out = torch.full_like(q, float("nan"))
+        ops.attn_prefill_f32(q, out, kc, vc, i32(tiles).view(-1), len(tiles), pos, seq_of, table, nq, nkv, hd, page, scale, window)
+        assert torch.allclose(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
+        outs.append(out)
+    err, err_ref = (outs[0].double().cpu() - want).abs().max().item(), (ref.double().cpu() - want).abs().max().item()
+    assert err <= 4 * err_ref + 1e-6, (err, err_ref)              # no reduced-precision mode
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    # a list of tokens for the one-by-one kernel: only those rows are written
+    some = [0, 5, 41, q.shape[0] - 1]
+    part = torch.full_like(q, float("nan"))
+    ops.attn_generic(q, part, kc, vc, pos, seq_of, table, len(some), nq, nkv, hd, page, scale, window, tokens=i32(some))
+    assert torch.equal(part[some], ref[some]) and torch.isnan(part[1]).all()
+
+
+@pytest.mark.parametrize("kernel", ["generic32", "generic16", "decode", "prefill", "prefill32"])
 def test_attention_finds_a_far_key(kernel):
     """Random scores would hide a key that is skipped or misplaced: make one far
     key (at a page's first slot, deep in a long context) dominate and check that
     the output is its value."""
     ops = _ops()
     nq, nkv, hd, page = 8, 2, 64, 16
-    dt = torch.float32 if kernel == "generic32" else torch.bfloat16
-    ctx_lens, q_lens = [900], [1 if kernel != "prefill" else 34]
+    dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
+    ctx_lens, q_lens = [900], [1 if not kernel.startswith("prefill") else 34]
     for target in (0, 16 * 20, 16 * 20 + 15, 899 - 34):
         q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=9)
         K, V = dense[0]
@@ -403,6 +442,8 @@ def test_attention_finds_a_far_key(kernel):
         elif kernel == "decode":
             acc, ml = torch.empty(n * nq * 8 * hd, device=DEV), torch.empty(n * nq * 16, device=DEV)
             ops.attn_decode_bf16(q, out, kc, vc, i32([0]), 1, pos, seq_of, table, acc, ml, 8, nq, nkv, hd, page, scale, 0)
+        elif kernel == "prefill32":
+            ops.attn_prefill_f32(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, 0)
         else:
             tiles = [(0, 32), (32, 2)]
             ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), 2, pos, seq_of, table, nq, nkv, hd, page, scale, 0)

@@ -82,6 +82,50 @@ def test_attention_is_the_library_routine():
     assert torch.allclose(w[:, 10], v[:, 7:11].mean(1)) and torch.allclose(w[:, 1], v[:, :2].mean(1))
 
 
+def test_attention_block_scale_biases_and_head_layout():
+    """The block around the attention, pinned where the formulas alone do not: with identity
+    projections it is the library's attention at its default scale head_dim ** -0.5
+    (`pyre/model.py:82,109`: a scale of 1 / head_dim, or one applied before the rotation's
+    table, fails this); q, k and v have biases, the output projection has none
+    (`pyre/model.py:83-87`); head n owns columns n * hd .. (n + 1) * hd - 1 of the projections
+    (`pyre/model.py:92-94`); V is not rotated."""
+    nq, nkv, hd, S = 4, 2, 8, 9
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": hd}
+    H = nq * hd
+    eye = torch.eye(H, dtype=torch.float64)
+    pick = torch.zeros(nkv * hd, H, dtype=torch.float64)      # k and v heads read the columns of q heads 0 and 2
+    for g, src in enumerate((0, 2)):
+        pick[g * hd:(g + 1) * hd, src * hd:(src + 1) * hd] = torch.eye(hd, dtype=torch.float64)
+    w = {"a.q_proj.weight": eye, "a.q_proj.bias": torch.zeros(H, dtype=torch.float64),
+         "a.k_proj.weight": pick, "a.k_proj.bias": torch.zeros(nkv * hd, dtype=torch.float64),
+         "a.v_proj.weight": pick, "a.v_proj.bias": torch.zeros(nkv * hd, dtype=torch.float64),
+         "a.o_proj.weight": eye}
+    h = torch.randn(S, H, dtype=torch.float64)
+    one, zero = torch.ones(S, hd, dtype=torch.float64), torch.zeros(S, hd, dtype=torch.float64)
+    out = P.attention_block(h, w, "a", cfg, one, zero, lambda t: t)           # cos = 1, sin = 0: no rotation
+    q = h.view(S, nq, hd).transpose(0, 1)
+    kv = q[[0, 0, 2, 2]]                                                      # query head i reads kv head i // 2
+    want = torch.nn.functional.scaled_dot_product_attention(q, kv, kv, is_causal=True).transpose(0, 1).reshape(S, H)
+    assert torch.allclose(out, want, atol=1e-12)
+    # the rotation reaches q and k only: with q = k = 0 (zero weights) any table gives the running mean of v
+    cos, sin = P.rope_tables(S, hd, 1e4)
+    w0 = dict(w)
+    w0["a.q_proj.weight"], w0["a.k_proj.weight"] = torch.zeros_like(eye), torch.zeros_like(pick)
+    mean = torch.cumsum(h, 0) / torch.arange(1, S + 1, dtype=torch.float64)[:, None]
+    got = P.attention_block(h, w0, "a", cfg, cos, sin, lambda t: t)
+    assert torch.allclose(got.view(S, nq, hd)[:, 1], mean.view(S, nq, hd)[:, 0], atol=1e-12)   # head 1 reads kv head 0 = columns of q head 0
+    # biases: a v bias passes straight through (the weights of attention sum to 1); an o bias does not exist
+    wb = dict(w0)
+    wb["a.v_proj.bias"] = torch.arange(nkv * hd, dtype=torch.float64)
+    shifted = P.attention_block(h, wb, "a", cfg, cos, sin, lambda t: t)
+    assert torch.allclose((shifted - got).view(S, nq, hd)[:, 3], torch.arange(hd, 2 * hd, dtype=torch.float64).expand(S, hd))
+    wb["a.o_proj.bias"] = torch.full((H,), 7.0, dtype=torch.float64)
+    assert torch.equal(P.attention_block(h, wb, "a", cfg, cos, sin, lambda t: t), shifted)
+    wq = dict(w)
+    wq["a.q_proj.bias"] = torch.randn(H, dtype=torch.float64)
+    assert not torch.allclose(P.attention_block(h, wq, "a", cfg, one, zero, lambda t: t), out)
+
+
 def test_swiglu_is_the_library_routine():
     h = torch.randn(6, 32, dtype=torch.float64)
     w = {"m.gate_proj.weight": torch.randn(40, 32, dtype=torch.float64),

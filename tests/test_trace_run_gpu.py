@@ -18,10 +18,10 @@ pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
 
 
-def run_trace(model_dir, dtype, out_dir, max_tokens, steps):
+def run_trace(model_dir, dtype, out_dir, max_tokens, steps, extra=()):
     proc = subprocess.Popen(
         [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
-         "--out", str(out_dir), "--max-tokens", str(max_tokens)],
+         "--out", str(out_dir), "--max-tokens", str(max_tokens), *extra],
         stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1)
     try:
         for st in steps:
@@ -36,8 +36,9 @@ def run_trace(model_dir, dtype, out_dir, max_tokens, steps):
             proc.kill()
 
 
-@pytest.mark.parametrize("model,dtype", [("tiny-a", "float32"), ("tiny-c", "bfloat16"), ("tiny-b", "bfloat16")])
-def test_trace_run(model, dtype, model_dirs, plain_models, tmp_path):
+@pytest.mark.parametrize("model,dtype,extra", [("tiny-a", "float32", ()), ("tiny-c", "bfloat16", ()), ("tiny-b", "bfloat16", ()),
+                                               ("tiny-b", "float32", ("--page-size", "8", "--max-seqs", "3", "--poison"))])
+def test_trace_run(model, dtype, extra, model_dirs, plain_models, tmp_path):
     plain = plain_models[model]
     vocab = plain[0]["vocab_size"]
     reqs = {"a": random_ids(vocab, 70, 1), "b": random_ids(vocab, 40, 2), "c": random_ids(vocab, 64, 3),
@@ -64,7 +65,7 @@ def test_trace_run(model, dtype, model_dirs, plain_models, tmp_path):
         live = [r for r in live if r not in end]
     steps.append({"step": len(steps), "entries": [], "end": []})          # an empty step is allowed
     out = tmp_path / "out"
-    run_trace(model_dirs[model], dtype, out, 384, steps)
+    run_trace(model_dirs[model], dtype, out, 384, steps, extra)
     ref = {r: plain_logits(plain, ids, torch.bfloat16 if dtype == "bfloat16" else None) for r, ids in reqs.items()}
     checked = 0
     for st, rows in wanted.items():
