@@ -130,7 +130,9 @@ def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
     splits = max(1, min(pieces, DECODE_MAX_SPLITS, target_waves // items))
     # The four waves of a block are four splits: a number that leaves waves of the last block
     # idle is rounded down (five splits would be two blocks and a second kernel to merge them).
-    return splits - splits % 4 if splits > 4 else splits
+    # A block that merges its own waves' results keeps all four of them until the end anyway:
+    # they may as well work, which also shortens the longest request of an uneven batch.
+    return splits - splits % 4 if splits > 4 else min(4, pieces)
 
 
 def attention(mixer, ctx, q, o, cache) -> bool:
