@@ -54,20 +54,34 @@ def model_numbers(cfg, n_layers: int, dtype_bytes: int):
 
 
 def environment() -> dict:
-    """Where and when: device, library versions, the revision of this tree."""
+    """Where and when: device, library versions, the revision of this tree (git's, and a hash of
+    the sources for trees that travel without their history)."""
     import datetime
+    import hashlib
     import os
     import subprocess
 
     import torch
 
+    root = os.path.dirname(os.path.abspath(__file__))
     try:
         sha = subprocess.run(["git", "rev-parse", "--short", "HEAD"], capture_output=True, text=True, timeout=10,
-                             cwd=os.path.dirname(os.path.abspath(__file__))).stdout.strip() or None
+                             cwd=root).stdout.strip() or None
     except (OSError, subprocess.SubprocessError):
         sha = None
-    return {"device": torch.cuda.get_device_name(0), "torch": torch.__version__, "rocm": torch.version.hip,
-            "git": sha, "time": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ")}
+    digest = hashlib.sha1()
+    for folder, _, files in sorted(os.walk(os.path.join(root, "pyre_amd"))):
+        if "_build" in folder or "__pycache__" in folder:
+            continue
+        for f in sorted(files):
+            if f.endswith((".py", ".hip", ".h")):
+                digest.update(open(os.path.join(folder, f), "rb").read())
+    digest.update(open(os.path.abspath(__file__), "rb").read())
+    props = torch.cuda.get_device_properties(0)
+    return {"device": props.name or torch.cuda.get_device_name(0), "arch": getattr(props, "gcnArchName", ""),
+            "compute_units": props.multi_processor_count, "memory_gb": round(props.total_memory / 2**30, 1),
+            "torch": torch.__version__, "rocm": torch.version.hip, "git": sha, "sources_sha1": digest.hexdigest()[:12],
+            "time": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ")}
 
 
 def serve(args) -> int:
