@@ -188,20 +188,20 @@ def test_config_b_workload_against_the_plain_sampler(dtype, model_dirs, plain_mo
 @pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
                                                 ("tiny-b", "float32", True), ("tiny-c", "float32", True)])
 def test_many_live_requests_generate_the_plain_tokens(model, dtype, graphs, model_dirs, plain_models):
-    """20 and then 50 requests of unequal lengths decode together (steps of 17 to 64 rows,
-    padded to their captured sizes), some greedy, some sampled; every token against the
-    plain implementation."""
+    """20, 50 and 150 requests of unequal lengths decode together (steps of 17 to 150 rows,
+    padded to their captured sizes; beyond 64 rows the products are the BLAS library's), some
+    greedy, some sampled; every token against the plain implementation."""
     from pyre_amd.api import Scheduler
 
     plain = plain_models[model]
     vocab = plain[0]["vocab_size"]
-    eng = _load(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=64, max_cached_tokens=64 * 96,
+    eng = _load(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=160, max_cached_tokens=160 * 96,
                 max_num_batched_tokens=512, prefill_chunk=64)
     tol = 1e-5 if dtype == "float32" else 4e-2
-    for count in (20, 50):
+    for count in (20, 50, 150) if graphs and dtype == "bfloat16" else (20, 50):
         prompts = [random_ids(vocab, 3 + (11 * i) % 47, seed=count + i) for i in range(count)]
         new = [6 + (5 * i) % 9 for i in range(count)]         # they end at different steps: the batch shrinks
-        sched = Scheduler(eng, max_batch=64)
+        sched = Scheduler(eng, max_batch=160)
         ids = [sched.add_request(p, n, temperature=0.7 if i % 3 == 0 else 0.0, seed=9) for i, (p, n) in
                enumerate(zip(prompts, new))]
         out = sched.run()

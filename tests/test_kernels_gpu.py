@@ -451,6 +451,52 @@ def test_attention_finds_a_far_key(kernel):
         assert torch.allclose(out.double().cpu(), want.expand(n, nq, hd), atol=3e-2), (kernel, target)
 
 
+@pytest.mark.parametrize("kernel", ["generic32", "generic16", "decode", "prefill", "prefill32"])
+def test_attention_at_a_windows_edge(kernel):
+    """A window of 100 keys: the oldest key that a query still sees dominates its scores, so
+    the output is that key's value; the key just before it dominates even more and must not
+    be seen at all (an off-by-one at the window's edge would return its value instead)."""
+    ops = _ops()
+    nq, nkv, hd, page, window = 8, 2, 64, 16, 100
+    dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
+    ql = 34 if kernel.startswith("prefill") else 1
+    ctx_lens, q_lens = [700], [ql]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=13)
+    K, V = dense[0]
+    q.zero_()
+    q[:, :, 0] = 8.0
+    pages = table[0].tolist()
+    last = 699
+    edge = last - window + 1            # the oldest key the last query sees; the queries before it see it too
+    for key, weight in ((edge, 40.0), (edge - ql, 90.0)):      # the second one lies before every query's window
+        kc[pages[key // page], :, key % page, :] = 0
+        kc[pages[key // page], :, key % page, 0] = weight
+    out = torch.empty_like(q)
+    n, scale = q.shape[0], hd ** -0.5
+    if kernel.startswith("generic"):
+        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, window)
+    elif kernel == "decode":
+        acc, ml = torch.empty(n * nq * 4 * hd, device=DEV), torch.empty(n * nq * 8, device=DEV)
+        ops.attn_decode_bf16(q, out, kc, vc, i32([0]), 1, pos, seq_of, table, acc, ml, 4, nq, nkv, hd, page, scale, window)
+    elif kernel == "prefill32":
+        ops.attn_prefill_f32(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, window)
+    else:
+        ops.attn_prefill_bf16(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, window)
+    want = V[edge].double().repeat_interleave(nq // nkv, 0)
+    assert torch.allclose(out.double().cpu(), want.expand(n, nq, hd), atol=3e-2), kernel
+    # one position on, the edge key itself has left the last query's window: the output is a mixture again
+    if ql == 1:
+        pos2 = pos + 1
+        full = torch.cat([K, torch.zeros(1, nkv, hd, dtype=K.dtype)])
+        kc[pages[(last + 1) // page], :, (last + 1) % page, :] = 0
+        out2 = torch.empty_like(q)
+        if kernel.startswith("generic"):
+            ops.attn_generic(q, out2, kc, vc, pos2, seq_of, table, n, nq, nkv, hd, page, scale, window)
+        else:
+            ops.attn_decode_bf16(q, out2, kc, vc, i32([0]), 1, pos2, seq_of, table, acc, ml, 4, nq, nkv, hd, page, scale, window)
+        assert not torch.allclose(out2.double().cpu(), want.expand(n, nq, hd), atol=0.2)
+
+
 # ----------------------------------------------------------------------------- sampling
 
 def test_argmax_first_of_equals():

@@ -209,6 +209,23 @@ def test_mixed_with_page_reuse_on_poisoned_pages(model, dtype, page, model_dirs,
                                plain_models)
 
 
+@pytest.mark.parametrize("model,dtype,page", [("tiny-c", "bfloat16", 16), ("tiny-b", "float32", 8), ("tiny-a", "bfloat16", 16)])
+def test_long_decoding_against_plain(model, dtype, page, model_dirs, plain_models):
+    """A prompt of five tokens, then 250 tokens one by one (captured steps, replayed): every
+    row against the plain implementation while the context crosses many page ends and the
+    block table grows past its first width."""
+    plain = plain_models[model]
+    ids = random_ids(plain[0]["vocab_size"], 255, seed=77)
+    eng = make_engine(model_dirs[model], dtype, use_graphs=True, page_size=page)
+    steps = [([("a", ids[:5], list(range(5)))], [])]
+    steps += [([("a", ids[i:i + 1], [0])], ["a"] if i == 254 else []) for i in range(5, 255)]
+    got = replay(eng, steps)
+    assert len(got) == 255
+    bad, worst = first_bad(got, {"a": plain_logits(plain, ids, torch.bfloat16 if dtype == "bfloat16" else None)}, TOL[dtype])
+    assert bad is None, bad
+    assert eng.graph_replays > 200
+
+
 def test_weights_stored_in_32_bits_run_in_either_mode(tmp_path, plain_models):
     """A tensor stored in 32 bits stays so: a float32 checkpoint runs in the 16-bit
     mode with float32 weights (mixed products), and exactly in the 32-bit mode."""
