@@ -2,13 +2,14 @@
 // for head sizes that are multiples of 32 up to 256 and page sizes that are
 // multiples of 16. Two kernels share one inner loop on 16x16x32 tiles:
 //
-//   attn_decode_kernel   one new token per request; the keys of a request are
-//                        split over many waves, each with a partial result
-//                        (max, sum, unnormalised output); the four waves of a
-//                        block merge theirs if they are all, else
-//                        attn_decode_reduce does. One wave serves up to 16 query
-//                        heads that share a key/value head, so K and V are read
-//                        once per group.
+//   attn_decode_work_kernel  one new token per request; the keys of a request are
+//                        dealt to blocks of four waves by a work list that the host
+//                        plans in proportion to the contexts, each wave with a
+//                        partial result (max, sum, unnormalised output); the waves
+//                        of a block join theirs through LDS, the blocks of a request
+//                        through memory in the block that finishes last. One wave
+//                        serves up to 16 query heads that share a key/value head, so
+//                        K and V are read once per group.
 //   attn_prefill_kernel  portions of prompts: a wave takes 32 consecutive tokens
 //                        of one request and one query head; the four waves of a
 //                        block take four heads of one key/value head, so their
@@ -271,26 +272,68 @@ __device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge,
 }
 
 // ---------------------------------------------------------------------------
-// Decode: grid (ceil(nsplits / 4), nkv * qtiles, tokens), 4 waves = 4 splits.
+// Decode: grid (capacity of the work list, nkv * qtiles), 4 waves. The host deals the
+// keys of every request to blocks in proportion to its context, so that a step whose
+// requests differ widely in length keeps all compute units busy for the same time:
+//   work[0]     = (blocks in the list, -, -, -)
+//   work[1 + i] = (token in the flat batch, block b of its request + 65536 * blocks nb of its
+//                  request, chunks of 32 keys per wave of this request, first partial slot of
+//                  the request)
+// Block b takes the chunks first + 4 b per .. of its request, a run of `per` chunks for each
+// of its four waves, and joins their results through LDS. A request with one block is
+// finished by it. Otherwise each block stores its joined partial result (max, sum,
+// unnormalised output) at slot (first slot + b) with stores that go through to memory and
+// counts itself in at the request's counter; the block that arrives last reads all nb
+// partial results with loads that come from memory and joins them in the order 0..nb-1,
+// whichever block it is. It leaves the counter at zero. Blocks past the list's end exit.
 // ---------------------------------------------------------------------------
-// ONE_BLOCK: at most four splits, the four waves of a single block: they join their
-// partial results through LDS and store the finished rows in `out`; the partial buffers
-// and the second kernel are not needed.
-template <int HD, bool ONE_BLOCK, bool STREAM_V>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-    const int* __restrict__ tokens, const int* __restrict__ positions,
-    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, bf16* __restrict__ out, int nq, int nkv,
-    int page_size, float scale_log2, int window, int nsplits) {
+constexpr int kMaxBlocksPerRequest = 64;
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16- and 4-byte accesses that go through to memory (buffer instructions with the sc0 and
+// sc1 bits): what one block stores this way, a block on another die reads this way, within
+// one kernel, once the first has waited for its stores and the second has seen a counter move.
+__device__ inline __amdgpu_buffer_rsrc_t rsrc_of(const void* p) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, 0x7fffffff, 0x00020000);
+}
+constexpr int kThrough = 1 | 16;
+__device__ inline void store_through(float* base, int elem, f32x4 v) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rsrc_of(base), 4 * elem, 0, kThrough);
+}
+__device__ inline void store_through(float* base, int elem, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rsrc_of(base), 4 * elem, 0, kThrough);
+}
+__device__ inline f32x4 load_through4(const float* base, int elem) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_of(base), 4 * elem, 0, kThrough));
+}
+__device__ inline float load_through(const float* base, int elem) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_of(base), 4 * elem, 0, kThrough));
+}
+
+#define PYRE_DECODE_WORK_PARAMS                                                                                   \
+  const bf16 *__restrict__ q, const bf16 *__restrict__ k_cache, const bf16 *__restrict__ v_cache,                 \
+      const int4 *__restrict__ work, const int *__restrict__ positions, const int *__restrict__ seq_of_token,     \
+      const int *__restrict__ block_table, int table_stride, float *__restrict__ part_acc,                        \
+      float *__restrict__ part_ml, int *__restrict__ counters, bf16 *__restrict__ out, int nq, int nkv,           \
+      int page_size, float scale_log2, int window
+#define PYRE_DECODE_WORK_ARGS                                                                                     \
+  q, k_cache, v_cache, work, positions, seq_of_token, block_table, table_stride, part_acc, part_ml, counters, out, \
+      nq, nkv, page_size, scale_log2, window
+
+template <int HD, bool STREAM_V>
+__device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) {
+  const int4 head_of_list = work[0];
+  if (static_cast<int>(blockIdx.x) >= head_of_list.x) return;
+  const int4 item = work[1 + blockIdx.x];
+  const int tok = item.x, b = item.y & 0xffff, nb = item.y >> 16, per = item.z, slot0 = item.w;
+  // a list that does not fit the launch is not followed
+  if (nb < 1 || nb > kMaxBlocksPerRequest || b < 0 || b >= nb || slot0 < 0 || slot0 + nb > static_cast<int>(gridDim.x) || per < 1)
+    return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
-  const int split = blockIdx.x * 4 + wave;
-  if (!ONE_BLOCK && split >= nsplits) return;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
   const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
   const int head0 = kvh * n_rep + qt * 16, nheads = min(16, n_rep - qt * 16);
-  const int idx = blockIdx.z, tok = tokens ? tokens[idx] : idx;  // no list: the batch holds single tokens only
   const int pos = positions[tok];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
 
@@ -308,8 +351,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   float m[1] = {-INFINITY}, l[1] = {0.f};
 
   const int first = lo / kChunk, last = pos / kChunk;
-  const int per = (last - first + 1 + nsplits - 1) / nsplits;
-  const int begin = first + split * per, end = split < nsplits ? min(last + 1, begin + per) : begin;
+  const int begin = first + (4 * b + wave) * per, end = min(last + 1, begin + per);  // may be empty
   if constexpr (HD <= 128) {
     // Two register sets: while one chunk is multiplied the next one's loads are in flight.
     ChunkRegs<HD> ra, rb;
@@ -332,80 +374,112 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
   }
 
-  if constexpr (ONE_BLOCK) {
-    // out[head, :] = sum_w o_w 2^(m_w - M) / sum_w l_w 2^(m_w - M), waves in the order 0..3.
-    __shared__ float acc_s[4][16][HD + 4];
-    __shared__ float ml_s[4][16][2];
-    if (g == 0) {
-      ml_s[wave][r][0] = m[0];
-      ml_s[wave][r][1] = l[0];
+  // The block's four waves: sum_w o_w 2^(m_w - M), sum_w l_w 2^(m_w - M), M = max_w m_w, waves in the order 0..3.
+  __shared__ float acc_s[4][16][HD + 4];
+  __shared__ float ml_s[4][16][2];
+  if (g == 0) {
+    ml_s[wave][r][0] = m[0];
+    ml_s[wave][r][1] = l[0];
+  }
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) *reinterpret_cast<f32x4*>(&acc_s[wave][r][dt * 16 + 4 * g]) = o[dt][0];
+  __syncthreads();
+  const int n_items = gridDim.y;
+  float* pa = part_acc + (static_cast<size_t>(slot0 + b) * n_items + blockIdx.y) * 16 * HD;
+  float* pm = part_ml + (static_cast<size_t>(slot0 + b) * n_items + blockIdx.y) * 32;
+  for (int i = threadIdx.x; i < nheads * (HD / 4); i += 256) {
+    const int h = i / (HD / 4), d = 4 * (i % (HD / 4));
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_s[w][h][0]);
+    float L = 0.f;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = ml_s[w][h][0];
+      const float ww = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+      L += ml_s[w][h][1] * ww;
+      sum += *reinterpret_cast<const f32x4*>(&acc_s[w][h][d]) * ww;
     }
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) *reinterpret_cast<f32x4*>(&acc_s[wave][r][dt * 16 + 4 * g]) = o[dt][0];
-    __syncthreads();
-    for (int i = threadIdx.x; i < nheads * (HD / 4); i += 256) {
-      const int h = i / (HD / 4), d = 4 * (i % (HD / 4));
-      float M = -INFINITY;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_s[w][h][0]);
-      float L = 0.f;
-      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const float mw = ml_s[w][h][0];
-        const float ww = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
-        L += ml_s[w][h][1] * ww;
-        sum += *reinterpret_cast<const f32x4*>(&acc_s[w][h][d]) * ww;
-      }
+    if (nb == 1) {
       // L is 0 only for a row that sees no key at all (padding of a captured step).
       const float inv = L > 0.f ? 1.f / L : 0.f;
       *reinterpret_cast<uint2*>(out + (static_cast<size_t>(tok) * nq + head0 + h) * HD + d) =
           uint2{pack2(sum[0] * inv, sum[1] * inv), pack2(sum[2] * inv, sum[3] * inv)};
+    } else {
+      store_through(pa, h * HD + d, sum);
+      if (d == 0) {
+        store_through(pm, 2 * h, M);
+        store_through(pm, 2 * h + 1, L);
+      }
     }
-  } else if (r < nheads) {
-    const size_t slot = (static_cast<size_t>(idx) * nq + head0 + r) * nsplits + split;
-    if (g == 0) {
-      part_ml[2 * slot] = m[0];
-      part_ml[2 * slot + 1] = l[0];
-    }
+  }
+  if (nb == 1) return;
+
+  // Count this block in once all its stores have arrived; the last one joins the request's blocks.
+  __shared__ int last_s;
+  __shared__ float ml_all[kMaxBlocksPerRequest][16][2];
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int* counter = counters + static_cast<size_t>(slot0) * n_items + blockIdx.y;
+    const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last_s = before == nb - 1;
+    if (last_s) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!last_s) return;
+  const float* pa0 = part_acc + (static_cast<size_t>(slot0) * n_items + blockIdx.y) * 16 * HD;
+  const float* pm0 = part_ml + (static_cast<size_t>(slot0) * n_items + blockIdx.y) * 32;
+  const int acc_step = n_items * 16 * HD, ml_step = n_items * 32;  // floats from one block's slot to the next
+  for (int i = threadIdx.x; i < nb * 32; i += 256) {
+    const int bb = i >> 5, j = i & 31;
+    ml_all[bb][j >> 1][j & 1] = load_through(pm0 + static_cast<size_t>(bb) * ml_step, j);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nheads * (HD / 4); i += 256) {
+    const int h = i / (HD / 4), d = 4 * (i % (HD / 4));
+    float M = -INFINITY;
+    for (int bb = 0; bb < nb; ++bb) M = fmaxf(M, ml_all[bb][h][0]);
+    float L = 0.f;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    constexpr int kAtOnce = 8;  // loads in flight
+    for (int b0 = 0; b0 < nb; b0 += kAtOnce) {
+      f32x4 v[kAtOnce];
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt)
-      *reinterpret_cast<f32x4*>(part_acc + slot * HD + dt * 16 + 4 * g) = o[dt][0];
+      for (int u = 0; u < kAtOnce; ++u)
+        if (b0 + u < nb) v[u] = load_through4(pa0 + static_cast<size_t>(b0 + u) * acc_step, h * HD + d);
+#pragma unroll
+      for (int u = 0; u < kAtOnce; ++u)
+        if (b0 + u < nb) {
+          const float mb = ml_all[b0 + u][h][0];
+          const float wb = mb == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mb - M);
+          L += ml_all[b0 + u][h][1] * wb;
+          sum += v[u] * wb;
+        }
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    *reinterpret_cast<uint2*>(out + (static_cast<size_t>(tok) * nq + head0 + h) * HD + d) =
+        uint2{pack2(sum[0] * inv, sum[1] * inv), pack2(sum[2] * inv, sum[3] * inv)};
   }
 }
 
-// out[token, head, :] = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s.
-// One block per (token, head); the weights of the splits are formed once in LDS.
-constexpr int kMaxSplits = 128;
-
-template <int HD>
-__global__ __launch_bounds__(128) void attn_decode_reduce(const float* __restrict__ part_acc,
-                                                          const float* __restrict__ part_ml,
-                                                          const int* __restrict__ tokens,
-                                                          bf16* __restrict__ out, int nq, int nsplits) {
-  __shared__ float w[kMaxSplits];
-  __shared__ float scratch[16];
-  const int idx = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
-  const size_t base = (static_cast<size_t>(idx) * nq + head) * nsplits;
-  float ms = -INFINITY, ls = 0.f;
-  if (tid < nsplits) {
-    const float2 v = *reinterpret_cast<const float2*>(part_ml + 2 * (base + tid));
-    ms = v.x;
-    ls = v.y;
-  }
-  const float M = block_max(ms, scratch);
-  const float ws = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
-  if (tid < nsplits) w[tid] = ws;
-  const float L = block_sum(ls * ws, scratch);  // its barriers publish w[]
-  const int tok = tokens ? tokens[idx] : idx;
-  for (int d = tid; d < HD; d += 128) {
-    float acc = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < nsplits; ++s) acc += part_acc[(base + s) * HD + d] * w[s];
-    // L is 0 only for a row that sees no key at all (padding of a captured step).
-    out[(static_cast<size_t>(tok) * nq + head) * HD + d] = from_float<bf16>(L > 0.f ? acc / L : 0.f);
-  }
+// Two forms of the kernel. The registers of a wave (two chunks of keys and values in flight)
+// leave room for two waves per SIMD. When the step has so few requests that a block per
+// compute unit covers them, a second block on the same unit would leave another unit idle
+// (the dispatcher fills units in order): that form keeps a unit to one block. With more
+// requests than units, two blocks per unit hide each other's latencies at start and end.
+template <int HD, bool STREAM_V>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_decode_work_alone_kernel(
+    PYRE_DECODE_WORK_PARAMS) {
+  attn_decode_work_block<HD, STREAM_V>(PYRE_DECODE_WORK_ARGS);
 }
+template <int HD, bool STREAM_V>
+__global__ __launch_bounds__(256, 2) void attn_decode_work_kernel(PYRE_DECODE_WORK_PARAMS) {
+  attn_decode_work_block<HD, STREAM_V>(PYRE_DECODE_WORK_ARGS);
+}
+#undef PYRE_DECODE_WORK_PARAMS
+#undef PYRE_DECODE_WORK_ARGS
 
 // ---------------------------------------------------------------------------
 // Prefill: grid (tiles, nkv * head groups); wave w takes head group*4 + w.
@@ -869,44 +943,38 @@ extern "C" int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv) {
          nq % nkv == 0;
 }
 
-extern "C" int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache,
-                                     const void* v_cache, const int* tokens, int n_tokens,
-                                     const int* positions, const int* seq_of_token,
-                                     const int* block_table, int table_stride, float* part_acc,
-                                     float* part_ml, int nsplits, int nq, int nkv, int hd,
-                                     int page_size, float scale, int window, hipStream_t stream) {
+extern "C" int pyre_attn_decode_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                                          const int* work, int capacity, const int* positions,
+                                          const int* seq_of_token, const int* block_table, int table_stride,
+                                          float* part_acc, float* part_ml, int* counters, int alone, int nq,
+                                          int nkv, int hd, int page_size, float scale, int window,
+                                          hipStream_t stream) {
   PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
-               "attn_decode_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
+               "attn_decode_work_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
-  PYRE_REQUIRE(nsplits >= 1 && nsplits <= kMaxSplits && table_stride > 0,
-               "attn_decode_bf16: split count %d is outside 1..%d, or bad table", nsplits, kMaxSplits);
-  if (n_tokens <= 0) return 0;
+  PYRE_REQUIRE(table_stride > 0 && capacity >= 0, "attn_decode_work_bf16: bad table or capacity");
+  PYRE_REQUIRE(reinterpret_cast<uintptr_t>(work) % 16 == 0, "attn_decode_work_bf16: the work list must lie on 16 bytes");
+  if (capacity == 0) return 0;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
-  PYRE_REQUIRE(n_tokens <= 65535 && nkv * qtiles <= 65535, "attn_decode_bf16: grid too large");
-  const dim3 grid((nsplits + 3) / 4, nkv * qtiles, n_tokens);
+  PYRE_REQUIRE(nkv * qtiles <= 65535, "attn_decode_work_bf16: grid too large");
+  const dim3 grid(capacity, nkv * qtiles);
   const float scale_log2 = scale * kLog2e;
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
-    auto launch = [&](auto one_block, auto stream_v) {
-      hipLaunchKernelGGL((attn_decode_kernel<HD, decltype(one_block)::value, decltype(stream_v)::value>), grid,
-                         dim3(256), 0, stream, static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),
-                         static_cast<const bf16*>(v_cache), tokens, positions, seq_of_token, block_table,
-                         table_stride, part_acc, part_ml, static_cast<bf16*>(out), nq, nkv, page_size,
-                         scale_log2, window, nsplits);
+    auto launch = [&](auto stream_v) {
+      constexpr bool SV = decltype(stream_v)::value;
+      auto kernel = alone ? attn_decode_work_alone_kernel<HD, SV> : attn_decode_work_kernel<HD, SV>;
+      hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
+                         static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache),
+                         reinterpret_cast<const int4*>(work), positions, seq_of_token, block_table, table_stride,
+                         part_acc, part_ml, counters, static_cast<bf16*>(out), nq, nkv, page_size, scale_log2,
+                         window);
     };
-    const bool stream_v = page_size <= 32;
-    if (nsplits <= 4) {  // one block per (token, key/value head): its waves join their results themselves
-      if (stream_v) launch(std::true_type{}, std::true_type{});
-      else launch(std::true_type{}, std::false_type{});
-      return;
-    }
-    if (stream_v) launch(std::false_type{}, std::true_type{});
-    else launch(std::false_type{}, std::false_type{});
-    hipLaunchKernelGGL(attn_decode_reduce<HD>, dim3(n_tokens, nq), dim3(128), 0, stream,
-                       part_acc, part_ml, tokens, static_cast<bf16*>(out), nq, nsplits);
+    if (page_size <= 32) launch(std::true_type{});
+    else launch(std::false_type{});
   });
-  PYRE_REQUIRE(rc == 0, "attn_decode_bf16: no kernel for head_dim %d", hd);
-  return check_launch("attn_decode_bf16");
+  PYRE_REQUIRE(rc == 0, "attn_decode_work_bf16: no kernel for head_dim %d", hd);
+  return check_launch("attn_decode_work_bf16");
 }
 
 extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache,

@@ -83,14 +83,24 @@ int pyre_attn_prefill_f32(const float* q, float* out, const float* k_cache, cons
 // 1 if the MFMA attention kernels take this geometry (else use pyre_attn_generic).
 int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv);
 
-// One new token per request. tokens[i] indexes the flat batch (null: token i itself, a batch
-// of single tokens only, which saves every wave a dependent load); part_acc is
-// [n_tokens, nq, nsplits, hd] floats and part_ml [n_tokens, nq, nsplits, 2] of scratch.
-int pyre_attn_decode_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
-                          const int* tokens, int n_tokens, const int* positions,
-                          const int* seq_of_token, const int* block_table, int table_stride,
-                          float* part_acc, float* part_ml, int nsplits, int nq, int nkv, int hd,
-                          int page_size, float scale, int window, hipStream_t stream);
+// One new token per request, from a work list that deals every request's keys to blocks of
+// four waves:
+// work[0] = (blocks in the list, 0, 0, 0), work[1 + i] = (token in the flat batch, block b of
+// its request + 65536 * blocks nb of its request (<= 64), chunks `per` of 32 keys that a wave
+// of this request takes, the request's first partial slot); block b takes chunks 4 b per ..
+// 4 (b + 1) per - 1 of its request, counted from the first chunk that the token sees, and the
+// nb blocks of a request cover all of them. The slots of the requests are disjoint runs of nb
+// within 0..capacity-1. `alone`: a compute unit runs one block at a time (for steps of so few
+// requests that a block per unit covers them); else two. The launch has
+// `capacity` blocks per key/value head (and group of 16 query heads); blocks past the list's
+// end exit. Scratch: part_acc [capacity, items, 16, hd] and part_ml [capacity, items, 16, 2]
+// floats, counters [capacity, items] ints that are zero before the first call and are left
+// at zero, items = nkv * ceil(nq / nkv / 16).
+int pyre_attn_decode_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                               const int* work, int capacity, const int* positions,
+                               const int* seq_of_token, const int* block_table, int table_stride,
+                               float* part_acc, float* part_ml, int* counters, int alone, int nq, int nkv,
+                               int hd, int page_size, float scale, int window, hipStream_t stream);
 
 // Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
 // all tokens of a tile from one request at consecutive positions. Heads of up to 128

@@ -83,8 +83,11 @@ class HostBatch:
         return rows, width * ps
 
     def attach(self, specs) -> "HostBatch":
-        """Build the arrays that the parts asked for."""
-        self.arrays = {s.name: np.ascontiguousarray(s.build(self), dtype=np.int32) for s in specs}
+        """Build the arrays that the parts asked for, in the order given: a later one may
+        be made from an earlier one."""
+        self.arrays = {}
+        for s in specs:
+            self.arrays[s.name] = np.ascontiguousarray(s.build(self), dtype=np.int32)
         return self
 
 

@@ -9,7 +9,7 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
-from pyre_amd.engine.batch import HostBatch
+from pyre_amd.engine.batch import HostBatch, round_decode_shape
 
 TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -29,7 +29,8 @@ class Workspace:
         self.keep_replaced = False
         self._replaced: list[torch.Tensor] = []
 
-    def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+    def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype, zeroed: bool = False) -> torch.Tensor:
+        """``zeroed``: the buffer is zero when it is made (and whoever uses it leaves it so)."""
         shape = tuple(shape)
         view = self._views.get((name, dtype, shape))
         if view is not None:
@@ -42,7 +43,7 @@ class Workspace:
                 raise RuntimeError(f"workspace buffer {name!r} would have to grow inside a captured step")
             if buf is not None and self.keep_replaced:
                 self._replaced.append(buf)
-            buf = torch.empty(numel, device=self.device, dtype=dtype)
+            buf = (torch.zeros if zeroed else torch.empty)(numel, device=self.device, dtype=dtype)
             self._bufs[key] = buf
             for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
                 del self._views[k]  # views of the buffer that this one replaces
@@ -86,8 +87,9 @@ def meta_layout(n_cap: int, s_cap: int, table_widths: list[int], extra=()) -> tu
 
     for name in ("tokens", "positions", "seq_of_token", "logit_rows", "token_src"):
         put(name, n_cap)
+    rows = round_decode_shape(s_cap, 1)[0]  # a part may plan single-token requests for the rounded number of them
     for spec in extra:
-        put("x:" + spec.name, int(spec.capacity(n_cap, s_cap)))
+        put("x:" + spec.name, int(spec.capacity(n_cap, rows)))
     put("q_start", s_cap + 1)
     put("ctx_len", s_cap)
     put("state_slots", s_cap)

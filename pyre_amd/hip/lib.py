@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class KernelError(RuntimeError):
@@ -33,7 +33,7 @@ _SIGNATURES = {
     "pyre_attn_generic": [P, P, I, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_f32": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_mfma_supports": [I, I, I, I],
-    "pyre_attn_decode_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
+    "pyre_attn_decode_work_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
     "pyre_argmax_static": [P, L, P, I, I, P],

@@ -399,22 +399,25 @@ def _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table,
     _i32("positions", positions), _i32("seq_of_token", seq_of_token)
 
 
-def attn_decode_bf16(q, out, k_cache, v_cache, tokens, n_tokens, positions, seq_of_token, block_table,
-                     part_acc, part_ml, nsplits, nq, nkv, hd, page_size, scale, window=0) -> None:
-    """Attention of ``n_tokens`` single new tokens (``tokens`` indexes the flat
-    batch; None: the batch is these tokens, in order) over the paged cache, keys split
-    ``nsplits`` ways."""
+def attn_decode_work_bf16(q, out, k_cache, v_cache, work, capacity, positions, seq_of_token, block_table,
+                          part_acc, part_ml, counters, alone, nq, nkv, hd, page_size, scale, window=0) -> None:
+    """Attention of single new tokens over the paged cache from a work list (int32
+    ``[1 + blocks, 4]``: see ``pyre_attn_decode_work_bf16`` in pyre_api.h) in a launch of
+    ``capacity`` blocks per key/value head, one (``alone``) or two to a compute unit.
+    ``counters`` must be zero and is left at zero."""
     _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
-    if tokens is not None:
-        _i32("tokens", tokens, n_tokens)
-    if part_acc.dtype != torch.float32 or part_acc.numel() < n_tokens * nq * nsplits * hd:
-        raise KernelError("attn_decode: partial accumulators too small")
-    if part_ml.dtype != torch.float32 or part_ml.numel() < n_tokens * nq * nsplits * 2:
-        raise KernelError("attn_decode: partial max/sum buffer too small")
-    call("pyre_attn_decode_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-         _ptr(tokens), n_tokens, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
-         block_table.stride(0), part_acc.data_ptr(), part_ml.data_ptr(), nsplits, nq, nkv, hd, page_size,
-         float(scale), int(window), _stream())
+    _i32("work", work, 4 * (1 + capacity))
+    items = nkv * -(-(nq // nkv) // 16)
+    if part_acc.dtype != torch.float32 or part_acc.numel() < capacity * items * 16 * hd:
+        raise KernelError("attn_decode_work: partial accumulators too small")
+    if part_ml.dtype != torch.float32 or part_ml.numel() < capacity * items * 32:
+        raise KernelError("attn_decode_work: partial max/sum buffer too small")
+    if counters.dtype != torch.int32 or counters.numel() < capacity * items:
+        raise KernelError("attn_decode_work: too few counters")
+    call("pyre_attn_decode_work_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         work.data_ptr(), capacity, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+         block_table.stride(0), part_acc.data_ptr(), part_ml.data_ptr(), counters.data_ptr(), int(bool(alone)), nq,
+         nkv, hd, page_size, float(scale), int(window), _stream())
 
 
 def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,

@@ -131,7 +131,8 @@ class StepArraySpec:
     """An int32 array that a part's kernels need of every step beside the common ones
     (tokens, positions, block tables, ...): work lists, tiles, anything that follows from
     the step's batch. ``build(host_batch)`` returns it (numpy int32, any shape);
-    ``capacity(max_tokens, max_seqs)`` bounds its number of elements. The engine builds it
+    ``capacity(max_tokens, max_seqs)`` bounds its number of elements
+    (``max_seqs`` as ``HostBatch.decode_shape`` rounds the number of single-token requests). The engine builds it
     on the host, uploads it in the step's one copy and hands it to the parts as
     ``ctx.arrays[name]`` (device) and ``ctx.host.arrays[name]`` (host). Parts that name the
     same array share it."""

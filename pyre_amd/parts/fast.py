@@ -10,6 +10,7 @@ never comes here.
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from pyre_amd.hip.ops import Partials
@@ -112,27 +113,92 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
     return True
 
 
-#: waves the split of decode attention aims at: the kernel holds two chunks of keys and
-#: values in registers, which leaves room for one wave on each of the 1,024 SIMDs; measured,
-#: time jumps as soon as a second round of waves is needed
-DECODE_TARGET_WAVES = 1024
-#: a split takes at least this many keys (two chunks)
-DECODE_MIN_KEYS_PER_SPLIT = 64
-DECODE_MAX_SPLITS = 128
+#: compute units; a unit runs one block of the decode kernel at a time, or two
+DECODE_UNITS = 256
+#: keys per chunk of the decode kernel, and the fewest chunks a block is given if its request has them
+DECODE_CHUNK = 32
+DECODE_MIN_CHUNKS_PER_BLOCK = 8
+#: the most blocks that share one request (the kernel's limit)
+DECODE_MAX_BLOCKS_PER_REQUEST = 64
 
 
-def decode_splits(n_tokens: int, nq: int, nkv: int, max_ctx: int, window: int,
-                  target_waves: int = DECODE_TARGET_WAVES) -> int:
-    """How many ways to split each request's keys so that the chip is full but not overfull."""
-    span = min(max_ctx, window + 32) if window > 0 else max_ctx
-    pieces = max(1, -(-span // DECODE_MIN_KEYS_PER_SPLIT))
-    items = n_tokens * nkv * -(-(nq // nkv) // 16)
-    splits = max(1, min(pieces, DECODE_MAX_SPLITS, target_waves // items))
-    # The four waves of a block are four splits: a number that leaves waves of the last block
-    # idle is rounded down (five splits would be two blocks and a second kernel to merge them).
-    # A block that merges its own waves' results keeps all four of them until the end anyway:
-    # they may as well work, which also shortens the longest request of an uneven batch.
-    return splits - splits % 4 if splits > 4 else min(4, pieces)
+def decode_items(nq: int, nkv: int) -> int:
+    """Independent pieces of one request's attention: key/value heads times groups of 16 query heads."""
+    return nkv * -(-(nq // nkv) // 16)
+
+
+def decode_alone(rows: int, nq: int, nkv: int) -> bool:
+    """Whether a step of ``rows`` single-token requests runs one block per compute unit: a
+    block for every request and item then fits the chip at once. (Measured on the 7B heads:
+    64 requests of 4,096 tokens take 79 us that way and 87 to 115 us with two blocks a unit,
+    which the dispatcher does not spread evenly; 256 requests take 405 and 332 us.)"""
+    return rows * decode_items(nq, nkv) <= DECODE_UNITS
+
+
+def _decode_slots(rows: int, nq: int, nkv: int) -> int:
+    """Blocks per item that run at once."""
+    at_once = DECODE_UNITS if decode_alone(rows, nq, nkv) else 2 * DECODE_UNITS
+    return max(1, at_once // decode_items(nq, nkv))
+
+
+def decode_capacity(rows: int, nq: int, nkv: int) -> int:
+    """Blocks that the work list of a step with ``rows`` single-token requests can come to."""
+    return rows + 2 * _decode_slots(rows, nq, nkv) + 1
+
+
+def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: int, nq: int, nkv: int,
+                size: int | None = None) -> np.ndarray:
+    """The decode kernel's work list (int32 ``[1 + blocks, 4]``) for the single tokens
+    ``tokens`` (flat indices) at ``positions``, planned as for ``rows`` requests (the rounded
+    number: the missing ones count as requests of one chunk, which is what the padding of a
+    captured step is, so that an eager step and a replayed one split alike).
+
+    A request of c chunks of 32 keys gets ceil(c / size) blocks of four waves and deals its
+    chunks evenly to them. The chip runs ``slots`` blocks per key/value item at once. If all
+    blocks can run in one round, ``size`` is the smallest at which they do: the step then
+    takes as long as one block. Otherwise (or if that is slower) ``size`` is half of what a
+    slot has to work off in all, and the list starts with the longest requests, so that the
+    rounds stay full to the end. Row 0 is (blocks, 0, 0, 0), row 1 + i is (token, block of its
+    request + 65536 * blocks of its request, chunks per wave, first partial slot of the
+    request). ``size`` fixes the block size instead (for tests of the kernel)."""
+    n = len(tokens)
+    if n == 0:
+        return np.zeros((1, 4), dtype=np.int32)
+    pos = positions[tokens].astype(np.int64)
+    lo = np.maximum(0, pos - window + 1) if window > 0 else np.zeros_like(pos)
+    chunks = pos // DECODE_CHUNK - lo // DECODE_CHUNK + 1
+    padding = max(0, rows - n)
+    total, longest = int(chunks.sum()) + padding, int(chunks.max())
+    slots = _decode_slots(rows, nq, nkv)
+    if size is None:
+        size = -(-total // (2 * slots))  # many rounds: half a slot's share
+        if n + padding <= slots:
+            a, b = 1, longest  # the smallest block size at which one round holds all blocks
+            while a < b:
+                mid = (a + b) // 2
+                if int((-(-chunks // mid)).sum()) + padding <= slots:
+                    b = mid
+                else:
+                    a = mid + 1
+            if a <= 3 * size:  # one round of blocks of a, against total / slots + size for many rounds
+                size = a
+        size = max(size, DECODE_MIN_CHUNKS_PER_BLOCK)
+    size = max(size, -(-longest // DECODE_MAX_BLOCKS_PER_REQUEST))
+    nb = -(-chunks // size)
+    per = -(-chunks // (4 * nb))
+    nb = -(-chunks // (4 * per))  # blocks that are left without a chunk by the rounding are dropped
+    order = np.argsort(-chunks, kind="stable")
+    nb_sorted = nb[order]
+    first = np.cumsum(nb_sorted) - nb_sorted
+    n_blocks = int(nb_sorted.sum())
+    which = np.repeat(np.arange(n), nb_sorted)
+    work = np.empty((1 + n_blocks, 4), dtype=np.int32)
+    work[0] = (n_blocks, 0, 0, 0)
+    work[1:, 0] = tokens[order][which]
+    work[1:, 1] = np.arange(n_blocks) - first[which] + 65536 * nb_sorted[which]
+    work[1:, 2] = per[order][which]
+    work[1:, 3] = first[which]
+    return work
 
 
 def attention(mixer, ctx, q, o, cache) -> bool:
@@ -150,19 +216,19 @@ def attention(mixer, ctx, q, o, cache) -> bool:
     dec, tiles = hb.arrays["attention.decode_tokens"], hb.arrays["attention.prefill_tiles"]
     n_dec, n_tiles = len(dec), len(tiles)
     if n_dec:
-        # The split is chosen from the step's rounded sizes, so that a step gives bit for bit
-        # the same result whether it runs eagerly or as a replayed graph at those sizes.
-        rows, span = hb.decode_shape()
-        nsplits = ctx.runtime.options.get("decode_splits") or decode_splits(
-            rows, s.num_heads, s.num_kv_heads, span, cache.window,
-            ctx.runtime.options.get("decode_target_waves", DECODE_TARGET_WAVES))
-        acc = ctx.workspace.get("attn.part_acc", (n_dec, s.num_heads, nsplits, s.head_dim), torch.float32)
-        ml = ctx.workspace.get("attn.part_ml", (n_dec, s.num_heads, nsplits, 2), torch.float32)
-        # a batch of single tokens only needs no list of them
-        which = None if n_dec == ctx.n_tokens else ctx.arrays["attention.decode_tokens"]
-        ops.attn_decode_bf16(q, o, k_pages, v_pages, which, n_dec, ctx.positions,
-                             ctx.seq_of_token, cache.table, acc, ml, nsplits, s.num_heads, s.num_kv_heads,
-                             s.head_dim, cache.page_size, mixer.scale, cache.window)
+        # The launch's size follows from the step's rounded sizes and the list from the rounded
+        # number of requests, so that a step gives bit for bit the same result whether it runs
+        # eagerly or as a replayed graph at those sizes.
+        rows, _ = hb.decode_shape()
+        capacity = decode_capacity(rows, s.num_heads, s.num_kv_heads)
+        items = decode_items(s.num_heads, s.num_kv_heads)
+        acc = ctx.workspace.get("attn.part_acc", (capacity, items, 16, s.head_dim), torch.float32)
+        ml = ctx.workspace.get("attn.part_ml", (capacity, items, 16, 2), torch.float32)
+        counters = ctx.workspace.get("attn.counters", (capacity, items), torch.int32, zeroed=True)
+        ops.attn_decode_work_bf16(q, o, k_pages, v_pages, ctx.arrays[mixer.decode_work_name], capacity, ctx.positions,
+                                  ctx.seq_of_token, cache.table, acc, ml, counters,
+                                  decode_alone(rows, s.num_heads, s.num_kv_heads), s.num_heads, s.num_kv_heads,
+                                  s.head_dim, cache.page_size, mixer.scale, cache.window)
     if n_tiles:
         ops.attn_prefill_bf16(q, o, k_pages, v_pages, ctx.arrays["attention.prefill_tiles"], n_tiles, ctx.positions,
                               ctx.seq_of_token, cache.table, s.num_heads, s.num_kv_heads, s.head_dim,

@@ -7,6 +7,7 @@ from __future__ import annotations
 import math
 import random
 
+import numpy as np
 import pytest
 import torch
 
@@ -339,8 +340,8 @@ MFMA_SHAPES = [(28, 4, 128, 16), (8, 8, 64, 16), (6, 1, 32, 32), (40, 2, 96, 16)
 
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 50])
-@pytest.mark.parametrize("nsplits", [1, 3, 16])
-def test_attn_decode_mfma(nq, nkv, hd, page, window, nsplits):
+@pytest.mark.parametrize("size", [None, 5, 100])
+def test_attn_decode_mfma(nq, nkv, hd, page, window, size):
     ops = _ops()
     assert ops.attn_mfma_supports(hd, page, nq, nkv)
     ctx_lens = [1, 31, 32, 33, 700, 2049]
@@ -348,13 +349,106 @@ def test_attn_decode_mfma(nq, nkv, hd, page, window, nsplits):
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=3)
     n = q.shape[0]
     out = torch.full_like(q, float("nan"))
-    acc = torch.empty(n * nq * nsplits * hd, device=DEV)
-    ml = torch.empty(n * nq * nsplits * 2, device=DEV)
-    toks = i32(list(range(n)))
     scale = hd ** -0.5
-    ops.attn_decode_bf16(q, out, kc, vc, toks, n, pos, seq_of, table, acc, ml, nsplits, nq, nkv, hd, page, scale, window)
+    decode_attention(ops, q, out, kc, vc, range(n), pos, seq_of, table, nq, nkv, hd, page, scale, window, size=size)
     want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
     assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
+
+
+def decode_attention(ops, q, out, kc, vc, tokens, pos, seq_of, table, nq, nkv, hd, page, scale, window=0, size=None,
+                     rows=None, alone=None):
+    """The decode kernel on the single tokens ``tokens`` with a list planned as the engine plans it."""
+    from pyre_amd.parts.fast import decode_alone, decode_capacity, decode_items, decode_work
+
+    tokens = np.asarray(tokens, dtype=np.int32)
+    rows = rows or len(tokens)
+    work = decode_work(tokens, pos.cpu().numpy(), rows, window, nq, nkv, size=size)
+    cap, items = max(decode_capacity(rows, nq, nkv), int(work[0, 0])), decode_items(nq, nkv)
+    acc = torch.full((cap * items * 16 * hd,), float("nan"), device=DEV)
+    ml = torch.full((cap * items * 32,), float("nan"), device=DEV)
+    counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
+    alone = decode_alone(rows, nq, nkv) if alone is None else alone
+    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap), cap, pos, seq_of, table, acc, ml, counters,
+                              alone, nq, nkv, hd, page, scale, window)
+    assert int(counters.abs().sum()) == 0
+    return work
+
+
+def work_on_device(work, cap, fill=0):
+    """The list in a buffer as large as the launch: the rows past its end are never read."""
+    flat = np.full(4 * (1 + cap), fill, dtype=np.int32)
+    flat[:work.size] = work.reshape(-1)
+    return i32(flat.tolist())
+
+
+@pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 50])
+@pytest.mark.parametrize("size,alone", [(None, True), (4, False), (12, True), (None, False)])
+def test_attn_decode_from_a_work_list(nq, nkv, hd, page, window, size, alone):
+    """Requests of very different lengths, their keys dealt to blocks by the planner (or
+    4 or 12 chunks per block: the longest requests then span many blocks that join
+    through memory). The second call finds the counters as the first left them; the third
+    plans for a larger step, as a captured one would, and must give the same bits."""
+    ops = _ops()
+    from pyre_amd.parts.fast import decode_capacity, decode_items, decode_work
+
+    ctx_lens = [1, 31, 32, 33, 700, 2049, 129, 5]
+    q_lens = [1] * len(ctx_lens)
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=3)
+    n, scale = q.shape[0], hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    rows = 8
+    cap, items = decode_capacity(rows, nq, nkv), decode_items(nq, nkv)
+    if size is not None:
+        cap = 600
+    acc = torch.full((cap * items * 16 * hd,), float("nan"), device=DEV)
+    ml = torch.full((cap * items * 32,), float("nan"), device=DEV)
+    counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
+    tokens = np.arange(n, dtype=np.int32)
+    work = decode_work(tokens, pos.cpu().numpy(), rows, window, nq, nkv, size=size)
+    assert work[0, 0] <= cap
+    if size is not None and window == 0:
+        assert work[1, 1] // 65536 > 4                            # the longest request spans many blocks
+    outs = []
+    for _ in range(2):
+        out = torch.full_like(q, float("nan"))
+        ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap), cap, pos, seq_of, table, acc, ml,
+                                  counters, alone, nq, nkv, hd, page, scale, window)
+        assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
+        assert int(counters.abs().sum()) == 0
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    # what lies past the list's end is not followed
+    out = torch.full_like(q, float("nan"))
+    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap, fill=-7), cap, pos, seq_of, table, acc, ml,
+                              counters, alone, nq, nkv, hd, page, scale, window)
+    assert torch.equal(out, outs[0])
+
+
+def test_attn_decode_work_list_in_a_mixed_batch():
+    """Single tokens between the tokens of prompt portions: the list names them by their
+    place in the flat batch, and nothing else is written."""
+    ops = _ops()
+    from pyre_amd.parts.fast import decode_capacity, decode_items, decode_work
+
+    nq, nkv, hd, page = 28, 4, 128, 16
+    ctx_lens, q_lens = [300, 40, 1500, 64, 9], [1, 7, 1, 33, 1]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=8)
+    scale = hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale)
+    singles = np.asarray([0, 8, 42], dtype=np.int32)
+    cap, items = decode_capacity(4, nq, nkv), decode_items(nq, nkv)
+    work = decode_work(singles, pos.cpu().numpy(), 4, 0, nq, nkv)
+    acc = torch.empty(cap * items * 16 * hd, device=DEV)
+    ml = torch.empty(cap * items * 32, device=DEV)
+    counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
+    out = torch.full_like(q, 7.0)
+    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap), cap, pos, seq_of, table, acc, ml, counters,
+                              True, nq, nkv, hd, page, scale)
+    got = out.double().cpu()
+    assert torch.allclose(got[singles.tolist()], want[singles.tolist()], atol=2e-2, rtol=2e-2)
+    others = [i for i in range(q.shape[0]) if i not in singles.tolist()]
+    assert (got[others] == 7.0).all()
 
 
 @pytest.mark.parametrize("form", [0, 1, 5])
@@ -440,8 +534,7 @@ def test_attention_finds_a_far_key(kernel):
         if kernel.startswith("generic"):
             ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, 0)
         elif kernel == "decode":
-            acc, ml = torch.empty(n * nq * 8 * hd, device=DEV), torch.empty(n * nq * 16, device=DEV)
-            ops.attn_decode_bf16(q, out, kc, vc, i32([0]), 1, pos, seq_of, table, acc, ml, 8, nq, nkv, hd, page, scale, 0)
+            decode_attention(ops, q, out, kc, vc, [0], pos, seq_of, table, nq, nkv, hd, page, scale)
         elif kernel == "prefill32":
             ops.attn_prefill_f32(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, 0)
         else:
@@ -476,8 +569,7 @@ def test_attention_at_a_windows_edge(kernel):
     if kernel.startswith("generic"):
         ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, window)
     elif kernel == "decode":
-        acc, ml = torch.empty(n * nq * 4 * hd, device=DEV), torch.empty(n * nq * 8, device=DEV)
-        ops.attn_decode_bf16(q, out, kc, vc, i32([0]), 1, pos, seq_of, table, acc, ml, 4, nq, nkv, hd, page, scale, window)
+        decode_attention(ops, q, out, kc, vc, [0], pos, seq_of, table, nq, nkv, hd, page, scale, window)
     elif kernel == "prefill32":
         ops.attn_prefill_f32(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, window)
     else:
@@ -493,7 +585,7 @@ def test_attention_at_a_windows_edge(kernel):
         if kernel.startswith("generic"):
             ops.attn_generic(q, out2, kc, vc, pos2, seq_of, table, n, nq, nkv, hd, page, scale, window)
         else:
-            ops.attn_decode_bf16(q, out2, kc, vc, i32([0]), 1, pos2, seq_of, table, acc, ml, 4, nq, nkv, hd, page, scale, window)
+            decode_attention(ops, q, out2, kc, vc, [0], pos2, seq_of, table, nq, nkv, hd, page, scale, window)
         assert not torch.allclose(out2.double().cpu(), want.expand(n, nq, hd), atol=0.2)
 
 

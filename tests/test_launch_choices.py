@@ -4,8 +4,10 @@ than it takes."""
 
 import random
 
-from pyre_amd.parts.fast import (DECODE_MAX_SPLITS, DECODE_MIN_KEYS_PER_SPLIT, SKINNY_MAX_KSPLIT, decode_splits,
-                                 skinny_ksplit)
+import numpy as np
+
+from pyre_amd.parts.fast import (DECODE_MAX_BLOCKS_PER_REQUEST, SKINNY_MAX_KSPLIT, decode_alone, decode_capacity,
+                                 decode_work, skinny_ksplit)
 
 
 def test_split_k_leaves_no_part_empty_and_is_a_function_of_the_sizes():
@@ -29,18 +31,79 @@ def test_split_k_of_the_7b_products():
     assert skinny_ksplit(8, 4608, 3584) == 7
 
 
-def test_decode_splits_stay_within_what_the_kernel_takes():
-    rng = random.Random(1)
-    for _ in range(300):
-        n = rng.randrange(1, 65)
-        nkv = rng.choice([1, 2, 4, 8])
-        nq = nkv * rng.choice([1, 2, 7, 8, 20])
-        ctx = rng.randrange(1, 40000)
-        window = rng.choice([0, 0, 50, 4096])
-        s = decode_splits(n, nq, nkv, ctx, window)
-        assert 1 <= s <= DECODE_MAX_SPLITS
-        span = min(ctx, window + 32) if window > 0 else ctx
-        assert s == 1 or (s - 1) * DECODE_MIN_KEYS_PER_SPLIT < span  # no split without keys of its own
+def _chunks(pos, window):
+    lo = np.maximum(0, pos - window + 1) if window > 0 else np.zeros_like(pos)
+    return pos // 32 - lo // 32 + 1
+
+
+def _check_work(work, tokens, positions, rows, window, nq, nkv):
+    """What the decode kernel relies on: every chunk of every request belongs to exactly one
+    wave of one block, slots are disjoint, and the list fits the launch."""
+    n_blocks = int(work[0, 0])
+    assert work.shape == (1 + n_blocks, 4)
+    assert n_blocks <= decode_capacity(rows, nq, nkv)
+    chunks = dict(zip(tokens.tolist(), _chunks(positions[tokens].astype(np.int64), window).tolist()))
+    seen, slots = {}, set()
+    for tok, b_nb, per, slot0 in work[1:].tolist():
+        b, nb = b_nb % 65536, b_nb // 65536
+        assert 1 <= nb <= DECODE_MAX_BLOCKS_PER_REQUEST and 0 <= b < nb and per >= 1
+        assert 4 * per * nb >= chunks[tok] > 4 * per * (nb - 1)        # all chunks covered, no block without one
+        seen.setdefault(tok, []).append(b)
+        assert slot0 + b not in slots and 0 <= slot0 and slot0 + nb <= n_blocks
+        slots.add(slot0 + b)
+    assert sorted(seen) == sorted(tokens.tolist())
+    assert all(sorted(bs) == list(range(len(bs))) for bs in seen.values())
+    longest_first = [chunks[t] for t in dict.fromkeys(work[1:, 0].tolist())]
+    assert longest_first == sorted(longest_first, reverse=True)
+
+
+def test_decode_work_lists_cover_every_key_once():
+    rng = np.random.default_rng(1)
+    for case in range(300):
+        n = int(rng.integers(1, 300))
+        rows = n + int(rng.integers(0, 20))
+        nkv = int(rng.choice([1, 2, 4, 8]))
+        nq = nkv * int(rng.choice([1, 2, 7, 8, 20]))
+        window = int(rng.choice([0, 0, 50, 4096]))
+        top = int(rng.choice([40, 700, 5000, 70000]))
+        # single tokens somewhere in a flat batch of other tokens, contexts log-uniform
+        flat = n + int(rng.integers(0, 50))
+        tokens = np.sort(rng.choice(flat, n, replace=False)).astype(np.int32)
+        positions = np.zeros(flat, dtype=np.int32)
+        positions[tokens] = np.exp(rng.uniform(0, np.log(top), n)).astype(np.int32) - 1
+        work = decode_work(tokens, positions, rows, window, nq, nkv)
+        _check_work(work, tokens, positions, rows, window, nq, nkv)
+        # the padding of a captured step (requests at position 0) changes nothing for the others
+        pad = rows - n
+        padded_tokens = np.concatenate([tokens, np.arange(flat, flat + pad, dtype=np.int32)])
+        padded_pos = np.concatenate([positions, np.zeros(pad, dtype=np.int32)])
+        padded = decode_work(padded_tokens, padded_pos, rows, window, nq, nkv)
+        _check_work(padded, padded_tokens, padded_pos, rows, window, nq, nkv)
+        real = padded[1:][np.isin(padded[1:, 0], tokens)]
+        assert (real[:, :3] == work[1:, :3]).all()                    # same blocks, same chunks per wave
+    assert (decode_work(np.zeros(0, np.int32), np.zeros(4, np.int32), 8, 0, 4, 2) == 0).all()
+
+
+def test_decode_work_of_known_shapes():
+    # 7B heads (28 query, 4 key/value: 64 blocks per key/value head at once), 4,096 tokens of context
+    pos = lambda n, ctx: np.full(n, ctx, dtype=np.int32)  # noqa: E731
+    tok = lambda n: np.arange(n, dtype=np.int32)          # noqa: E731
+    assert decode_alone(8, 28, 4) and decode_alone(64, 28, 4) and not decode_alone(65, 28, 4)
+    w = decode_work(tok(8), pos(8, 4096), 8, 0, 28, 4)
+    assert w[0, 0] == 56 and (w[1:, 1] // 65536 == 7).all() and (w[1:, 2] == 5).all()   # 7 blocks of 4 x 5 for 129 chunks
+    w = decode_work(tok(64), pos(64, 4096), 64, 0, 28, 4)
+    assert w[0, 0] == 64 and (w[1:, 1] == 65536).all() and (w[1:, 2] == 33).all()       # a block each: nothing crosses blocks
+    w = decode_work(tok(48), pos(48, 4096), 48, 0, 28, 4)
+    assert w[0, 0] <= 64                                               # still one round
+    for n in (96, 256):                                                # two blocks a unit: whole requests again
+        w = decode_work(tok(n), pos(n, 4096), n, 0, 28, 4)
+        assert w[0, 0] == n and (w[1:, 2] == 33).all()
+    # 256 requests of very different lengths on two key/value heads: the long ones are cut
+    rng = np.random.default_rng(0)
+    p = np.exp(rng.uniform(np.log(16), np.log(2560), 256)).astype(np.int32)
+    w = decode_work(tok(256), p, 256, 0, 12, 2)
+    assert w[1, 1] // 65536 >= 4 and w[1, 0] == int(np.argmax(p))
+    assert 4 * w[1:, 2].max() * 32 <= p.sum() // 256 + 256             # a block is about half a slot's share
 
 
 def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():

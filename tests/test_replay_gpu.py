@@ -169,6 +169,41 @@ def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_m
         assert eng.graph_replays >= 4
 
 
+@pytest.mark.parametrize("others,graphs", [(30, True), (30, False), (150, True)])
+def test_decode_steps_of_requests_of_very_different_lengths(others, graphs, model_dirs, plain_models):
+    """One request of 900 tokens and one of 400 among many of 3 to 40: the decode kernel's
+    work list deals the long ones to several blocks, which join their results through memory,
+    and puts them first; with 150 others two blocks share a compute unit. Ten decoded tokens
+    each, captured and replayed (or eager), every row against the plain implementation."""
+    plain = plain_models["tiny-c"]
+    vocab = plain[0]["vocab_size"]
+    prompt = {0: 40, 1: 900, 2: 7, 3: 400}
+    prompt.update({i: 3 + (11 * i) % 38 for i in range(4, others + 2)})
+    reqs = {i: random_ids(vocab, n + 10, 1300 + i) for i, n in prompt.items()}
+    want = _expected(plain, reqs, "bfloat16")
+    n = len(reqs)
+    eng = make_engine(model_dirs["tiny-c"], "bfloat16", use_graphs=graphs, max_num_seqs=n,
+                      max_cached_tokens=1400 + 64 * n, max_num_batched_tokens=1024)
+    ids = sorted(reqs)
+    steps, batch, size = [], [], 0
+    for i in ids:                                                    # whole prompts, packed into steps of up to 1,000 tokens
+        if size + prompt[i] > 1000:
+            steps.append((batch, []))
+            batch, size = [], 0
+        batch.append((i, reqs[i][:prompt[i]], [prompt[i] - 1]))
+        size += prompt[i]
+    steps.append((batch, []))
+    for k in range(10):
+        steps.append(([(i, [reqs[i][prompt[i] + k]], [0]) for i in ids], ids if k == 9 else []))
+    got = replay(eng, steps)
+    assert len(got) == 11 * n
+    bad, worst = first_bad(got, want, TOL["bfloat16"])
+    assert bad is None, bad
+    eng.cache.check_invariants()
+    if graphs:
+        assert eng.graph_replays >= 7
+
+
 @pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
                                                 ("tiny-b", "float32", True)])
 def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, model_dirs, plain_models):
