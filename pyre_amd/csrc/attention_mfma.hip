@@ -272,7 +272,9 @@ __device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge,
 }
 
 // ---------------------------------------------------------------------------
-// Decode: grid (capacity of the work list, nkv * qtiles), 4 waves. The host deals the
+// Decode: grid (nkv * qtiles, capacity of the work list), 4 waves. The blocks of one row of
+// the list (one per key/value head and group of 16 query heads) are neighbours in the order
+// of dispatch, so that the list's order, longest first, is the order in which work starts. The host deals the
 // keys of every request to blocks in proportion to its context, so that a step whose
 // requests differ widely in length keeps all compute units busy for the same time:
 //   work[0]     = (blocks in the list, -, -, -)
@@ -323,16 +325,16 @@ __device__ inline float load_through(const float* base, int elem) {
 template <int HD, bool STREAM_V>
 __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) {
   const int4 head_of_list = work[0];
-  if (static_cast<int>(blockIdx.x) >= head_of_list.x) return;
-  const int4 item = work[1 + blockIdx.x];
+  if (static_cast<int>(blockIdx.y) >= head_of_list.x) return;
+  const int4 item = work[1 + blockIdx.y];
   const int tok = item.x, b = item.y & 0xffff, nb = item.y >> 16, per = item.z, slot0 = item.w;
   // a list that does not fit the launch is not followed
-  if (nb < 1 || nb > kMaxBlocksPerRequest || b < 0 || b >= nb || slot0 < 0 || slot0 + nb > static_cast<int>(gridDim.x) || per < 1)
+  if (nb < 1 || nb > kMaxBlocksPerRequest || b < 0 || b >= nb || slot0 < 0 || slot0 + nb > static_cast<int>(gridDim.y) || per < 1)
     return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
-  const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
+  const int kvh = blockIdx.x / qtiles, qt = blockIdx.x % qtiles;
   const int head0 = kvh * n_rep + qt * 16, nheads = min(16, n_rep - qt * 16);
   const int pos = positions[tok];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
@@ -384,9 +386,9 @@ __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) 
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) *reinterpret_cast<f32x4*>(&acc_s[wave][r][dt * 16 + 4 * g]) = o[dt][0];
   __syncthreads();
-  const int n_items = gridDim.y;
-  float* pa = part_acc + (static_cast<size_t>(slot0 + b) * n_items + blockIdx.y) * 16 * HD;
-  float* pm = part_ml + (static_cast<size_t>(slot0 + b) * n_items + blockIdx.y) * 32;
+  const int n_items = gridDim.x;
+  float* pa = part_acc + (static_cast<size_t>(slot0 + b) * n_items + blockIdx.x) * 16 * HD;
+  float* pm = part_ml + (static_cast<size_t>(slot0 + b) * n_items + blockIdx.x) * 32;
   for (int i = threadIdx.x; i < nheads * (HD / 4); i += 256) {
     const int h = i / (HD / 4), d = 4 * (i % (HD / 4));
     float M = -INFINITY;
@@ -422,15 +424,15 @@ __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) 
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (threadIdx.x == 0) {
-    int* counter = counters + static_cast<size_t>(slot0) * n_items + blockIdx.y;
+    int* counter = counters + static_cast<size_t>(slot0) * n_items + blockIdx.x;
     const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     last_s = before == nb - 1;
     if (last_s) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   if (!last_s) return;
-  const float* pa0 = part_acc + (static_cast<size_t>(slot0) * n_items + blockIdx.y) * 16 * HD;
-  const float* pm0 = part_ml + (static_cast<size_t>(slot0) * n_items + blockIdx.y) * 32;
+  const float* pa0 = part_acc + (static_cast<size_t>(slot0) * n_items + blockIdx.x) * 16 * HD;
+  const float* pm0 = part_ml + (static_cast<size_t>(slot0) * n_items + blockIdx.x) * 32;
   const int acc_step = n_items * 16 * HD, ml_step = n_items * 32;  // floats from one block's slot to the next
   for (int i = threadIdx.x; i < nb * 32; i += 256) {
     const int bb = i >> 5, j = i & 31;
@@ -577,12 +579,23 @@ __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_b
 // LOADER: the block's last wave has no head of its own (the group has fewer heads than
 // the block has waves) and does all the loading; the others only compute, and keep the
 // registers and the instructions of the loads for themselves.
+//
+// work[2 i], work[2 i + 1] = (first token of the tile in the flat batch, tokens <= 32, first
+// chunk of 64 keys, last chunk), (first partial slot of the tile, this block's number b among
+// the tile's blocks, their number nb, -): the host deals the chunks of a tile to nb blocks
+// when there are fewer tiles than compute units (a portion of a prompt late in a long
+// context) or when the tiles differ much in length (the triangle of a whole prompt). A tile
+// with one block is finished by it. Otherwise every wave stores its head's partial result
+// (max, sum, unnormalised output) at slot (first slot + b) with stores that go through to
+// memory and counts itself in at the counter of (tile, head); the wave that arrives last
+// reads the nb partial results with loads that come from memory and joins them in the order
+// 0..nb-1, whichever wave it is, and leaves the counter at zero.
 template <int HD, int NW, bool LOADER>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-    bf16* __restrict__ out, const int* __restrict__ tiles, const int* __restrict__ positions,
-    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
-    int nq, int nkv, int page_size, float scale_log2, int window) {
+    bf16* __restrict__ out, const int4* __restrict__ work, float* __restrict__ partials, int* __restrict__ counters,
+    int n_slots, const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+    int table_stride, int nq, int nkv, int page_size, float scale_log2, int window) {
   constexpr int KS = HD + 8, VS = kKeys + 8;
   constexpr int SEG = HD / 8;            // 16-byte pieces of one K row
   // A run of 16 keys is HD / 32 blocks of 64 pieces (1 KB) of K, contiguous in its page,
@@ -598,11 +611,12 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r = lane & 31,
             g = lane >> 5;
   const int n_rep = nq / nkv, hgroups = (n_rep + NW - 1) / NW;
-  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int kvh = blockIdx.x / hgroups, hg = blockIdx.x % hgroups;
   const int hin = hg * NW + wave;
   const bool active = hin < n_rep;  // a wave without a head still helps loading
   const int head = kvh * n_rep + (active ? hin : 0);
-  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+  const int4 item = work[2 * blockIdx.y], share = work[2 * blockIdx.y + 1];
+  const int t0 = item.x, ntok = item.y;
   const int pos0 = positions[t0];
   const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
 
@@ -623,7 +637,8 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
 
   const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int hi_all = pos0 + ntok - 1;
-  const int first = lo_all / kKeys, last = hi_all / kKeys;
+  // this block's chunks, kept within the tile's whatever the list says
+  const int first = min(max(item.z, lo_all / kKeys), hi_all / kKeys), last = min(max(item.w, first), hi_all / kKeys);
   const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
 
   const int n = last - first + 1;
@@ -908,6 +923,59 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
 
   if (!active) return;
   l += __shfl_xor(l, 32, 64);
+  const int slot0 = share.x, b = share.y, nb = share.z;
+  if (nb > 1) {
+    if (slot0 < 0 || b < 0 || b >= nb || slot0 + nb > n_slots) return;  // a list that does not fit the scratch is not followed
+    // floats of one wave's partial result: element (dt, 4 q .. 4 q + 3) of lane x at 4 ((4 dt + q) 64 + x), then (m, l)
+    constexpr int kPart = (HD / 32) * 16 * 64 + 2 * 64;
+    const size_t per_slot = static_cast<size_t>(gridDim.x) * NW * kPart;
+    float* mine = partials + (static_cast<size_t>(slot0 + b) * gridDim.x + blockIdx.x) * NW * kPart + wave * kPart;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd)
+        store_through(mine, 4 * ((4 * dt + qd) * 64 + lane),
+                      f32x4{o[dt][4 * qd], o[dt][4 * qd + 1], o[dt][4 * qd + 2], o[dt][4 * qd + 3]});
+    store_through(mine, (HD / 32) * 16 * 64 + 2 * lane, m);
+    store_through(mine, (HD / 32) * 16 * 64 + 2 * lane + 1, l);
+    __builtin_amdgcn_s_waitcnt(0);  // the stores have arrived
+    int is_last = 0;
+    if (lane == 0) {
+      int* counter = counters + (static_cast<size_t>(slot0) * gridDim.x + blockIdx.x) * NW + wave;
+      const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = before == nb - 1;
+      if (is_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!__builtin_amdgcn_readfirstlane(is_last)) return;
+    const float* theirs = partials + (static_cast<size_t>(slot0) * gridDim.x + blockIdx.x) * NW * kPart + wave * kPart;
+    m = -INFINITY;
+    l = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+    for (int p = 0; p < nb; ++p, theirs += per_slot) {
+      f32x4 v[HD / 32][4];
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) v[dt][qd] = load_through4(theirs, 4 * ((4 * dt + qd) * 64 + lane));
+      const float mp = load_through(theirs, (HD / 32) * 16 * 64 + 2 * lane);
+      const float lp = load_through(theirs, (HD / 32) * 16 * 64 + 2 * lane + 1);
+      const float m_new = fmaxf(m, mp);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float wa = __builtin_amdgcn_exp2f((m - m_use) * scale_log2);   // 0 for m = -inf
+      const float wp = __builtin_amdgcn_exp2f((mp - m_use) * scale_log2);
+      m = m_new;
+      l = l * wa + lp * wp;
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[dt][4 * qd + e] = o[dt][4 * qd + e] * wa + v[dt][qd][e] * wp;
+    }
+  }
   if (r >= ntok) return;
   const float inv = 1.f / l;
   bf16* dst = out + (static_cast<size_t>(t0 + r) * nq + head) * HD + 4 * g;
@@ -956,8 +1024,8 @@ extern "C" int pyre_attn_decode_work_bf16(const void* q, void* out, const void* 
   PYRE_REQUIRE(reinterpret_cast<uintptr_t>(work) % 16 == 0, "attn_decode_work_bf16: the work list must lie on 16 bytes");
   if (capacity == 0) return 0;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
-  PYRE_REQUIRE(nkv * qtiles <= 65535, "attn_decode_work_bf16: grid too large");
-  const dim3 grid(capacity, nkv * qtiles);
+  PYRE_REQUIRE(capacity <= 65535, "attn_decode_work_bf16: a list of %d blocks is too long for one launch", capacity);
+  const dim3 grid(nkv * qtiles, capacity);
   const float scale_log2 = scale * kLog2e;
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
@@ -981,52 +1049,69 @@ extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_ca
                                       const void* v_cache, const int* tiles, int n_tiles,
                                       const int* positions, const int* seq_of_token,
                                       const int* block_table, int table_stride, int nq, int nkv,
-                                      int hd, int page_size, float scale, int window, int form,
-                                      hipStream_t stream) {
+                                      int hd, int page_size, float scale, int window, hipStream_t stream) {
   PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
                "attn_prefill_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
   PYRE_REQUIRE(table_stride > 0, "attn_prefill_bf16: bad table");
   if (n_tiles <= 0) return 0;
-  const int n_rep = nq / nkv;
-  const float scale_log2 = scale * kLog2e;
-  const bf16* qp = static_cast<const bf16*>(q);
-  const bf16* kp = static_cast<const bf16*>(k_cache);
-  const bf16* vp = static_cast<const bf16*>(v_cache);
-  bf16* op = static_cast<bf16*>(out);
-  // Up to 128 elements per head, K and V go through LDS in chunks of 64 keys for 32x32 MFMA
-  // tiles (form 1; form 5: the same, never with a loading wave); larger heads, and form 0,
-  // read the cache directly in every wave.
-  const bool tile32 = hd <= 128 && form != 0;
-  const int nw = tile32 && n_rep > 4 ? 8 : 4;
-  const int hgroups = (n_rep + nw - 1) / nw;
+  const int hgroups = (nq / nkv + 3) / 4;
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_prefill_bf16: grid too large");
   const dim3 grid(n_tiles, nkv * hgroups);
-#define PYRE_PREFILL_ARGS \
-  qp, kp, vp, op, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale_log2, window
+  const int rc = dispatch_head(hd, [&](auto HDc) {
+    constexpr int HD = decltype(HDc)::value;
+    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
+                       static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), static_cast<bf16*>(out),
+                       tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, page_size, scale * kLog2e,
+                       window);
+  });
+  PYRE_REQUIRE(rc == 0, "attn_prefill_bf16: no kernel for head_dim %d", hd);
+  return check_launch("attn_prefill_bf16");
+}
+
+extern "C" int pyre_attn_prefill_waves(int nq, int nkv) { return nq / nkv > 4 ? 8 : 4; }
+
+extern "C" int pyre_attn_prefill_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                                           const int* work, int n_items, float* partials, int* counters,
+                                           int n_slots, const int* positions, const int* seq_of_token, const int* block_table,
+                                           int table_stride, int nq, int nkv, int hd, int page_size, float scale,
+                                           int window, int loader, hipStream_t stream) {
+  PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv) && hd <= 128,
+               "attn_prefill_work_bf16: head_dim %d (multiples of 32 up to 128), page_size %d (multiples of 16), "
+               "heads %d/%d are not supported", hd, page_size, nq, nkv);
+  PYRE_REQUIRE(table_stride > 0 && n_slots >= 0, "attn_prefill_work_bf16: bad table or slots");
+  PYRE_REQUIRE(reinterpret_cast<uintptr_t>(work) % 16 == 0, "attn_prefill_work_bf16: the work list must lie on 16 bytes");
+  if (n_items <= 0) return 0;
+  const int n_rep = nq / nkv;
+  const int nw = pyre_attn_prefill_waves(nq, nkv);
+  const int hgroups = (n_rep + nw - 1) / nw;
+  PYRE_REQUIRE(n_items <= 65535, "attn_prefill_work_bf16: a list of %d blocks is too long for one launch", n_items);
+  // the blocks of one row of the list are neighbours in the order of dispatch: the list's order is the order of starts
+  const dim3 grid(nkv * hgroups, n_items);
+  // a wave to spare in every block (one group of fewer heads than waves): it loads for the others
+  const bool use_loader = n_rep < nw && loader != 0;
+#define PYRE_PREFILL_ARGS                                                                                          \
+  static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache),               \
+      static_cast<bf16*>(out), reinterpret_cast<const int4*>(work), partials, counters, n_slots, positions,        \
+      seq_of_token,                                                                                                \
+      block_table, table_stride, nq, nkv, page_size, scale * kLog2e, window
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
     if constexpr (HD <= 128) {
-      // a wave to spare in every block (one group of fewer heads than waves): it loads for the others
-      const bool loader = n_rep < nw && form != 5;
-      if (tile32 && nw == 8) {
-        if (loader)
+      if (nw == 8) {
+        if (use_loader)
           hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8, true>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
         else
           hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8, false>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
-        return;
-      }
-      if (tile32) {
-        if (loader)
+      } else {
+        if (use_loader)
           hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, true>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
         else
           hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, false>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
-        return;
       }
     }
-    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
   });
 #undef PYRE_PREFILL_ARGS
-  PYRE_REQUIRE(rc == 0, "attn_prefill_bf16: no kernel for head_dim %d", hd);
-  return check_launch("attn_prefill_bf16");
+  PYRE_REQUIRE(rc == 0, "attn_prefill_work_bf16: no kernel for head_dim %d", hd);
+  return check_launch("attn_prefill_work_bf16");
 }

@@ -103,15 +103,30 @@ int pyre_attn_decode_work_bf16(const void* q, void* out, const void* k_cache, co
                                int hd, int page_size, float scale, int window, hipStream_t stream);
 
 // Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
-// all tokens of a tile from one request at consecutive positions. Heads of up to 128
-// elements: form 1 stages K and V through LDS in chunks of 64 keys for 32x32 MFMA tiles
-// (form 5: the same, never with a wave that only loads); form 0, and every larger head,
-// reads the cache directly in each wave.
+// all tokens of a tile from one request at consecutive positions. Every wave reads the
+// cache directly (any head size that pyre_attn_mfma_supports takes).
 int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
                            const int* tiles, int n_tiles, const int* positions,
                            const int* seq_of_token, const int* block_table, int table_stride,
-                           int nq, int nkv, int hd, int page_size, float scale, int window, int form,
+                           int nq, int nkv, int hd, int page_size, float scale, int window,
                            hipStream_t stream);
+
+// The same for heads of up to 128 elements from a work list: K and V go through LDS in chunks
+// of 64 keys for 32x32 MFMA tiles, and the chunks of a tile may be dealt to several blocks.
+// work[2 i] = (first token of the tile, tokens <= 32, first chunk, last chunk), work[2 i + 1] =
+// (first partial slot of the tile, this block's number among the tile's blocks, their number
+// nb, 0); the nb blocks of a tile cover the chunks lo / 64 .. hi / 64 of the keys lo .. hi that
+// its tokens see, each chunk once. A block has pyre_attn_prefill_waves(nq, nkv) waves, one per
+// query head of a key/value head (groups of that many heads: `groups`). Scratch for tiles
+// of more than one block: partials [slots, nkv * groups, waves, hd / 32 * 1024 + 128] floats
+// and counters [slots, nkv * groups, waves] ints that are zero before the first call and are
+// left at zero. `loader`: a block with a wave to spare lets it do all the loading.
+int pyre_attn_prefill_waves(int nq, int nkv);
+int pyre_attn_prefill_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                                const int* work, int n_items, float* partials, int* counters,
+                                int n_slots, const int* positions, const int* seq_of_token, const int* block_table,
+                                int table_stride, int nq, int nkv, int hd, int page_size, float scale,
+                                int window, int loader, hipStream_t stream);
 
 // scratch: m * 64 floats followed by m * 64 ints of device memory.
 int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,

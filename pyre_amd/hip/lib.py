@@ -34,7 +34,9 @@ _SIGNATURES = {
     "pyre_attn_prefill_f32": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_mfma_supports": [I, I, I, I],
     "pyre_attn_decode_work_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
-    "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+    "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
+    "pyre_attn_prefill_waves": [I, I],
+    "pyre_attn_prefill_work_bf16": [P, P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
     "pyre_argmax_static": [P, L, P, I, I, P],
     "pyre_gemm_skinny_supports": [I, I, I, L, L],

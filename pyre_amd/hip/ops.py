@@ -421,13 +421,40 @@ def attn_decode_work_bf16(q, out, k_cache, v_cache, work, capacity, positions, s
 
 
 def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,
-                      nq, nkv, hd, page_size, scale, window=0, form=1) -> None:
-    """Attention of prompt portions; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32)."""
+                      nq, nkv, hd, page_size, scale, window=0) -> None:
+    """Attention of prompt portions, every wave reading the cache directly; ``tiles`` is int32
+    [n_tiles, 2] = (first token, count <= 32)."""
     _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
     _i32("tiles", tiles, 2 * n_tiles)
     call("pyre_attn_prefill_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
          tiles.data_ptr(), n_tiles, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
-         block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), int(form), _stream())
+         block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), _stream())
+
+
+def attn_prefill_waves(nq: int, nkv: int) -> int:
+    from pyre_amd.hip.lib import lib
+
+    return int(lib().pyre_attn_prefill_waves(nq, nkv))
+
+
+def attn_prefill_work_bf16(q, out, k_cache, v_cache, work, n_items, partials, counters, n_slots, positions,
+                           seq_of_token, block_table, nq, nkv, hd, page_size, scale, window=0, loader=True) -> None:
+    """Attention of prompt portions for heads of up to 128 elements from a work list (int32
+    ``[n_items, 8]``: see ``pyre_attn_prefill_work_bf16`` in pyre_api.h) whose tiles of several
+    blocks use the partial slots 0..n_slots-1. ``counters`` must be zero and is left at zero."""
+    _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
+    _i32("work", work, 8 * n_items)
+    waves = attn_prefill_waves(nq, nkv)
+    per_slot = nkv * -(-(nq // nkv) // waves) * waves
+    if n_slots:
+        if partials.dtype != torch.float32 or partials.numel() < n_slots * per_slot * (hd // 32 * 1024 + 128):
+            raise KernelError("attn_prefill_work: partial results do not fit")
+        if counters.dtype != torch.int32 or counters.numel() < n_slots * per_slot:
+            raise KernelError("attn_prefill_work: too few counters")
+    call("pyre_attn_prefill_work_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         work.data_ptr(), n_items, _ptr(partials) if n_slots else None, _ptr(counters) if n_slots else None,
+         n_slots, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+         nq, nkv, hd, page_size, float(scale), int(window), int(bool(loader)), _stream())
 
 
 def gemm_skinny_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:

@@ -69,22 +69,31 @@ class Attention(Mixer):
         self.qkv = Linear(spec.hidden_size, self.q_dim + 2 * self.kv_dim, "attn.qkv")
         self.out = Linear(self.q_dim, spec.hidden_size, "attn.out")
         self.decode_work_name = f"attention.decode_work.{spec.num_heads}.{spec.num_kv_heads}.{spec.window}"
+        self.prefill_work_name = f"attention.prefill_work.{spec.num_heads}.{spec.num_kv_heads}.{spec.window}"
 
     def cache_spec(self):
         s = self.spec
         return KVCacheSpec(s.num_kv_heads, s.head_dim, s.window)
 
     def step_arrays(self):
-        """The lists of single tokens and of tiles, and the decode kernel's work list, which
-        depends on the head counts and the window and is shared by all layers that agree in them."""
+        """The lists of single tokens and of tiles, and the work lists of the decode and the
+        prompt-portion kernel, which depend on the head counts and the window and are shared by
+        all layers that agree in them."""
         s = self.spec
 
         def work(hb):
             return fast.decode_work(hb.arrays["attention.decode_tokens"], hb.positions, hb.decode_shape()[0],
                                     s.window, s.num_heads, s.num_kv_heads)
 
-        return [*STEP_ARRAYS, StepArraySpec(
-            self.decode_work_name, lambda n_cap, s_cap: 4 * (1 + fast.decode_capacity(s_cap, s.num_heads, s.num_kv_heads)), work)]
+        def portions(hb):
+            return fast.prefill_work(hb.arrays["attention.prefill_tiles"], hb.positions, s.window,
+                                     fast.prefill_items(s.num_heads, s.num_kv_heads))
+
+        return [*STEP_ARRAYS,
+                StepArraySpec(self.decode_work_name,
+                              lambda n_cap, s_cap: 4 * (1 + fast.decode_capacity(s_cap, s.num_heads, s.num_kv_heads)), work),
+                StepArraySpec(self.prefill_work_name,
+                              lambda n_cap, s_cap: 8 * (n_cap // TILE + s_cap + 2 * fast.DECODE_UNITS + 1), portions)]
 
     def linears(self) -> list:
         return [self.qkv, self.out]

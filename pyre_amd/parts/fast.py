@@ -10,6 +10,8 @@ never comes here.
 
 from __future__ import annotations
 
+import math
+
 import numpy as np
 import torch
 
@@ -201,6 +203,105 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
     return work
 
 
+#: keys per chunk of the prompt-portion kernel; a block of it fills a compute unit (its LDS)
+PREFILL_CHUNK = 64
+#: What a further block costs its tile, in chunks' worth of time: each block of a tile that has
+#: several stores a partial result of 16 KB per head (4), and the wave that comes last reads
+#: them all back (0.25 per block). Fitted to the kernel's times on the 7B heads: whole prompts
+#: of 1,024 to 4,096 tokens and portions of 128 and 512 tokens after 4,096 to 32,768, each with
+#: blocks of 6 to 512 chunks; the fit picks the fastest of the measured sizes in every case.
+PREFILL_BLOCK_COST = 4.0
+PREFILL_JOIN_COST = 0.25
+#: block sizes that are tried, as parts of the longest tile
+PREFILL_SIZES = (1, 3 / 4, 1 / 2, 3 / 8, 1 / 4, 3 / 16, 1 / 8, 3 / 32, 1 / 16, 3 / 64, 1 / 32, 1 / 64)
+
+
+def prefill_items(nq: int, nkv: int) -> int:
+    """Blocks per tile of the prompt-portion kernel: key/value heads times groups of as many
+    query heads as a block has waves."""
+    from pyre_amd.hip import ops
+
+    return nkv * -(-(nq // nkv) // ops.attn_prefill_waves(nq, nkv))
+
+
+def _deal(chunks: np.ndarray, size: int):
+    """Blocks per tile and chunks per block when no block takes more than ``size`` chunks."""
+    nb = -(-chunks // size)
+    per = -(-chunks // nb)
+    return -(-chunks // per), per
+
+
+def _time_of(chunks: np.ndarray, size: int, slots: int) -> float:
+    """How long the blocks of this deal take, in chunks' worth of time, when the dispatcher
+    hands them, longest tile first, to whichever of ``slots`` units is free next."""
+    nb, per = _deal(chunks, size)
+    cost = np.where(nb > 1, per + PREFILL_BLOCK_COST + PREFILL_JOIN_COST * nb, per).astype(np.float64)
+    jobs = np.repeat(cost, nb)  # tiles come longest first, their blocks together
+    loads = np.zeros(slots)
+    for i in range(0, len(jobs), slots):
+        batch = jobs[i:i + slots]
+        loads.sort()
+        loads[:len(batch)] += batch
+    return float(loads.max())
+
+
+def prefill_work(tiles: np.ndarray, positions: np.ndarray, window: int, items: int, size: int | None = None) -> np.ndarray:
+    """The prompt-portion kernel's work list (int32 ``[blocks, 8]``) for ``tiles`` ([T, 2]:
+    first token, count) at ``positions``; ``items`` blocks run per tile and chunk range.
+
+    A tile of c chunks of 64 keys gets ceil(c / size) blocks and deals its chunks evenly to
+    them; a block fills a compute unit. ``size`` is the one of a few candidates (parts of the
+    longest tile) with which the step is over soonest by a replay of the
+    dispatcher on the blocks' estimated times. So the few tiles of a portion late in a long
+    context spread over the whole chip, and the long tiles at the end of a whole prompt do not
+    run alone, while many tiles are left whole. The longest tiles come first.
+    Row i is (first token, tokens, first chunk, last chunk, first partial slot of the tile,
+    this block's number among the tile's, their number, 0); tiles of one block use no slot.
+    ``size`` fixes the block size instead (for tests of the kernel)."""
+    if len(tiles) == 0:
+        return np.zeros((0, 8), dtype=np.int32)
+    t0, ntok = tiles[:, 0].astype(np.int64), tiles[:, 1].astype(np.int64)
+    pos0 = positions[t0].astype(np.int64)
+    lo = np.maximum(0, pos0 - window + 1) if window > 0 else np.zeros_like(pos0)
+    first, last = lo // PREFILL_CHUNK, (pos0 + ntok - 1) // PREFILL_CHUNK
+    chunks = last - first + 1
+    order = np.argsort(-chunks, kind="stable")
+    n, longest = len(tiles), int(chunks.max())
+    slots = max(1, DECODE_UNITS // items)
+    if size is None:
+        size = longest
+        if n < 4 * slots:  # with many tiles the units stay busy to the end anyway
+            sorted_chunks = chunks[order]
+            best = _time_of(sorted_chunks, size, slots)
+            for part in PREFILL_SIZES[1:]:
+                cand = math.ceil(longest * part)
+                if cand < 2 or int(_deal(sorted_chunks, cand)[0].sum()) > n + 2 * slots:
+                    break  # the list holds the tiles and two rounds of blocks more at most
+                t = _time_of(sorted_chunks, cand, slots)
+                if t < 0.97 * best:
+                    size, best = cand, t
+    nb, per = _deal(chunks, size)
+    nb_sorted = nb[order]
+    which = np.repeat(np.arange(n), nb_sorted)
+    n_blocks = int(nb_sorted.sum())
+    b = np.arange(n_blocks) - (np.cumsum(nb_sorted) - nb_sorted)[which]
+    shared = np.where(nb_sorted > 1, nb_sorted, 0)
+    slot0 = np.where(shared > 0, np.cumsum(shared) - shared, 0)[which]
+    src = order[which]
+    work = np.zeros((n_blocks, 8), dtype=np.int32)
+    work[:, 0], work[:, 1] = t0[src], ntok[src]
+    work[:, 2] = first[src] + b * per[src]
+    work[:, 3] = np.minimum(last[src], work[:, 2] + per[src] - 1)
+    work[:, 4], work[:, 5], work[:, 6] = slot0, b, nb_sorted[which]
+    return work
+
+
+def prefill_slots(work: np.ndarray) -> int:
+    """Partial slots that a work list of :func:`prefill_work` uses."""
+    shared = work[:, 6] > 1
+    return int((work[shared, 4] + work[shared, 6]).max()) if shared.any() else 0
+
+
 def attention(mixer, ctx, q, o, cache) -> bool:
     from pyre_amd.hip import ops
 
@@ -229,7 +330,19 @@ def attention(mixer, ctx, q, o, cache) -> bool:
                                   ctx.seq_of_token, cache.table, acc, ml, counters,
                                   decode_alone(rows, s.num_heads, s.num_kv_heads), s.num_heads, s.num_kv_heads,
                                   s.head_dim, cache.page_size, mixer.scale, cache.window)
-    if n_tiles:
+    if n_tiles and s.head_dim <= 128:
+        work = hb.arrays[mixer.prefill_work_name]
+        n_slots = prefill_slots(work)
+        per_slot = prefill_items(s.num_heads, s.num_kv_heads) * ops.attn_prefill_waves(s.num_heads, s.num_kv_heads)
+        partials = counters = None
+        if n_slots:
+            partials = ctx.workspace.get("attn.prefill_partials", (n_slots, per_slot, s.head_dim // 32 * 1024 + 128),
+                                         torch.float32)
+            counters = ctx.workspace.get("attn.prefill_counters", (n_slots, per_slot), torch.int32, zeroed=True)
+        ops.attn_prefill_work_bf16(q, o, k_pages, v_pages, ctx.arrays[mixer.prefill_work_name], len(work), partials,
+                                   counters, n_slots, ctx.positions, ctx.seq_of_token, cache.table, s.num_heads,
+                                   s.num_kv_heads, s.head_dim, cache.page_size, mixer.scale, cache.window)
+    elif n_tiles:
         ops.attn_prefill_bf16(q, o, k_pages, v_pages, ctx.arrays["attention.prefill_tiles"], n_tiles, ctx.positions,
                               ctx.seq_of_token, cache.table, s.num_heads, s.num_kv_heads, s.head_dim,
                               cache.page_size, mixer.scale, cache.window)

@@ -451,24 +451,76 @@ def test_attn_decode_work_list_in_a_mixed_batch():
     assert (got[others] == 7.0).all()
 
 
-@pytest.mark.parametrize("form", [0, 1, 5])
+def prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window=0, size=None,
+                      loader=True):
+    """Prompt portions through the kernel for the head size: from a work list planned as the
+    engine plans it (or with blocks of ``size`` chunks of 64 keys) for heads of up to 128
+    elements, from the tiles themselves for larger ones. Returns the work list, if any."""
+    from pyre_amd.parts.fast import prefill_items, prefill_slots, prefill_work
+
+    tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+    if hd > 128:
+        ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles.reshape(-1).tolist()), len(tiles), pos, seq_of, table,
+                              nq, nkv, hd, page, scale, window)
+        return None
+    items = prefill_items(nq, nkv)
+    work = prefill_work(tiles, pos.cpu().numpy(), window, items, size=size)
+    n_slots = prefill_slots(work)
+    per_slot = items * ops.attn_prefill_waves(nq, nkv)
+    partials = torch.full((max(1, n_slots) * per_slot * (hd // 32 * 1024 + 128),), float("nan"), device=DEV)
+    counters = torch.zeros(max(1, n_slots) * per_slot, dtype=torch.int32, device=DEV)
+    ops.attn_prefill_work_bf16(q, out, kc, vc, i32(work.reshape(-1).tolist()), len(work), partials, counters, n_slots,
+                               pos, seq_of, table, nq, nkv, hd, page, scale, window, loader)
+    assert int(counters.abs().sum()) == 0
+    return work
+
+
+@pytest.mark.parametrize("size,loader", [(None, True), (None, False), (3, True), (1, False)])
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
-@pytest.mark.parametrize("window", [0, 50])
-def test_attn_prefill_mfma(nq, nkv, hd, page, window, form):
+@pytest.mark.parametrize("window", [0, 50, 300])
+def test_attn_prefill_mfma(nq, nkv, hd, page, window, size, loader):
+    """Prompt portions of several requests. Blocks of one or three chunks of 64 keys deal the
+    tiles of the longer requests to many blocks, whose partial results join through memory."""
     ops = _ops()
     from pyre_amd.parts.attention import TILE
 
+    if hd > 128 and (size is not None or not loader):
+        pytest.skip("larger heads have one form")
     ctx_lens, q_lens = [2, 40, 97, 700, 1100], [2, 40, 33, 3, 600]
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=4)
-    out = torch.full_like(q, float("nan"))
     tiles, base = [], 0
     for ql in q_lens:
         tiles += [(t0, min(TILE, base + ql - t0)) for t0 in range(base, base + ql, TILE)]
         base += ql
     scale = hd ** -0.5
-    ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), len(tiles), pos, seq_of, table, nq, nkv, hd, page, scale, window, form)
     want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    outs = []
+    for _ in range(2):                                              # the second call finds the counters as the first left them
+        out = torch.full_like(q, float("nan"))
+        work = prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window, size, loader)
+        assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    if size is not None and window == 0:
+        assert work[:, 6].max() >= 6                                # the long request's tiles span many blocks
+
+
+def test_attn_prefill_of_a_portion_late_in_a_long_context():
+    """64 tokens at the end of 6,000: two tiles, which the planner deals to as many blocks as
+    the chip has units; the result is that of undivided tiles up to rounding."""
+    ops = _ops()
+    nq, nkv, hd, page = 28, 4, 128, 16
+    ctx_lens, q_lens = [6000], [64]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=21)
+    scale = hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale)
+    out = torch.full_like(q, float("nan"))
+    work = prefill_attention(ops, q, out, kc, vc, [(0, 32), (32, 32)], pos, seq_of, table, nq, nkv, hd, page, scale)
+    assert len(work) >= 8 and work[:, 6].min() > 1
     assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
+    whole = torch.full_like(q, float("nan"))
+    prefill_attention(ops, q, whole, kc, vc, [(0, 32), (32, 32)], pos, seq_of, table, nq, nkv, hd, page, scale, size=10 ** 6)
+    assert torch.allclose(out.float(), whole.float(), atol=1e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("nq,nkv,hd,page", GENERIC_SHAPES + [(3, 1, 10, 8), (7, 1, 72, 16), (12, 2, 128, 48)])
@@ -538,8 +590,7 @@ def test_attention_finds_a_far_key(kernel):
         elif kernel == "prefill32":
             ops.attn_prefill_f32(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, 0)
         else:
-            tiles = [(0, 32), (32, 2)]
-            ops.attn_prefill_bf16(q, out, kc, vc, i32(tiles).view(-1), 2, pos, seq_of, table, nq, nkv, hd, page, scale, 0)
+            prefill_attention(ops, q, out, kc, vc, [(0, 32), (32, 2)], pos, seq_of, table, nq, nkv, hd, page, scale)
         want = V[target].double().repeat_interleave(nq // nkv, 0)      # nq, hd
         assert torch.allclose(out.double().cpu(), want.expand(n, nq, hd), atol=3e-2), (kernel, target)
 
@@ -573,7 +624,7 @@ def test_attention_at_a_windows_edge(kernel):
     elif kernel == "prefill32":
         ops.attn_prefill_f32(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, window)
     else:
-        ops.attn_prefill_bf16(q, out, kc, vc, i32([0, 32, 32, 2]), 2, pos, seq_of, table, nq, nkv, hd, page, scale, window)
+        prefill_attention(ops, q, out, kc, vc, [(0, 32), (32, 2)], pos, seq_of, table, nq, nkv, hd, page, scale, window)
     want = V[edge].double().repeat_interleave(nq // nkv, 0)
     assert torch.allclose(out.double().cpu(), want.expand(n, nq, hd), atol=3e-2), kernel
     # one position on, the edge key itself has left the last query's window: the output is a mixture again

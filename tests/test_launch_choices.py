@@ -6,8 +6,8 @@ import random
 
 import numpy as np
 
-from pyre_amd.parts.fast import (DECODE_MAX_BLOCKS_PER_REQUEST, SKINNY_MAX_KSPLIT, decode_alone, decode_capacity,
-                                 decode_work, skinny_ksplit)
+from pyre_amd.parts.fast import (DECODE_MAX_BLOCKS_PER_REQUEST, DECODE_UNITS, SKINNY_MAX_KSPLIT, decode_alone,
+                                 decode_capacity, decode_work, prefill_slots, prefill_work, skinny_ksplit)
 
 
 def test_split_k_leaves_no_part_empty_and_is_a_function_of_the_sizes():
@@ -104,6 +104,51 @@ def test_decode_work_of_known_shapes():
     w = decode_work(tok(256), p, 256, 0, 12, 2)
     assert w[1, 1] // 65536 >= 4 and w[1, 0] == int(np.argmax(p))
     assert 4 * w[1:, 2].max() * 32 <= p.sum() // 256 + 256             # a block is about half a slot's share
+
+
+def test_prefill_work_lists_cover_every_chunk_once():
+    rng = np.random.default_rng(2)
+    for case in range(200):
+        items = int(rng.choice([1, 2, 4, 8, 16]))
+        window = int(rng.choice([0, 0, 100, 3000]))
+        # a few requests with portions of any length at any depth of their context
+        tiles, positions = [], []
+        for _ in range(int(rng.integers(1, 6))):
+            start = int(rng.choice([0, 0, 37, 5000, 30000]))
+            n = int(rng.integers(2, int(rng.choice([40, 700, 3000]))))
+            base = len(positions)
+            positions += list(range(start, start + n))
+            tiles += [(t0, min(32, base + n - t0)) for t0 in range(base, base + n, 32)]
+        tiles, positions = np.asarray(tiles, dtype=np.int32), np.asarray(positions, dtype=np.int32)
+        work = prefill_work(tiles, positions, window, items)
+        assert len(work) <= len(tiles) + 2 * DECODE_UNITS
+        seen, slots = {}, set()
+        for t0, ntok, c0, c1, slot0, b, nb, _ in work.tolist():
+            assert c0 <= c1 and 0 <= b < nb
+            seen.setdefault((t0, ntok), []).append((b, nb, c0, c1))
+            if nb > 1:
+                assert slot0 + b not in slots and slot0 + nb <= prefill_slots(work)
+                slots.add(slot0 + b)
+        assert sorted(seen) == sorted(map(tuple, tiles.tolist()))
+        for (t0, ntok), blocks in seen.items():
+            pos0 = int(positions[t0])
+            lo = max(0, pos0 - window + 1) if window else 0
+            blocks.sort()
+            assert [b for b, *_ in blocks] == list(range(blocks[0][1]))
+            assert blocks[0][2] == lo // 64 and blocks[-1][3] == (pos0 + ntok - 1) // 64
+            assert all(x[3] + 1 == y[2] for x, y in zip(blocks, blocks[1:]))     # neither a gap nor an overlap
+        assert len(slots) == prefill_slots(work)
+    # 512 tokens at the end of 32,768 on 4 key/value heads: 16 tiles, each dealt to 4 blocks (64 blocks a head)
+    positions = np.arange(32768 - 512, 32768, dtype=np.int32)
+    tiles = np.asarray([(t0, 32) for t0 in range(0, 512, 32)], dtype=np.int32)
+    work = prefill_work(tiles, positions, 0, 4)
+    assert len(work) == 64 and (work[:, 6] == 4).all()
+    # a whole prompt of 8,192 tokens: 256 tiles are plenty, none is cut
+    positions = np.arange(8192, dtype=np.int32)
+    tiles = np.asarray([(t0, 32) for t0 in range(0, 8192, 32)], dtype=np.int32)
+    work = prefill_work(tiles, positions, 0, 4)
+    assert len(work) == 256 and work[0, 0] in (8128, 8160)               # a longest tile first
+    assert prefill_work(np.zeros((0, 2), np.int32), positions, 0, 4).shape == (0, 8)
 
 
 def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():
