@@ -189,6 +189,9 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiling): no decode steps")
+    ap.add_argument("--portion", type=int, default=0, metavar="TOKENS",
+                    help="with --prefill-only: also time the last portion of this many tokens of a prompt of "
+                         "--context tokens that is fed in such portions (chunked prefill late in a long context)")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-tune", action="store_true", help="keep the BLAS library's default kernels for prefill")
     ap.add_argument("--opt", action="append", default=[], metavar="KEY=VALUE",
@@ -293,8 +296,30 @@ def main() -> int:
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
 
     if args.prefill_only:
+        portion = None
+        if args.portion:
+            from pyre_amd.engine.batch import Entry
+
+            ids = prompt(args.context)
+            times = []
+            for trial in range(3):  # the prompt in portions; the last three portions are timed, the median counts
+                cuts = list(range(0, args.context, args.portion))
+                for a in cuts:
+                    last = a + args.portion >= args.context
+                    timed = trial == 2 and a in cuts[-3:]
+                    if timed:
+                        sync()
+                        t = time.perf_counter()
+                    engine.step([Entry("long", ids[a:a + args.portion], [min(args.portion, args.context - a) - 1] if last else [])])
+                    if timed:
+                        sync()
+                        times.append(time.perf_counter() - t)
+                engine.finish("long")
+            ms = statistics.median(times) * 1e3
+            portion = {"context": args.context, "tokens": args.portion, "ms": round(ms, 3),
+                       "value": round(args.portion / (ms / 1e3), 1)}
         print(json.dumps({"metric": "prefill tok/s (%s shape, %d tokens)" % (args.model, PREFILL_TOKENS),
-                          "prefill": prefill, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32"}))
+                          "prefill": prefill, "portion": portion, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32"}))
         return 0
     main_point = decode(args.batch, args.steps, args.warmup)
     value, ms_per_step, achieved = main_point["tok_s"], main_point["ms"], main_point["gbs"]

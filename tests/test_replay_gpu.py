@@ -169,6 +169,36 @@ def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_m
         assert eng.graph_replays >= 4
 
 
+@pytest.mark.parametrize("model,page", [("tiny-c", 16), ("tiny-c", 32)])
+def test_portions_late_in_a_long_prompt(model, page, model_dirs, plain_models):
+    """700 tokens at once, then portions of 64, 40, 2 and 33 tokens, beside a second request's
+    whole prompt: the few tiles of a late portion are dealt to several blocks each (the
+    planner's choice is asserted), whose partial results join through memory."""
+    from pyre_amd.parts import fast
+
+    plain = plain_models[model]
+    cfg = plain[0]
+    ids = random_ids(cfg["vocab_size"], 839, seed=5)
+    other = random_ids(cfg["vocab_size"], 90, seed=6)
+    eng = make_engine(model_dirs[model], "bfloat16", page_size=page, max_cached_tokens=1200, max_num_batched_tokens=1024)
+    cuts = [0, 700, 764, 804, 806, 839]
+    steps = []
+    for k, (a, b) in enumerate(zip(cuts, cuts[1:])):
+        entries = [("a", ids[a:b], list(range(b - a)) if a else [b - a - 1])]
+        if k == 2:
+            entries.append(("b", other, list(range(90))))
+        steps.append((entries, ["a", "b"] if b == 839 else []))
+    got = replay(eng, steps)
+    want = {"a": plain_logits(plain, ids, torch.bfloat16), "b": plain_logits(plain, other, torch.bfloat16)}
+    bad, worst = first_bad(got, want, TOL["bfloat16"])
+    assert bad is None, bad
+    import numpy as np
+    tiles = np.asarray([[0, 32], [32, 32]], dtype=np.int32)
+    work = fast.prefill_work(tiles, np.arange(700, 764, dtype=np.int32), 0,
+                             fast.prefill_items(cfg["num_attention_heads"], cfg["num_key_value_heads"]))
+    assert work[:, 6].min() >= 2
+
+
 @pytest.mark.parametrize("others,graphs", [(30, True), (30, False), (150, True)])
 def test_decode_steps_of_requests_of_very_different_lengths(others, graphs, model_dirs, plain_models):
     """One request of 900 tokens and one of 400 among many of 3 to 40: the decode kernel's
