@@ -557,28 +557,51 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 // ---------------------------------------------------------------------------
 // Prefill on 32x32x16 tiles: the NW waves of a block take NW query heads of one
 // key/value head over the same 32 tokens (one MFMA tile of columns per wave);
-// keys and values come through LDS in chunks of 64, three stages, loaded once
+// keys and values come through LDS in chunks of 64, four stages, loaded once
 // per block. Per chunk and wave: S^T (64 keys x 32 tokens) in two tiles, one
 // exchange between the two lanes that share a column for the running maximum,
 // and O^T (HD x 32) += V^T P^T. The sum of a column is kept per lane (each lane
 // adds the keys it holds) and joined once at the end.
 //
-// A stage is K rows as stored, [key][HD + 8] (the padding puts 16 rows on distinct
-// banks), followed by V^T, [d][64 + 8]; within each run of 16 keys the V^T order is
-// (4g + j, 8 + 4g + j -> 8g + j, 8g + 4 + j), so that the eight keys a lane needs
-// for one MFMA are 16 contiguous bytes.
+// The chunks go from the cache straight into LDS (global_load_lds_dwordx4: 16 bytes
+// per lane, the 64 pieces of an instruction at consecutive LDS addresses, each from
+// an address of its lane's choosing), no register in between: two chunks are in
+// flight while two are being read, which hides the latency of L2 and memory that one
+// register set per wave could not (a 2,048-token portion after 30,000 tokens took
+// 1,230 us per layer on the 7B heads with staging through registers, 900 us with
+// loads that always hit). Such loads cannot pad rows, so rows are rotated instead:
+//   K    rows of SEGP slots of 16 bytes (SEGP = 4, 8 or 16 >= HD / 8), 64 of them; piece p
+//        of row j lies in slot (p + j / RPB) % SEGP, RPB = rows per 256 bytes, so that 16
+//        lanes reading the same piece of 16 consecutive rows hit distinct banks.
+//        Row 16 h + 8 a + 4 c + b of a tile of 32 holds key 16 h + 8 c + 4 a + b: with the
+//        rows in this order the eight scores that a lane packs for one MFMA of the second
+//        product belong to eight consecutive keys, and V^T needs no reordering.
+//   V^T  four runs of 16 keys, each [HD][16 keys] (32 bytes a row, two pieces); the piece
+//        of keys 8 x .. 8 x + 7 of row d lies in slot x ^ ((d >> 3) & 1).
+// A page that is not there (released, or past the request's end) is read from 16 bytes of
+// zeros instead: all its keys are out of every column's bounds, and a hidden key's value is
+// weighted with an exact 0, which only a finite value survives.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 64;
 
 // A barrier that waits for this wave's LDS traffic only. __syncthreads() also waits for
 // every global load in flight, which would put the latency of the next chunks' loads
-// into each half-step; their registers are waited for where they are used.
+// into each half-step.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// LOADER: the block's last wave has no head of its own (the group has fewer heads than
-// the block has waves) and does all the loading; the others only compute, and keep the
-// registers and the instructions of the loads for themselves.
+// 16 bytes per lane from global memory straight into LDS: lane x's piece lands at
+// lds_addr + 16 x. The compiler does not know of these loads; whoever reads the bytes
+// waits for them with wait_loads (they finish in the order of issue) and a barrier.
+__device__ inline void load_to_lds(const void* src, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
+}
+template <int N>
+__device__ inline void wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 0u, 0u};
+
 //
 // work[2 i], work[2 i + 1] = (first token of the tile in the flat batch, tokens <= 32, first
 // chunk of 64 keys, last chunk), (first partial slot of the tile, this block's number b among
@@ -590,23 +613,25 @@ __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_b
 // memory and counts itself in at the counter of (tile, head); the wave that arrives last
 // reads the nb partial results with loads that come from memory and joins them in the order
 // 0..nb-1, whichever wave it is, and leaves the counter at zero.
-template <int HD, int NW, bool LOADER>
+template <int HD, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, const int4* __restrict__ work, float* __restrict__ partials, int* __restrict__ counters,
-    int n_slots, const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
-    int table_stride, int nq, int nkv, int page_size, float scale_log2, int window) {
-  constexpr int KS = HD + 8, VS = kKeys + 8;
-  constexpr int SEG = HD / 8;            // 16-byte pieces of one K row
-  // A run of 16 keys is HD / 32 blocks of 64 pieces (1 KB) of K, contiguous in its page,
-  // and as many of V^T. Block `blk` of a run: K for blk < HD / 32, else V^T; a wave loads
-  // blocks wave, wave + NW, ... of each of the chunk's four runs, one piece per lane.
-  constexpr int BR = 2 * (HD / 32);      // blocks per run
-  constexpr int PB = (BR + NW - 1) / NW;  // blocks per run and wave
-  constexpr int PER = (kKeys / 16) * PB;
-  constexpr int NS = 3;                  // stages: a chunk is read during four half-steps (see below)
-  constexpr int kBytesK = 2 * kKeys * KS, kStage = kBytesK + 2 * HD * VS;  // bytes: a stage is K rows, then V^T rows
-  __shared__ __attribute__((aligned(16))) unsigned char lds[NS * kStage];
+    int n_slots, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+    const int* __restrict__ block_table, int table_stride, int nq, int nkv, int page_size, float scale_log2,
+    int window) {
+  constexpr int SEG = HD / 8;                              // 16-byte pieces of one K row
+  constexpr int SEGP = SEG <= 4 ? 4 : SEG <= 8 ? 8 : 16;   // slots of a K row in LDS
+  constexpr int KROW = 16 * SEGP;                          // bytes of a K row in LDS
+  constexpr int RPB = 16 / SEGP;                           // K rows per 256 bytes
+  constexpr int kBytesK = kKeys * KROW, kBytesV = 2 * HD * kKeys, kStage = kBytesK + kBytesV;
+  constexpr int VRUN = 32 * HD;                            // bytes of one run of V^T: [HD][16 keys]
+  constexpr int NS = 4;                                    // stages: two chunks being read, two in flight
+  constexpr int NI = 4;                                    // waves that issue loads: the first wave of each SIMD
+  constexpr int KI = kBytesK / 1024, VI = kBytesV / 1024;  // load instructions (1 KB each) per chunk
+  constexpr int PER = (KI + VI) / NI;                      // per issuing wave
+  static_assert((KI + VI) % NI == 0 && VRUN % 1024 == 0 && NS * kStage <= 160 * 1024 - 1024, "stage geometry");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[NS * kStage];
 
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r = lane & 31,
             g = lane >> 5;
@@ -642,100 +667,43 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
   const int lo_max = window > 0 ? max(0, hi_all - window + 1) : 0;
 
   const int n = last - first + 1;
-  if (LOADER && wave == NW - 1) {
-    // Chunk x is written in half-step 2x - 2, as soon as the chunk that lay in its stage
-    // has been left, and its loads were asked for two half-steps before that.
-    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-    int pi = (first * kKeys) / page_size, sl = (first * kKeys) % page_size;
-    const size_t page_elems = static_cast<size_t>(page_size) * HD;
-    u32x4 lr[(kKeys / 16) * BR];
-    auto fetch_all = [&]() {
-#pragma unroll
-      for (int run = 0; run < kKeys / 16; ++run) {
-        const int page = table[min(pi, table_stride - 1)];
-        const size_t base = (static_cast<size_t>(max(page, 0)) * nkv + kvh) * page_elems;
-#pragma unroll
-        for (int blk = 0; blk < BR; ++blk) {
-          constexpr int kHalfBlocks = HD / 32;
-          const bool is_k = blk < kHalfBlocks;
-          const int idx = (is_k ? blk : blk - kHalfBlocks) * 64 + lane;
-          const bf16* src = is_k ? k_cache + base + static_cast<size_t>(sl) * HD + 8 * idx
-                                 : v_cache + base + static_cast<size_t>(idx >> 1) * page_size + sl + 8 * (idx & 1);
-          // a page that is not there reads page 0, which may belong to anyone: its bytes are dropped
-          const unsigned keep = page < 0 ? 0u : ~0u;
-          const u32x4 got = *reinterpret_cast<const u32x4*>(src);
-          lr[run * BR + blk] = u32x4{got.x & keep, got.y & keep, got.z & keep, got.w & keep};
-        }
-        sl += 16;
-        const bool wrap = sl >= page_size;
-        sl = wrap ? 0 : sl;
-        pi += wrap ? 1 : 0;
-      }
-    };
-    auto stash_all = [&](int stage) {
-#pragma unroll
-      for (int run = 0; run < kKeys / 16; ++run)
-#pragma unroll
-        for (int blk = 0; blk < BR; ++blk) {
-          const u32x4 v = lr[run * BR + blk];
-          if (blk < HD / 32) {
-            const int idx = blk * 64 + lane;
-            *reinterpret_cast<u32x4*>(lds + stage * kStage + 2 * ((16 * run + idx / SEG) * KS + 8 * (idx % SEG))) = v;
-          } else {
-            const int idx = (blk - HD / 32) * 64 + lane, d = idx >> 1, h = idx & 1;
-            // keys 8h .. 8h+3 of the run go to places 4h .. 4h+3, keys 8h+4 .. 8h+7 to 8+4h .. 8+4h+3
-            unsigned char* dst = lds + stage * kStage + kBytesK + 2 * (d * VS + 16 * run + 4 * h);
-            *reinterpret_cast<uint2*>(dst) = uint2{v.x, v.y};
-            *reinterpret_cast<uint2*>(dst + 16) = uint2{v.z, v.w};
-          }
-        }
-    };
-    fetch_all();
-    stash_all(0);
-    if (1 < n) fetch_all();
-    lds_barrier();
-    int stage = 1;
-    for (int t = 0; t < 2 * n + 2; ++t) {
-      const int x = t / 2 + 1;
-      if ((t & 1) == 0 && x < n) {
-        stash_all(stage);
-        stage = stage == NS - 1 ? 0 : stage + 1;
-        if (x + 1 < n) fetch_all();
-      }
-      lds_barrier();
-    }
-    return;
-  }
 
-  // Where this wave's pieces come from and go to, fixed for the whole kernel. Block j of
-  // a run is K (rows of 16 keys as stored) or V^T (HD rows of 16 keys); the addresses of
-  // a piece differ from run to run by a multiple of the run's slot and of the run's index:
+  // Loads: the first NI waves issue them, instructions wave, wave + NI, ... of the chunk's
+  // KI + VI. An instruction's 64 pieces come from one run of 16 keys, so from one page. What
+  // is fixed for the whole kernel is worked out here:
   //   global: cache + ((page * nkv + kvh) * page_size * HD + slot * g_mul) + g_lane
-  //   LDS:    stage * kStage + run * l_run + l_lane, two 8-byte halves 8 or 16 bytes apart
-  // No branch depends on the page, the block or the run: scalar branches cost far more
-  // here than the few values they would save.
-  const bf16* g_ptr[PB];
-  int g_lane[PB], g_mul[PB], l_lane[PB], l_run[PB], l_half[PB];
+  //   LDS:    stage * kStage + g_lds
+  const bool issuer = wave < NI;
+  const unsigned lds_base = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds)));
+  const bf16* g_ptr[PER];
+  int g_run[PER], g_mul[PER], g_lane[PER], g_lds[PER];
 #pragma unroll
-  for (int j = 0; j < PB; ++j) {
-    const int blk = min(wave + NW * j, BR - 1);  // a wave beyond the last block repeats it (same bytes, same place)
-    const bool is_k = blk < HD / 32;
-    const int idx = (is_k ? blk : blk - HD / 32) * 64 + lane;
-    g_ptr[j] = is_k ? k_cache : v_cache;
-    g_mul[j] = is_k ? HD : 1;
-    g_lane[j] = is_k ? 8 * idx : (idx >> 1) * page_size + 8 * (idx & 1);
-    // V^T: keys 8h .. 8h+3 of the run go to places 4h .. 4h+3, keys 8h+4 .. 8h+7 to 8+4h .. 8+4h+3
-    l_lane[j] = is_k ? 2 * ((idx / SEG) * KS + 8 * (idx % SEG)) : kBytesK + 2 * ((idx >> 1) * VS + 4 * (idx & 1));
-    l_run[j] = is_k ? 2 * 16 * KS : 2 * 16;
-    l_half[j] = is_k ? 8 : 16;
+  for (int t = 0; t < PER; ++t) {
+    const int j = min(wave, NI - 1) + NI * t;
+    g_lds[t] = 1024 * j;
+    if (j < KI) {
+      const int row = j * (1024 / KROW) + lane / SEGP, slot = lane % SEGP;
+      int piece = (slot + SEGP - (row / RPB) % SEGP) % SEGP;
+      if (piece >= SEG) piece = 0;  // a slot that no piece maps to (heads of 96): any bytes that are there
+      const int in_tile = row & 31;
+      const int key = (row & 32) + (in_tile & 16) + 8 * ((in_tile >> 2) & 1) + 4 * ((in_tile >> 3) & 1) + (in_tile & 3);
+      g_ptr[t] = k_cache;
+      g_run[t] = __builtin_amdgcn_readfirstlane(key >> 4);
+      g_mul[t] = HD;
+      g_lane[t] = (key & 15) * HD + 8 * piece;
+    } else {
+      const int jv = j - KI;
+      const int d = 32 * (jv % (VRUN / 1024)) + (lane >> 1), half = (lane & 1) ^ ((d >> 3) & 1);
+      g_ptr[t] = v_cache;
+      g_run[t] = jv / (VRUN / 1024);
+      g_mul[t] = 1;
+      g_lane[t] = d * page_size + 8 * half;
+    }
   }
   // (pi, sl): index into the block table and slot within that page of the first key of
   // the next chunk to look up; both advance by whole runs, without a division per chunk.
-  // The pages of a chunk are looked up one load ahead of the chunk's own loads, so that
-  // the latency of the table is never waited for. A page that is not there (released, or
-  // past the request's end) reads page 0 instead and is replaced by zeros: all its keys are
-  // out of every column's bounds, and a hidden key's value is weighted with an exact 0,
-  // which only a finite value survives.
+  // The pages of a chunk are looked up one chunk ahead of its loads, so that the latency
+  // of the table is never waited for.
   int pi = (first * kKeys) / page_size, sl = (first * kKeys) % page_size;
   int run_page[kKeys / 16], run_slot[kKeys / 16];
   auto lookup = [&]() {
@@ -750,70 +718,66 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     }
   };
   const size_t page_elems = static_cast<size_t>(page_size) * HD;
-  auto fetch = [&](uint4 (&regs)[PER]) {
+  // The chunk whose pages were looked up last goes into `stage`.
+  auto issue = [&](int stage) {
     size_t base[kKeys / 16];
     int slot[kKeys / 16];
-    unsigned keep[kKeys / 16];
+    bool there[kKeys / 16];
 #pragma unroll
     for (int run = 0; run < kKeys / 16; ++run) {
       base[run] = (static_cast<size_t>(max(run_page[run], 0)) * nkv + kvh) * page_elems;
       slot[run] = run_slot[run];
-      keep[run] = run_page[run] < 0 ? 0u : ~0u;  // page 0 stands in, and may belong to anyone: its bytes are dropped
+      there[run] = run_page[run] >= 0;
     }
     lookup();  // for the chunk after this one
+    const unsigned dst = lds_base + stage * kStage;
 #pragma unroll
-    for (int run = 0; run < kKeys / 16; ++run)
-#pragma unroll
-      for (int j = 0; j < PB; ++j) {
-        const uint4 got = *reinterpret_cast<const uint4*>(g_ptr[j] + base[run] + slot[run] * g_mul[j] + g_lane[j]);
-        regs[run * PB + j] = uint4{got.x & keep[run], got.y & keep[run], got.z & keep[run], got.w & keep[run]};
-      }
-  };
-  auto stash = [&](int stage, const uint4 (&regs)[PER]) {
-#pragma unroll
-    for (int run = 0; run < kKeys / 16; ++run)
-#pragma unroll
-      for (int j = 0; j < PB; ++j) {
-        unsigned char* dst = lds + stage * kStage + run * l_run[j] + l_lane[j];
-        const uint4 v = regs[run * PB + j];
-        *reinterpret_cast<uint2*>(dst) = uint2{v.x, v.y};
-        *reinterpret_cast<uint2*>(dst + l_half[j]) = uint2{v.z, v.w};
-      }
+    for (int t = 0; t < PER; ++t) {
+      const int run = g_run[t];
+      const size_t b = run == 0 ? base[0] : run == 1 ? base[1] : run == 2 ? base[2] : base[3];
+      const int sr = run == 0 ? slot[0] : run == 1 ? slot[1] : run == 2 ? slot[2] : slot[3];
+      const bool ok = run == 0 ? there[0] : run == 1 ? there[1] : run == 2 ? there[2] : there[3];
+      const bf16* src = ok ? g_ptr[t] + b + sr * g_mul[t] + g_lane[t] : reinterpret_cast<const bf16*>(kZeroPiece);
+      load_to_lds(src, dst + g_lds[t]);
+    }
   };
 
   // The loop runs in half-steps with a barrier after each. A wave alternates between a
   // matrix half-step (O^T += V^T P^T of the previous chunk, then S^T of the next) and an
-  // arithmetic half-step (softmax of that S^T, its share of the loads). The second wave of
-  // each SIMD (waves NW/2 ..) runs one half-step behind the first, so that at any time one
-  // of the two is on the matrix cores and the other on the vector ALU.
-  //   chunk x (counted from `first`) is read in half-steps 2x .. 2x+3, lies in stage x % 3,
-  //   and is written in half-steps 2x-2 (second waves) and 2x-1 (first waves).
+  // arithmetic half-step (softmax of that S^T; the issuing waves ask for the chunk after
+  // the next first and wait for the next one last). The second wave of each SIMD
+  // (waves NW/2 ..) runs one half-step behind the first, so that at any time one of the
+  // two is on the matrix cores and the other on the vector ALU.
+  //   chunk x (counted from `first`) is read in half-steps 2x-1 .. 2x+2 and lies in stage
+  //   x % 4; its loads are issued in half-step 2x-4, when chunk x-4 was last read in 2x-6,
+  //   and have arrived before the barrier that ends half-step 2x-2.
   const int off = NW == 8 ? wave >> 2 : 0;
-  uint4 regs[PER];
-  int held = 1, held_stage = 1;  // the chunk whose pieces `regs` holds, and its stage
-  if (!LOADER) {
+  if (issuer) {
     lookup();
-    fetch(regs);
-    stash(0, regs);
-    if (held < n) fetch(regs);
+    issue(0);
   }
   // The query operands have arrived before the loop starts. Without this the compiler,
-  // which cannot tell the first round from the others, waits for all loads in flight
-  // (the next chunk's among them) before the first product of every round.
+  // which cannot tell the first round from the others, waits in every round for all loads
+  // in flight; here that wait takes in the first chunk, which is needed now anyway.
 #pragma unroll
   for (int c = 0; c < HD / 16; ++c) asm volatile("" : "+v"(qr[c]));
+  if (issuer) {
+    wait_loads<0>();
+    if (1 < n) issue(1);
+  }
   lds_barrier();
   f32x16 s[2];
   bf16x8 p[2][2];
+  const int k_swz = (r / RPB) % SEGP;  // the rotation of row 32 kt + r is the same for both tiles: 32 / RPB is a multiple of SEGP
 
-  // S^T of the chunk in stage sk: tile kt has rows = keys key0 + 32 kt + 8 (i / 4) + 4 g + i % 4, column r.
+  // S^T of the chunk in stage sk: tile kt, row i of a lane = key key0 + 32 kt + 16 (i / 8) + 8 g + 4 (i / 4 % 2) + i % 4, column r.
   auto scores = [&](int sk) {
     constexpr int AHEAD = 4;  // head slices whose operands are in flight
     bf16x8 a[AHEAD][2];
     auto load_k = [&](int slot, int cc) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
-        a[slot][kt] = *reinterpret_cast<const bf16x8*>(lds + sk * kStage + 2 * ((32 * kt + r) * KS + 16 * cc + 8 * g));
+        a[slot][kt] = *reinterpret_cast<const bf16x8*>(lds + sk * kStage + (32 * kt + r) * KROW + 16 * ((2 * cc + g + k_swz) % SEGP));
     };
 #pragma unroll
     for (int cc = 0; cc < AHEAD && cc < HD / 16; ++cc) load_k(cc, cc);
@@ -829,13 +793,14 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
       if (cc + AHEAD < HD / 16) load_k(cc % AHEAD, cc + AHEAD);
     }
   };
-  // O^T += V^T P^T for the chunk in stage sv; k = the chunk's keys in the order P^T holds them.
+  // O^T += V^T P^T for the chunk in stage sv; MFMA `pair` takes keys 16 pair .. 16 pair + 15, eight per half-wave.
   auto weighted_values = [&](int sv) {
     bf16x8 va[2][HD / 32];
-    auto load_v = [&](int slot, int pair) {  // pair = 2 kt + h
+    const int v_lane = r * 32 + 16 * (g ^ ((r >> 3) & 1));
+    auto load_v = [&](int slot, int pair) {
 #pragma unroll
       for (int dt = 0; dt < HD / 32; ++dt)
-        va[slot][dt] = *reinterpret_cast<const bf16x8*>(lds + sv * kStage + kBytesK + 2 * ((32 * dt + r) * VS + 16 * pair + 8 * g));
+        va[slot][dt] = *reinterpret_cast<const bf16x8*>(lds + sv * kStage + kBytesK + pair * VRUN + dt * 1024 + v_lane);
     };
     load_v(0, 0);
     load_v(1, 1);
@@ -854,7 +819,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int key = key0 + 32 * kt + 8 * (i >> 2) + 4 * g + (i & 3);
+          const int key = key0 + 32 * kt + 16 * (i >> 3) + 8 * g + 4 * ((i >> 2) & 1) + (i & 3);
           if (key < lo || key > hi) s[kt][i] = -INFINITY;
         }
     }
@@ -891,27 +856,20 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
         for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
     }
   };
-  // This wave's share of the loads: the held chunk into its stage, the next one into registers.
-  auto load_work = [&]() {
-    if (LOADER) return;
-    if (held < n) stash(held_stage, regs);
-    ++held;
-    held_stage = held_stage == NS - 1 ? 0 : held_stage + 1;
-    if (held < n) fetch(regs);
-  };
 
-  if (off) {  // the second waves start one half-step later
-    load_work();
-    lds_barrier();
-  }
+  if (off) lds_barrier();  // the second waves start one half-step later
   if (active) scores(0);
   int st = 0;  // stage of chunk c
   for (int c = 0; c < n; ++c) {
     lds_barrier();
+    if (issuer && c + 2 < n) issue((st + 2) % NS);
     if (active) softmax((first + c) * kKeys);
-    load_work();
+    if (issuer) {  // chunk c + 1 is there
+      if (c + 2 < n) wait_loads<PER>();
+      else wait_loads<0>();
+    }
     lds_barrier();
-    const int nx = st == NS - 1 ? 0 : st + 1;
+    const int nx = (st + 1) % NS;
     if (active) {
       weighted_values(st);
       if (c + 1 < n) scores(nx);
@@ -1075,7 +1033,7 @@ extern "C" int pyre_attn_prefill_work_bf16(const void* q, void* out, const void*
                                            const int* work, int n_items, float* partials, int* counters,
                                            int n_slots, const int* positions, const int* seq_of_token, const int* block_table,
                                            int table_stride, int nq, int nkv, int hd, int page_size, float scale,
-                                           int window, int loader, hipStream_t stream) {
+                                           int window, hipStream_t stream) {
   PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv) && hd <= 128,
                "attn_prefill_work_bf16: head_dim %d (multiples of 32 up to 128), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
@@ -1088,27 +1046,17 @@ extern "C" int pyre_attn_prefill_work_bf16(const void* q, void* out, const void*
   PYRE_REQUIRE(n_items <= 65535, "attn_prefill_work_bf16: a list of %d blocks is too long for one launch", n_items);
   // the blocks of one row of the list are neighbours in the order of dispatch: the list's order is the order of starts
   const dim3 grid(nkv * hgroups, n_items);
-  // a wave to spare in every block (one group of fewer heads than waves): it loads for the others
-  const bool use_loader = n_rep < nw && loader != 0;
 #define PYRE_PREFILL_ARGS                                                                                          \
   static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache),               \
       static_cast<bf16*>(out), reinterpret_cast<const int4*>(work), partials, counters, n_slots, positions,        \
-      seq_of_token,                                                                                                \
-      block_table, table_stride, nq, nkv, page_size, scale * kLog2e, window
+      seq_of_token, block_table, table_stride, nq, nkv, page_size, scale * kLog2e, window
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
     if constexpr (HD <= 128) {
-      if (nw == 8) {
-        if (use_loader)
-          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8, true>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
-        else
-          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8, false>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
-      } else {
-        if (use_loader)
-          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, true>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
-        else
-          hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4, false>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
-      }
+      if (nw == 8)
+        hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 8>), grid, dim3(512), 0, stream, PYRE_PREFILL_ARGS);
+      else
+        hipLaunchKernelGGL((attn_prefill_tile32_kernel<HD, 4>), grid, dim3(256), 0, stream, PYRE_PREFILL_ARGS);
     }
   });
 #undef PYRE_PREFILL_ARGS

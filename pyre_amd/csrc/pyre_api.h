@@ -111,8 +111,8 @@ int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const 
                            int nq, int nkv, int hd, int page_size, float scale, int window,
                            hipStream_t stream);
 
-// The same for heads of up to 128 elements from a work list: K and V go through LDS in chunks
-// of 64 keys for 32x32 MFMA tiles, and the chunks of a tile may be dealt to several blocks.
+// The same for heads of up to 128 elements from a work list: K and V go straight into LDS in
+// chunks of 64 keys for 32x32 MFMA tiles, and the chunks of a tile may be dealt to several blocks.
 // work[2 i] = (first token of the tile, tokens <= 32, first chunk, last chunk), work[2 i + 1] =
 // (first partial slot of the tile, this block's number among the tile's blocks, their number
 // nb, 0); the nb blocks of a tile cover the chunks lo / 64 .. hi / 64 of the keys lo .. hi that
@@ -120,13 +120,13 @@ int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache, const 
 // query head of a key/value head (groups of that many heads: `groups`). Scratch for tiles
 // of more than one block: partials [slots, nkv * groups, waves, hd / 32 * 1024 + 128] floats
 // and counters [slots, nkv * groups, waves] ints that are zero before the first call and are
-// left at zero. `loader`: a block with a wave to spare lets it do all the loading.
+// left at zero.
 int pyre_attn_prefill_waves(int nq, int nkv);
 int pyre_attn_prefill_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
                                 const int* work, int n_items, float* partials, int* counters,
                                 int n_slots, const int* positions, const int* seq_of_token, const int* block_table,
                                 int table_stride, int nq, int nkv, int hd, int page_size, float scale,
-                                int window, int loader, hipStream_t stream);
+                                int window, hipStream_t stream);
 
 // scratch: m * 64 floats followed by m * 64 ints of device memory.
 int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, int m, int vocab,

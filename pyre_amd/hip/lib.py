@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 class KernelError(RuntimeError):
@@ -36,7 +36,7 @@ _SIGNATURES = {
     "pyre_attn_decode_work_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_waves": [I, I],
-    "pyre_attn_prefill_work_bf16": [P, P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+    "pyre_attn_prefill_work_bf16": [P, P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
     "pyre_argmax_static": [P, L, P, I, I, P],
     "pyre_gemm_skinny_supports": [I, I, I, L, L],

@@ -438,7 +438,7 @@ def attn_prefill_waves(nq: int, nkv: int) -> int:
 
 
 def attn_prefill_work_bf16(q, out, k_cache, v_cache, work, n_items, partials, counters, n_slots, positions,
-                           seq_of_token, block_table, nq, nkv, hd, page_size, scale, window=0, loader=True) -> None:
+                           seq_of_token, block_table, nq, nkv, hd, page_size, scale, window=0) -> None:
     """Attention of prompt portions for heads of up to 128 elements from a work list (int32
     ``[n_items, 8]``: see ``pyre_attn_prefill_work_bf16`` in pyre_api.h) whose tiles of several
     blocks use the partial slots 0..n_slots-1. ``counters`` must be zero and is left at zero."""
@@ -454,7 +454,7 @@ def attn_prefill_work_bf16(q, out, k_cache, v_cache, work, n_items, partials, co
     call("pyre_attn_prefill_work_bf16", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
          work.data_ptr(), n_items, _ptr(partials) if n_slots else None, _ptr(counters) if n_slots else None,
          n_slots, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0),
-         nq, nkv, hd, page_size, float(scale), int(window), int(bool(loader)), _stream())
+         nq, nkv, hd, page_size, float(scale), int(window), _stream())
 
 
 def gemm_skinny_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:

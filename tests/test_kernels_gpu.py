@@ -451,8 +451,7 @@ def test_attn_decode_work_list_in_a_mixed_batch():
     assert (got[others] == 7.0).all()
 
 
-def prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window=0, size=None,
-                      loader=True):
+def prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window=0, size=None):
     """Prompt portions through the kernel for the head size: from a work list planned as the
     engine plans it (or with blocks of ``size`` chunks of 64 keys) for heads of up to 128
     elements, from the tiles themselves for larger ones. Returns the work list, if any."""
@@ -470,21 +469,21 @@ def prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, h
     partials = torch.full((max(1, n_slots) * per_slot * (hd // 32 * 1024 + 128),), float("nan"), device=DEV)
     counters = torch.zeros(max(1, n_slots) * per_slot, dtype=torch.int32, device=DEV)
     ops.attn_prefill_work_bf16(q, out, kc, vc, i32(work.reshape(-1).tolist()), len(work), partials, counters, n_slots,
-                               pos, seq_of, table, nq, nkv, hd, page, scale, window, loader)
+                               pos, seq_of, table, nq, nkv, hd, page, scale, window)
     assert int(counters.abs().sum()) == 0
     return work
 
 
-@pytest.mark.parametrize("size,loader", [(None, True), (None, False), (3, True), (1, False)])
+@pytest.mark.parametrize("size", [None, 3, 1])
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 50, 300])
-def test_attn_prefill_mfma(nq, nkv, hd, page, window, size, loader):
+def test_attn_prefill_mfma(nq, nkv, hd, page, window, size):
     """Prompt portions of several requests. Blocks of one or three chunks of 64 keys deal the
     tiles of the longer requests to many blocks, whose partial results join through memory."""
     ops = _ops()
     from pyre_amd.parts.attention import TILE
 
-    if hd > 128 and (size is not None or not loader):
+    if hd > 128 and size is not None:
         pytest.skip("larger heads have one form")
     ctx_lens, q_lens = [2, 40, 97, 700, 1100], [2, 40, 33, 3, 600]
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=4)
@@ -497,7 +496,7 @@ def test_attn_prefill_mfma(nq, nkv, hd, page, window, size, loader):
     outs = []
     for _ in range(2):                                              # the second call finds the counters as the first left them
         out = torch.full_like(q, float("nan"))
-        work = prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window, size, loader)
+        work = prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window, size)
         assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
         outs.append(out)
     assert torch.equal(outs[0], outs[1])
