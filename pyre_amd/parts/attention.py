@@ -7,6 +7,7 @@ import torch
 import numpy as np
 
 from pyre_amd.hip import ops
+from pyre_amd.parts import attention_work as plan
 from pyre_amd.parts import fast
 from pyre_amd.parts.base import (AttentionSpec, Mixer, PagedCacheSpec, PagedTensorSpec, StepArraySpec, TensorSpec,
                                  make_part)
@@ -82,18 +83,18 @@ class Attention(Mixer):
         s = self.spec
 
         def work(hb):
-            return fast.decode_work(hb.arrays["attention.decode_tokens"], hb.positions, hb.decode_shape()[0],
+            return plan.decode_work(hb.arrays["attention.decode_tokens"], hb.positions, hb.decode_shape()[0],
                                     s.window, s.num_heads, s.num_kv_heads)
 
         def portions(hb):
-            return fast.prefill_work(hb.arrays["attention.prefill_tiles"], hb.positions, s.window,
-                                     fast.prefill_items(s.num_heads, s.num_kv_heads))
+            return plan.prefill_work(hb.arrays["attention.prefill_tiles"], hb.positions, s.window,
+                                     plan.prefill_items(s.num_heads, s.num_kv_heads))
 
         return [*STEP_ARRAYS,
                 StepArraySpec(self.decode_work_name,
-                              lambda n_cap, s_cap: 4 * (1 + fast.decode_capacity(s_cap, s.num_heads, s.num_kv_heads)), work),
+                              lambda n_cap, s_cap: 4 * (1 + plan.decode_capacity(s_cap, s.num_heads, s.num_kv_heads)), work),
                 StepArraySpec(self.prefill_work_name,
-                              lambda n_cap, s_cap: 8 * (n_cap // TILE + s_cap + 2 * fast.DECODE_UNITS + 1), portions)]
+                              lambda n_cap, s_cap: 8 * (n_cap // TILE + s_cap + 2 * plan.DECODE_UNITS + 1), portions)]
 
     def linears(self) -> list:
         return [self.qkv, self.out]

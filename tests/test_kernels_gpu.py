@@ -358,7 +358,7 @@ def test_attn_decode_mfma(nq, nkv, hd, page, window, size):
 def decode_attention(ops, q, out, kc, vc, tokens, pos, seq_of, table, nq, nkv, hd, page, scale, window=0, size=None,
                      rows=None, alone=None):
     """The decode kernel on the single tokens ``tokens`` with a list planned as the engine plans it."""
-    from pyre_amd.parts.fast import decode_alone, decode_capacity, decode_items, decode_work
+    from pyre_amd.parts.attention_work import decode_alone, decode_capacity, decode_items, decode_work
 
     tokens = np.asarray(tokens, dtype=np.int32)
     rows = rows or len(tokens)
@@ -390,7 +390,7 @@ def test_attn_decode_from_a_work_list(nq, nkv, hd, page, window, size, alone):
     through memory). The second call finds the counters as the first left them; the third
     plans for a larger step, as a captured one would, and must give the same bits."""
     ops = _ops()
-    from pyre_amd.parts.fast import decode_capacity, decode_items, decode_work
+    from pyre_amd.parts.attention_work import decode_capacity, decode_items, decode_work
 
     ctx_lens = [1, 31, 32, 33, 700, 2049, 129, 5]
     q_lens = [1] * len(ctx_lens)
@@ -429,7 +429,7 @@ def test_attn_decode_work_list_in_a_mixed_batch():
     """Single tokens between the tokens of prompt portions: the list names them by their
     place in the flat batch, and nothing else is written."""
     ops = _ops()
-    from pyre_amd.parts.fast import decode_capacity, decode_items, decode_work
+    from pyre_amd.parts.attention_work import decode_capacity, decode_items, decode_work
 
     nq, nkv, hd, page = 28, 4, 128, 16
     ctx_lens, q_lens = [300, 40, 1500, 64, 9], [1, 7, 1, 33, 1]
@@ -455,7 +455,7 @@ def prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, h
     """Prompt portions through the kernel for the head size: from a work list planned as the
     engine plans it (or with blocks of ``size`` chunks of 64 keys) for heads of up to 128
     elements, from the tiles themselves for larger ones. Returns the work list, if any."""
-    from pyre_amd.parts.fast import prefill_items, prefill_slots, prefill_work
+    from pyre_amd.parts.attention_work import prefill_items, prefill_slots, prefill_work
 
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
     if hd > 128:

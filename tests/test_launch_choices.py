@@ -6,8 +6,9 @@ import random
 
 import numpy as np
 
-from pyre_amd.parts.fast import (DECODE_MAX_BLOCKS_PER_REQUEST, DECODE_UNITS, SKINNY_MAX_KSPLIT, decode_alone,
-                                 decode_capacity, decode_work, prefill_slots, prefill_work, skinny_ksplit)
+from pyre_amd.parts.attention_work import (DECODE_MAX_BLOCKS_PER_REQUEST, DECODE_UNITS, decode_alone, decode_capacity,
+                                           decode_work, prefill_slots, prefill_work)
+from pyre_amd.parts.fast import SKINNY_MAX_KSPLIT, skinny_ksplit
 
 
 def test_split_k_leaves_no_part_empty_and_is_a_function_of_the_sizes():

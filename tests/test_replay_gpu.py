@@ -174,7 +174,7 @@ def test_portions_late_in_a_long_prompt(model, page, model_dirs, plain_models):
     """700 tokens at once, then portions of 64, 40, 2 and 33 tokens, beside a second request's
     whole prompt: the few tiles of a late portion are dealt to several blocks each (the
     planner's choice is asserted), whose partial results join through memory."""
-    from pyre_amd.parts import fast
+    from pyre_amd.parts import attention_work as fast
 
     plain = plain_models[model]
     cfg = plain[0]
