@@ -504,6 +504,43 @@ def test_attn_prefill_mfma(nq, nkv, hd, page, window, size):
         assert work[:, 6].max() >= 6                                # the long request's tiles span many blocks
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_attention_work_lists_on_random_batches(seed):
+    """Random numbers of requests with random contexts, windows and head counts, some with a
+    portion of their prompt and some with a single token, through both MFMA kernels with the
+    lists the planner makes for them: every row against the plain attention."""
+    ops = _ops()
+    rng = random.Random(100 + seed)
+    nkv = rng.choice([1, 2, 4])
+    nq = nkv * rng.choice([1, 3, 7, 8])
+    hd, page = rng.choice([(64, 16), (128, 16), (128, 32), (32, 48), (96, 16)])
+    window = rng.choice([0, 0, 200])
+    n_req = rng.randrange(1, 24)
+    ctx_lens, q_lens = [], []
+    for _ in range(n_req):
+        ctx = int(math.exp(rng.uniform(0, math.log(2500)))) + 1
+        ql = 1 if rng.random() < 0.6 else rng.randrange(2, min(ctx, 130) + 1)
+        ctx_lens.append(max(ctx, ql))
+        q_lens.append(ql)
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=seed)
+    scale = hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    out = torch.full_like(q, float("nan"))
+    singles, tiles, base = [], [], 0
+    for ql in q_lens:
+        if ql == 1:
+            singles.append(base)
+        else:
+            tiles += [(t0, min(32, base + ql - t0)) for t0 in range(base, base + ql, 32)]
+        base += ql
+    if singles:
+        decode_attention(ops, q, out, kc, vc, singles, pos, seq_of, table, nq, nkv, hd, page, scale, window,
+                         rows=len(singles) + rng.randrange(0, 5))
+    if tiles:
+        prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale, window)
+    assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2), (nq, nkv, hd, page, window, ctx_lens, q_lens)
+
+
 def test_attn_prefill_of_a_portion_late_in_a_long_context():
     """64 tokens at the end of 6,000: two tiles, which the planner deals to as many blocks as
     the chip has units; the result is that of undivided tiles up to rounding."""
