@@ -112,6 +112,10 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
     return True
 
 
+#: rows of the prompt-portion kernel's work list that one launch takes (the grid's second dimension)
+PREFILL_MAX_LAUNCH = 65535
+
+
 def attention(mixer, ctx, q, o, cache) -> bool:
     from pyre_amd.hip import ops
     from pyre_amd.parts.attention_work import (decode_alone, decode_capacity, decode_items, prefill_items,
@@ -151,9 +155,12 @@ def attention(mixer, ctx, q, o, cache) -> bool:
             partials = ctx.workspace.get("attn.prefill_partials", (n_slots, per_slot, s.head_dim // 32 * 1024 + 128),
                                          torch.float32)
             counters = ctx.workspace.get("attn.prefill_counters", (n_slots, per_slot), torch.int32, zeroed=True)
-        ops.attn_prefill_work_bf16(q, o, k_pages, v_pages, ctx.arrays[mixer.prefill_work_name], len(work), partials,
-                                   counters, n_slots, ctx.positions, ctx.seq_of_token, cache.table, s.num_heads,
-                                   s.num_kv_heads, s.head_dim, cache.page_size, mixer.scale, cache.window)
+        listed = ctx.arrays[mixer.prefill_work_name]
+        for at in range(0, len(work), PREFILL_MAX_LAUNCH):  # a launch takes 65,535 rows of the list
+            count = min(PREFILL_MAX_LAUNCH, len(work) - at)
+            ops.attn_prefill_work_bf16(q, o, k_pages, v_pages, listed[8 * at:], count, partials, counters, n_slots,
+                                       ctx.positions, ctx.seq_of_token, cache.table, s.num_heads, s.num_kv_heads,
+                                       s.head_dim, cache.page_size, mixer.scale, cache.window)
     elif n_tiles:
         ops.attn_prefill_bf16(q, o, k_pages, v_pages, ctx.arrays["attention.prefill_tiles"], n_tiles, ctx.positions,
                               ctx.seq_of_token, cache.table, s.num_heads, s.num_kv_heads, s.head_dim,

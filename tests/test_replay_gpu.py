@@ -169,12 +169,17 @@ def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_m
         assert eng.graph_replays >= 4
 
 
-@pytest.mark.parametrize("model,page", [("tiny-c", 16), ("tiny-c", 32)])
-def test_portions_late_in_a_long_prompt(model, page, model_dirs, plain_models):
+@pytest.mark.parametrize("model,page,per_launch", [("tiny-c", 16, None), ("tiny-c", 32, None), ("tiny-c", 16, 5)])
+def test_portions_late_in_a_long_prompt(model, page, per_launch, model_dirs, plain_models, monkeypatch):
     """700 tokens at once, then portions of 64, 40, 2 and 33 tokens, beside a second request's
     whole prompt: the few tiles of a late portion are dealt to several blocks each (the
-    planner's choice is asserted), whose partial results join through memory."""
+    planner's choice is asserted), whose partial results join through memory. With five rows
+    of the work list per launch the blocks of a tile also lie in different launches."""
     from pyre_amd.parts import attention_work as fast
+    from pyre_amd.parts import fast as kernel_choice
+
+    if per_launch:
+        monkeypatch.setattr(kernel_choice, "PREFILL_MAX_LAUNCH", per_launch)
 
     plain = plain_models[model]
     cfg = plain[0]
