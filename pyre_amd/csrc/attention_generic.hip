@@ -1,6 +1,6 @@
 // Causal (optionally windowed) attention of every token of a step over the paged
 // cache, for any head size up to 256, any page size, any grouping of heads and
-// either element type; all arithmetic fp32. One block per (token, query head).
+// either element type; all arithmetic fp32. One block per (token, query head, span of keys).
 //
 //   scores[j] = (q . k_j) * scale      for lo <= j <= pos     (pyre/model.py:109)
 //   probs     = softmax(scores)                               (pyre/model.py:122)
@@ -10,8 +10,11 @@
 // A token at position `pos` sees the keys lo..pos of its request, all read from
 // the cache (this step's keys were written before the call), so prompt portions
 // and single decoded tokens are the same case. lo = max(0, pos - window + 1) for
-// a window, else 0. The order of every sum depends on (lo, pos) alone, so the
-// result for a position does not depend on how the step was cut or batched.
+// a window, else 0. The keys of a token are taken in spans of 512, one block each (grid.z),
+// whose partial results (max, sum, unnormalised output) a second kernel joins in the order of
+// the spans; a launch whose block tables hold no more than one span writes the result
+// directly. The order of every sum depends on (lo, pos) alone, so the result for a position
+// does not depend on how the step was cut or batched.
 // This is the 32-bit path's attention and the 16-bit path's fallback; it stands
 // where the reference has `forward_paged`'s gather + matmuls (pyre/model.py:274-290)
 // and its decode kernel (pyre/kernels/paged_attn.py:26-71).
@@ -23,7 +26,7 @@ using namespace pyre;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kChunk = 1024;   // keys whose scores are held in LDS at a time
+constexpr int kSpan = 512;     // keys that one block takes, and whose scores are held in LDS
 constexpr int kMaxHead = 256;
 
 template <typename TQ, typename TC>
@@ -31,9 +34,9 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
     TQ* __restrict__ out, const int* __restrict__ tokens, const int* __restrict__ positions,
     const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride, int nq, int nkv,
-    int hd, int page_size, float scale, int window) {
+    int hd, int page_size, float scale, int window, float* __restrict__ part) {
   __shared__ float qs[kMaxHead];
-  __shared__ float sc[kChunk];
+  __shared__ float sc[kSpan];
   __shared__ float accs[kThreads];
   __shared__ float scratch[16];
 
@@ -42,6 +45,8 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
   const int pos = positions[n];
   const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int base = lo + static_cast<int>(blockIdx.z) * kSpan;  // this block's span
+  if (base > pos) return;
 
   for (int d = tid; d < hd; d += kThreads) qs[d] = to_float(q[(static_cast<size_t>(n) * nq + h) * hd + d]);
   __syncthreads();
@@ -53,8 +58,8 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
   const bool active = g < groups;
 
   float m = -INFINITY, l = 0.f, acc = 0.f;
-  for (int base = lo; base <= pos; base += kChunk) {
-    const int cnt = min(kChunk, pos - base + 1);
+  {
+    const int cnt = min(kSpan, pos - base + 1);
     float lmax = -INFINITY;
     for (int j = tid; j < cnt; j += kThreads) {
       const int key = base + j;
@@ -69,18 +74,16 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
       sc[j] = s;
       lmax = fmaxf(lmax, s);
     }
-    const float m_new = fmaxf(m, block_max(lmax, scratch));
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = expf(m - m_use);  // 0 on the first chunk (m = -inf)
+    m = block_max(lmax, scratch);
+    const float m_use = m == -INFINITY ? 0.f : m;
     float lsum = 0.f;
     for (int j = tid; j < cnt; j += kThreads) {
       const float p = expf(sc[j] - m_use);
       sc[j] = p;
       lsum += p;
     }
-    l = l * alpha + block_sum(lsum, scratch);  // block_sum's barriers publish sc[]
+    l = block_sum(lsum, scratch);  // block_sum's barriers publish sc[]
     if (active) {
-      acc *= alpha;
       for (int j = g; j < cnt; j += groups) {
         const int key = base + j;
         const int page = table[key / page_size], off = key % page_size;
@@ -89,8 +92,6 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
         acc = fmaf(sc[j], to_float(*vp), acc);
       }
     }
-    m = m_new;
-    __syncthreads();  // sc[] is rewritten by the next chunk
   }
 
   accs[tid] = active ? acc : 0.f;
@@ -98,28 +99,76 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
   if (tid < hd) {
     float total = 0.f;
     for (int gg = 0; gg < groups; ++gg) total += accs[gg * hd + tid];
+    if (part) {  // [token of the list][head][span][hd + 2]: unnormalised output, max, sum
+      float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + h) * gridDim.z + blockIdx.z) * (hd + 2);
+      dst[tid] = total;
+      if (tid == 0) {
+        dst[hd] = m;
+        dst[hd + 1] = l;
+      }
+    } else {
+      out[(static_cast<size_t>(n) * nq + h) * hd + tid] = from_float<TQ>(l > 0.f ? total / l : 0.f);
+    }
+  }
+}
+
+// out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the spans that the token has, in their order.
+template <typename TQ>
+__global__ __launch_bounds__(kThreads) void attn_generic_join_kernel(
+    const float* __restrict__ part, TQ* __restrict__ out, const int* __restrict__ tokens,
+    const int* __restrict__ positions, int nq, int hd, int window, int max_spans) {
+  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int pos = positions[n];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int spans = min(max_spans, (pos - lo) / kSpan + 1);
+  const float* src = part + (static_cast<size_t>(blockIdx.x) * nq + h) * max_spans * (hd + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < spans; ++s) M = fmaxf(M, src[s * (hd + 2) + hd]);
+  const float m_use = M == -INFINITY ? 0.f : M;
+  if (tid < hd) {
+    float total = 0.f, l = 0.f;
+    for (int s = 0; s < spans; ++s) {
+      const float w = expf(src[s * (hd + 2) + hd] - m_use);
+      total = fmaf(src[s * (hd + 2) + tid], w, total);
+      l = fmaf(src[s * (hd + 2) + hd + 1], w, l);
+    }
     out[(static_cast<size_t>(n) * nq + h) * hd + tid] = from_float<TQ>(l > 0.f ? total / l : 0.f);
   }
 }
 
 }  // namespace
 
+extern "C" int pyre_attn_generic_spans(int max_keys) { return max_keys <= kSpan ? 1 : (max_keys + kSpan - 1) / kSpan; }
+
+// `max_keys`: no token of the launch sees more keys than this (the block tables' width in tokens
+// will do). `part`: scratch of n * nq * pyre_attn_generic_spans(max_keys) * (hd + 2) floats, needed
+// when there is more than one span.
 extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                                  const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                                  const int* seq_of_token, const int* block_table, int table_stride,
                                  int n, int nq, int nkv, int hd, int page_size, float scale,
-                                 int window, hipStream_t stream) {
+                                 int window, int max_keys, float* part, hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(q_dt) && known_dtype(cache_dt), "attn_generic: unknown dtype");
   PYRE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attn_generic: %d query heads do not divide over %d kv heads", nq, nkv);
   PYRE_REQUIRE(hd > 0 && hd <= kMaxHead, "attn_generic: head_dim %d is outside 1..%d", hd, kMaxHead);
   PYRE_REQUIRE(page_size > 0 && table_stride > 0, "attn_generic: bad page geometry");
   PYRE_REQUIRE(nq <= 65535, "attn_generic: too many heads");
+  PYRE_REQUIRE(max_keys > 0, "attn_generic: max_keys=%d", max_keys);
   if (n <= 0) return 0;
+  const int spans = pyre_attn_generic_spans(max_keys);
+  PYRE_REQUIRE(spans <= 65535, "attn_generic: %d keys are too many for one launch", max_keys);
+  PYRE_REQUIRE(spans == 1 || part, "attn_generic: %d spans of keys need scratch memory", spans);
+  float* scratch = spans == 1 ? nullptr : part;
   PYRE_DISPATCH(q_dt, TQ, PYRE_DISPATCH(cache_dt, TC,
-      hipLaunchKernelGGL((attn_generic_kernel<TQ, TC>), dim3(n, nq), dim3(kThreads), 0, stream,
+      hipLaunchKernelGGL((attn_generic_kernel<TQ, TC>), dim3(n, nq, spans), dim3(kThreads), 0, stream,
                          static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),
                          static_cast<const TC*>(v_cache), static_cast<TQ*>(out), tokens, positions,
                          seq_of_token, block_table, table_stride, nq, nkv, hd, page_size, scale,
-                         window)));
+                         window, scratch)));
+  if (spans > 1) {
+    PYRE_DISPATCH(q_dt, TQ,
+        hipLaunchKernelGGL((attn_generic_join_kernel<TQ>), dim3(n, nq), dim3(kThreads), 0, stream, scratch,
+                           static_cast<TQ*>(out), tokens, positions, nq, hd, window, spans));
+  }
   return check_launch("attn_generic");
 }

@@ -65,12 +65,15 @@ int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, floa
 int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
                                int two_i, int K, hipStream_t stream);
 
-// tokens: the n tokens of the flat batch to attend for, or null for tokens 0..n-1.
+// tokens: the n tokens of the flat batch to attend for, or null for tokens 0..n-1. max_keys: a
+// bound on the keys that any of them sees (the block table's width in tokens will do); part:
+// n * nq * pyre_attn_generic_spans(max_keys) * (hd + 2) floats of scratch when that is more than one span.
+int pyre_attn_generic_spans(int max_keys);
 int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                       const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                       const int* seq_of_token, const int* block_table, int table_stride, int n,
-                      int nq, int nkv, int hd, int page_size, float scale, int window,
-                      hipStream_t stream);
+                      int nq, int nkv, int hd, int page_size, float scale, int window, int max_keys,
+                      float* part, hipStream_t stream);
 
 // Prompt portions in true float32 on the matrix cores' float32 instruction: tiles as for
 // pyre_attn_prefill_bf16, float32 queries, caches and output, any head size up to 256, any

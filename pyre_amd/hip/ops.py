@@ -280,10 +280,13 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: t
 def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                  n: int, nq: int, nkv: int, hd: int, page_size: int, scale: float,
-                 window: int = 0, tokens: torch.Tensor | None = None) -> None:
+                 window: int = 0, tokens: torch.Tensor | None = None,
+                 scratch: torch.Tensor | None = None) -> None:
     """Causal attention of n tokens over the paged cache (``tokens``: which of the flat batch,
-    else the first n); see attention_generic.hip."""
-    _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table, tokens)
+    else the first n); see attention_generic.hip. ``scratch``: float32 memory of
+    ``attn_generic_scratch(...)`` elements for the partial results of the spans of keys; without
+    it the memory is allocated here when the block table is wider than one span."""
+    _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table, tokens, scratch)
     if q.dtype != out.dtype or q.numel() < n * nq * hd or out.numel() < n * nq * hd:
         raise KernelError("attn: q/out buffers do not fit")
     if tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
@@ -296,10 +299,50 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_ca
         _i32("tokens", tokens, n)
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
         raise KernelError("attn: block table must be int32 [rows, pages]")
-    call("pyre_attn_generic", q.data_ptr(), out.data_ptr(), dtype_code(q), k_cache.data_ptr(),
-         v_cache.data_ptr(), dtype_code(k_cache), _ptr(tokens), positions.data_ptr(), seq_of_token.data_ptr(),
-         block_table.data_ptr(), block_table.stride(0), n, nq, nkv, hd, page_size, float(scale),
-         int(window), _stream())
+    max_keys = _attn_generic_keys(block_table.shape[1], page_size, window)
+    need = attn_generic_scratch(n, nq, hd, block_table.shape[1], page_size, window)
+    if need and scratch is None:
+        scratch = torch.empty(need, dtype=torch.float32, device=q.device)
+    if need and (scratch.dtype != torch.float32 or not scratch.is_contiguous() or scratch.numel() < need):
+        raise KernelError(f"attn: scratch of {need} float32 elements needed")
+    per_launch = _attn_generic_rows(n, nq, hd, max_keys)
+    flat_q, flat_out = q.view(-1), out.view(-1)
+    for at in range(0, n, per_launch):
+        rows = min(per_launch, n - at)
+        if tokens is not None:  # the list moves on; q, out and positions are indexed by its entries
+            args = (flat_q, flat_out, tokens[at:], positions, seq_of_token)
+        else:
+            args = (flat_q[at * nq * hd:], flat_out[at * nq * hd:], None, positions[at:], seq_of_token[at:])
+        call("pyre_attn_generic", args[0].data_ptr(), args[1].data_ptr(), dtype_code(q), k_cache.data_ptr(),
+             v_cache.data_ptr(), dtype_code(k_cache), _ptr(args[2]), args[3].data_ptr(), args[4].data_ptr(),
+             block_table.data_ptr(), block_table.stride(0), rows, nq, nkv, hd, page_size, float(scale),
+             int(window), max_keys, _ptr(scratch) if need else None, _stream())
+
+
+ATTN_GENERIC_SCRATCH = 1 << 25   #: float32 elements of scratch that one launch of attn_generic may use
+
+
+def _attn_generic_keys(table_width: int, page_size: int, window: int) -> int:
+    """No token sees more keys than its block table holds, or than its window."""
+    keys = max(1, table_width * page_size)
+    return min(keys, window) if window > 0 else keys
+
+
+def _attn_generic_rows(n: int, nq: int, hd: int, max_keys: int) -> int:
+    """Tokens to a launch: all of them, or as many as the scratch of one launch allows."""
+    from pyre_amd.hip.lib import lib
+
+    spans = int(lib().pyre_attn_generic_spans(max_keys))
+    return n if spans <= 1 else max(1, min(n, ATTN_GENERIC_SCRATCH // (nq * spans * (hd + 2))))
+
+
+def attn_generic_scratch(n: int, nq: int, hd: int, table_width: int, page_size: int, window: int = 0) -> int:
+    """Float32 elements of scratch that ``attn_generic`` needs for such a call (0: none)."""
+    from pyre_amd.hip.lib import lib
+
+    max_keys = _attn_generic_keys(table_width, page_size, window)
+    spans = int(lib().pyre_attn_generic_spans(max_keys))
+    return 0 if spans <= 1 or n <= 0 else _attn_generic_rows(n, nq, hd, max_keys) * nq * spans * (hd + 2)
 
 
 def attn_prefill_f32(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,

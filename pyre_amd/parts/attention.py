@@ -142,6 +142,14 @@ class Attention(Mixer):
             singles = ctx.host.arrays["attention.decode_tokens"]
             if len(singles):
                 ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, len(singles),
-                                 *geometry, tokens=ctx.arrays["attention.decode_tokens"])
+                                 *geometry, tokens=ctx.arrays["attention.decode_tokens"],
+                                 scratch=self._spans_scratch(ctx, cache, len(singles)))
         else:
-            ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, n, *geometry)
+            ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, n, *geometry,
+                             scratch=self._spans_scratch(ctx, cache, n))
+
+    def _spans_scratch(self, ctx, cache, n):
+        """Workspace for the partial results of the spans of keys, if the tables are wider than one."""
+        s = self.spec
+        need = ops.attn_generic_scratch(n, s.num_heads, s.head_dim, cache.table.shape[1], cache.page_size, cache.window)
+        return ctx.workspace.get("attn.spans", (need,), torch.float32) if need else None

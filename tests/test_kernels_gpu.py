@@ -335,6 +335,39 @@ def test_attn_generic(dtype, nq, nkv, hd, page, window):
         assert torch.allclose(out[0].double().cpu(), dense[0][1][0].double().repeat_interleave(nq // nkv, 0), atol=tol)
 
 
+@pytest.mark.parametrize("listed", [False, True])
+def test_attn_generic_in_several_launches_and_with_given_scratch(monkeypatch, listed):
+    """Spans of keys leave partial results in scratch memory; a call whose scratch would pass the
+    limit of one launch goes out in several, with the same bits."""
+    ops = _ops()
+    nq, nkv, hd, page, window = 6, 2, 40, 8, 0
+    ctx_lens, q_lens = [700, 1300, 30], [9, 1, 30]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.float32, seed=5)
+    n, scale = q.shape[0], hd ** -0.5
+    some = list(range(0, n, 3)) if listed else None
+    count = len(some) if listed else n
+    tokens = i32(some) if listed else None
+    ref = torch.zeros_like(q)
+    ops.attn_generic(q, ref, kc, vc, pos, seq_of, table, count, nq, nkv, hd, page, scale, window, tokens=tokens)
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    rows = some if listed else list(range(n))
+    assert torch.allclose(ref.double().cpu()[rows], want[rows], atol=2e-5, rtol=2e-5)
+    spans = -(-table.shape[1] * page // 512)
+    assert spans > 1
+    monkeypatch.setattr(ops, "ATTN_GENERIC_SCRATCH", 7 * nq * spans * (hd + 2))   # seven tokens a launch
+    need = ops.attn_generic_scratch(count, nq, hd, table.shape[1], page, window)
+    assert need == 7 * nq * spans * (hd + 2)
+    out = torch.zeros_like(q)
+    scratch = torch.full((need + 3,), float("nan"), device=DEV)
+    ops.attn_generic(q, out, kc, vc, pos, seq_of, table, count, nq, nkv, hd, page, scale, window, tokens=tokens,
+                     scratch=scratch)
+    assert torch.equal(out, ref)
+    assert torch.isnan(scratch[need:]).all()
+    with pytest.raises(Exception, match="scratch"):
+        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, count, nq, nkv, hd, page, scale, window, tokens=tokens,
+                         scratch=scratch[:need - 1])
+
+
 MFMA_SHAPES = [(28, 4, 128, 16), (8, 8, 64, 16), (6, 1, 32, 32), (40, 2, 96, 16), (3, 1, 256, 48), (4, 2, 64, 48)]
 
 
