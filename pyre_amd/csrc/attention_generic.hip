@@ -29,7 +29,19 @@ constexpr int kThreads = 256;
 constexpr int kSpan = 512;     // keys that one block takes, and whose scores are held in LDS
 constexpr int kMaxHead = 256;
 
-template <typename TQ, typename TC>
+// Four consecutive elements as one load; p is aligned to four elements.
+template <typename T>
+__device__ inline void load4(const T* p, float (&v)[4]) {
+  struct __attribute__((aligned(4 * sizeof(T)))) Quad { T e[4]; };
+  const Quad q = *reinterpret_cast<const Quad*>(p);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) v[u] = to_float(q.e[u]);
+}
+
+// VEC: head size and page size are multiples of four and the caches start on 16 bytes, so
+// that keys are read four elements and values four keys at a time. The sums of a score run
+// over the elements in their order either way.
+template <typename TQ, typename TC, bool VEC>
 __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
     TQ* __restrict__ out, const int* __restrict__ tokens, const int* __restrict__ positions,
@@ -68,7 +80,16 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
       if (page >= 0) {
         const TC* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * hd;
         s = 0.f;
-        for (int e = 0; e < hd; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+        if (VEC) {
+          for (int e = 0; e < hd; e += 4) {
+            float kv[4];
+            load4(kp + e, kv);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s = fmaf(qs[e + u], kv[u], s);
+          }
+        } else {
+          for (int e = 0; e < hd; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+        }
         s *= scale;
       }
       sc[j] = s;
@@ -83,7 +104,18 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
       lsum += p;
     }
     l = block_sum(lsum, scratch);  // block_sum's barriers publish sc[]
-    if (active) {
+    if (active && VEC) {  // groups of four keys that lie side by side in a page
+      for (int quad = base / 4 + g; quad <= (base + cnt - 1) / 4; quad += groups) {
+        const int key = 4 * quad;
+        const int page = table[key / page_size], off = key % page_size;
+        if (page < 0) continue;
+        float vv[4];
+        load4(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off, vv);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (key + u >= base && key + u < base + cnt) acc = fmaf(sc[key + u - base], vv[u], acc);
+      }
+    } else if (active) {
       for (int j = g; j < cnt; j += groups) {
         const int key = base + j;
         const int page = table[key / page_size], off = key % page_size;
@@ -159,12 +191,21 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
   PYRE_REQUIRE(spans <= 65535, "attn_generic: %d keys are too many for one launch", max_keys);
   PYRE_REQUIRE(spans == 1 || part, "attn_generic: %d spans of keys need scratch memory", spans);
   float* scratch = spans == 1 ? nullptr : part;
-  PYRE_DISPATCH(q_dt, TQ, PYRE_DISPATCH(cache_dt, TC,
-      hipLaunchKernelGGL((attn_generic_kernel<TQ, TC>), dim3(n, nq, spans), dim3(kThreads), 0, stream,
-                         static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),
-                         static_cast<const TC*>(v_cache), static_cast<TQ*>(out), tokens, positions,
-                         seq_of_token, block_table, table_stride, nq, nkv, hd, page_size, scale,
-                         window, scratch)));
+  const bool vec = hd % 4 == 0 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+#define PYRE_LAUNCH_GENERIC(VEC)                                                                          \
+  PYRE_DISPATCH(q_dt, TQ, PYRE_DISPATCH(cache_dt, TC,                                                     \
+      hipLaunchKernelGGL((attn_generic_kernel<TQ, TC, VEC>), dim3(n, nq, spans), dim3(kThreads), 0, stream, \
+                         static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),                      \
+                         static_cast<const TC*>(v_cache), static_cast<TQ*>(out), tokens, positions,       \
+                         seq_of_token, block_table, table_stride, nq, nkv, hd, page_size, scale,          \
+                         window, scratch)))
+  if (vec) {
+    PYRE_LAUNCH_GENERIC(true);
+  } else {
+    PYRE_LAUNCH_GENERIC(false);
+  }
+#undef PYRE_LAUNCH_GENERIC
   if (spans > 1) {
     PYRE_DISPATCH(q_dt, TQ,
         hipLaunchKernelGGL((attn_generic_join_kernel<TQ>), dim3(n, nq), dim3(kThreads), 0, stream, scratch,

@@ -144,6 +144,137 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_f32_mfma_kernel(
   }
 }
 
+// The same product for a decode step's few rows (M <= 8), as a stream over the weights. A block
+// is one wave with 32 output columns, so there is no barrier. It has a ring of R slots in LDS, a
+// slot being 32 k (two stages) of its 32 rows of W (4 KB) and of the rows of A (1 KB), filled by
+// loads that go from memory straight into LDS: while slot j is multiplied, slot j + 1 is read
+// from LDS into registers and the R - 2 after it are on their way. A load instruction takes
+// whole 128-byte lines (8 rows x 32 k); the 16-byte pieces of a row are exchanged among
+// themselves by the row's number so that the matrix instruction's operand reads (a lane's row,
+// eight k of a stage) spread over the banks. Stages, steps and parts of k are those of the
+// kernel above: the sums are the same bit for bit. With one row in 32 columns of the matrix
+// instruction the chain of dependent instructions of a wave, not memory, sets the pace (a slot
+// of 4 KB in about 0.6 us); a small ring lets eight blocks share a compute unit.
+constexpr int kStreamRows = 8;
+constexpr int kSlotK = 32;
+constexpr int kSlotBytes = 5 * 1024;
+
+__device__ inline void load_to_lds(const void* src, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
+}
+template <int N>
+__device__ inline void wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 0u, 0u};
+
+template <int R>
+__global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
+    const float* __restrict__ A, size_t lda, const float* __restrict__ W, size_t ldw,
+    const void* __restrict__ bias, int bias_dt, float* __restrict__ out, size_t ldo, size_t part_stride, int M,
+    int N, int K, int kper) {
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[R * kSlotBytes];
+  const int lane = threadIdx.x, half = lane >> 5, c = lane & 31;
+  const int n0 = blockIdx.x * 32;
+  const int kbeg = blockIdx.z * kper;
+  K = min(K, kbeg + kper);  // this part's end
+  out += blockIdx.z * part_stride;
+  if (blockIdx.z) bias = nullptr;  // the bias belongs to one part only
+  const int slots = (K - kbeg + kSlotK - 1) / kSlotK;
+
+  // This lane's share of a slot's five loads: of load i, the piece that lands at row 8 i + lane / 8,
+  // place lane % 8, which is piece (place ^ swizzle of the row) of the row's 32 k. Columns past
+  // the end read the last one's weights and are not stored.
+  const int lr = lane >> 3, lp = lane & 7;
+  const float* wsrc[4];
+  int wk[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 8 * i + lr;
+    wk[i] = 4 * (lp ^ ((r >> 1) & 7));
+    wsrc[i] = W + static_cast<size_t>(min(n0 + r, N - 1)) * ldw + kbeg + wk[i];
+  }
+  const float* xsrc = A + static_cast<size_t>(lr < M ? lr : 0) * lda + kbeg + 4 * lp;
+  const unsigned mine = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(ring)));
+  const float* zero = reinterpret_cast<const float*>(kZeroPiece);
+
+  int fill = 0;  // ring position of the next slot to load
+  auto issue = [&](int j) {
+    const unsigned dst = mine + fill * kSlotBytes;
+    fill = fill + 1 == R ? 0 : fill + 1;
+    const int k0 = kSlotK * j, left = j < slots ? K - kbeg - k0 : 0;  // k of this part from the slot's start on
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_to_lds(wk[i] < left ? wsrc[i] + k0 : zero, dst + 1024 * i);
+    load_to_lds(lr < M && 4 * lp < left ? xsrc + k0 : zero, dst + 4096);
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  const unsigned char* wpiece = ring + c * 128;
+  const unsigned char* xpiece = ring + 4096 + (c & 7) * 128;
+  const int swz = (c >> 1) & 7;
+  const bool has_x = c < M;
+  int at = 0;  // ring position of the next slot to read
+  auto read = [&](f32x4 (&a)[2][2], f32x4 (&b)[2][2]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int piece = 4 * t + 2 * half + h;
+        a[t][h] = *reinterpret_cast<const f32x4*>(wpiece + at * kSlotBytes + 16 * (piece ^ swz));
+        b[t][h] = *reinterpret_cast<const f32x4*>(xpiece + at * kSlotBytes + 16 * piece);
+        if (!has_x) b[t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+    at = at + 1 == R ? 0 : at + 1;
+  };
+
+  // Slot j + 1 is read from LDS while slot j is multiplied, so of the R slots of the ring one is
+  // in registers, one being read and R - 2 on their way.
+#pragma unroll
+  for (int j = 0; j < R - 1; ++j) issue(j);
+  f32x4 a[2][2], b[2][2], an[2][2], bn[2][2];
+  wait_loads<5 * (R - 2)>();  // loads finish in the order of issue: slot 0 is there
+  read(a, b);
+  for (int j = 0; j < slots; ++j) {
+    issue(j + R - 1);            // into the position of slot j - 1, read a turn ago
+    wait_loads<5 * (R - 2)>();   // slot j + 1 is there
+    read(an, bn);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (kSlotK * j + BK * t >= K - kbeg) break;  // a part that ends with half a slot
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s >> 2][s & 3], b[t][s >> 2][s & 3], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) a[t][h] = an[t][h], b[t][h] = bn[t][h];
+  }
+  wait_loads<0>();  // the loads past the end
+
+  // acc[4 i + j]: output column n = tile row 8 i + 4 half + j, output row m = tile column c.
+  if (c >= M) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + 8 * i + 4 * half;
+    if (n >= N) continue;
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = acc[4 * i + j];
+      if (bias && n + j < N) v[j] += load_as_float(bias, bias_dt, n + j);
+    }
+    float* dst = out + static_cast<size_t>(c) * ldo + n;
+    if (n + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+      *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+    } else {
+      for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = v[j];
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw, const void* bias, int bias_dt,
@@ -160,7 +291,12 @@ extern "C" int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw,
   // 16-byte loads along k need rows that start on 16 bytes
   const int vec_ok = lda % 4 == 0 && ldw % 4 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(W) % 16 == 0;
-  if (M <= 32) {  // a decode step's few rows: four waves side by side along n
+  if (M <= kStreamRows && vec_ok && K % 4 == 0) {  // a decode step's few rows: the weights as a stream
+    const dim3 grid((N + 31) / 32, 1, ksplit);
+    hipLaunchKernelGGL((gemm_f32_stream_kernel<4>), grid, dim3(64), 0, stream, A, static_cast<size_t>(lda), W,
+                       static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),
+                       static_cast<size_t>(part_stride), M, N, K, kper);
+  } else if (M <= 32) {  // four waves side by side along n
     const dim3 grid((N + 127) / 128, (M + 31) / 32, ksplit);
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<4, 1, 1, 1>), grid, dim3(256), 0, stream, A, static_cast<size_t>(lda), W,
                        static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),

@@ -314,7 +314,7 @@ def attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window=0):
     return torch.cat(outs)
 
 
-GENERIC_SHAPES = [(4, 2, 16, 16), (8, 2, 12, 8), (6, 6, 40, 4), (28, 4, 128, 16), (5, 1, 256, 32)]
+GENERIC_SHAPES = [(4, 2, 16, 16), (8, 2, 12, 8), (4, 2, 10, 6), (3, 1, 20, 5), (6, 6, 40, 4), (28, 4, 128, 16), (5, 1, 256, 32)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
