@@ -10,7 +10,7 @@
 // A token at position `pos` sees the keys lo..pos of its request, all read from
 // the cache (this step's keys were written before the call), so prompt portions
 // and single decoded tokens are the same case. lo = max(0, pos - window + 1) for
-// a window, else 0. The keys of a token are taken in spans of 512, one block each (grid.z),
+// a window, else 0. The keys of a token are taken in spans of 128, one block each (grid.z),
 // whose partial results (max, sum, unnormalised output) a second kernel joins in the order of
 // the spans; a launch whose block tables hold no more than one span writes the result
 // directly. The order of every sum depends on (lo, pos) alone, so the result for a position
@@ -26,7 +26,7 @@ using namespace pyre;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kSpan = 512;     // keys that one block takes, and whose scores are held in LDS
+constexpr int kSpan = 128;     // keys that one block takes, and whose scores are held in LDS
 constexpr int kMaxHead = 256;
 
 // Four consecutive elements as one load; p is aligned to four elements.
@@ -81,6 +81,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
         const TC* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * hd;
         s = 0.f;
         if (VEC) {
+#pragma unroll 8
           for (int e = 0; e < hd; e += 4) {
             float kv[4];
             load4(kp + e, kv);
@@ -105,6 +106,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
     }
     l = block_sum(lsum, scratch);  // block_sum's barriers publish sc[]
     if (active && VEC) {  // groups of four keys that lie side by side in a page
+#pragma unroll 4
       for (int quad = base / 4 + g; quad <= (base + cnt - 1) / 4; quad += groups) {
         const int key = 4 * quad;
         const int page = table[key / page_size], off = key % page_size;
@@ -154,11 +156,14 @@ __global__ __launch_bounds__(kThreads) void attn_generic_join_kernel(
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int spans = min(max_spans, (pos - lo) / kSpan + 1);
   const float* src = part + (static_cast<size_t>(blockIdx.x) * nq + h) * max_spans * (hd + 2);
-  float M = -INFINITY;
-  for (int s = 0; s < spans; ++s) M = fmaxf(M, src[s * (hd + 2) + hd]);
+  __shared__ float scratch[16];
+  float mine = -INFINITY;
+  for (int s = tid; s < spans; s += kThreads) mine = fmaxf(mine, src[s * (hd + 2) + hd]);
+  const float M = block_max(mine, scratch);
   const float m_use = M == -INFINITY ? 0.f : M;
   if (tid < hd) {
     float total = 0.f, l = 0.f;
+#pragma unroll 8
     for (int s = 0; s < spans; ++s) {
       const float w = expf(src[s * (hd + 2) + hd] - m_use);
       total = fmaf(src[s * (hd + 2) + tid], w, total);

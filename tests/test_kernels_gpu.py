@@ -352,7 +352,9 @@ def test_attn_generic_in_several_launches_and_with_given_scratch(monkeypatch, li
     want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
     rows = some if listed else list(range(n))
     assert torch.allclose(ref.double().cpu()[rows], want[rows], atol=2e-5, rtol=2e-5)
-    spans = -(-table.shape[1] * page // 512)
+    from pyre_amd.hip.lib import lib
+
+    spans = lib().pyre_attn_generic_spans(table.shape[1] * page)
     assert spans > 1
     monkeypatch.setattr(ops, "ATTN_GENERIC_SCRATCH", 7 * nq * spans * (hd + 2))   # seven tokens a launch
     need = ops.attn_generic_scratch(count, nq, hd, table.shape[1], page, window)
