@@ -145,8 +145,7 @@ __global__ void rope_kv_write_kernel(const void* __restrict__ qkv, int qkv_dt, i
         const float x1 = value(base + ia), x2 = value(base + ib);
         const float c = cos_t[static_cast<size_t>(pos) * half + j];
         const float s = sin_t[static_cast<size_t>(pos) * half + j];
-        a = x1 * c - x2 * s;
-        b = x2 * c + x1 * s;
+        rotate_pair(x1, x2, c, s, a, b);
       } else {
         ia = rotary_dim + (j - half);
         a = value(base + ia);

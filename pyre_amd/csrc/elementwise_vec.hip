@@ -156,8 +156,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
     const float4 x1 = value4(base + j), x2 = value4(base + j + half);
     const size_t t = static_cast<size_t>(positions[n]) * half + j;
     const float4 c = Vec4<float>::load(cos_t + t), s = Vec4<float>::load(sin_t + t);
-    const float4 a{x1.x * c.x - x2.x * s.x, x1.y * c.y - x2.y * s.y, x1.z * c.z - x2.z * s.z, x1.w * c.w - x2.w * s.w};
-    const float4 b{x2.x * c.x + x1.x * s.x, x2.y * c.y + x1.y * s.y, x2.z * c.z + x1.z * s.z, x2.w * c.w + x1.w * s.w};
+    float4 a, b;
+    rotate_pair(x1.x, x2.x, c.x, s.x, a.x, b.x);
+    rotate_pair(x1.y, x2.y, c.y, s.y, a.y, b.y);
+    rotate_pair(x1.z, x2.z, c.z, s.z, a.z, b.z);
+    rotate_pair(x1.w, x2.w, c.w, s.w, a.w, b.w);
     TC* dst = head < nq ? q_out + static_cast<size_t>(n) * nq * hd + base
                         : k_cache + ((static_cast<size_t>(page) * nkv + (head - nq)) * page_size + off) * hd;
     Vec4<TC>::store(dst + j, a);

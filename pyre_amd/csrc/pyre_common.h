@@ -50,6 +50,13 @@ __host__ __device__ inline uint16_t bf16_bits(float f) {
   return static_cast<uint16_t>(x.u >> 16);
 }
 
+// One rotary pair turned by the angle with cosine c and sine s (pyre/model.py:54-63), with
+// explicit fused multiply-adds: the same roundings in every kernel that rotates.
+__device__ inline void rotate_pair(float x1, float x2, float c, float s, float& a, float& b) {
+  a = fmaf(x1, c, -(x2 * s));
+  b = fmaf(x2, c, x1 * s);
+}
+
 template <typename T> __host__ __device__ inline T from_float(float v);
 template <> __host__ __device__ inline float from_float<float>(float v) { return v; }
 template <> __host__ __device__ inline bf16 from_float<bf16>(float v) {
