@@ -65,6 +65,13 @@ int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, long ldw, floa
 int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
                                int two_i, int K, hipStream_t stream);
 
+// The first of them for up to 256 rows (a decode step of many requests), for products with few
+// output columns: a block keeps all rows of X against 64 rows of W, and ksplit blocks share
+// them. out: float32 [ksplit][M][N].
+int pyre_gemm_mid_supports(int M, int N, int K, long ldx, long ldw);
+int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N, int K,
+                       int ksplit, hipStream_t stream);
+
 // tokens: the n tokens of the flat batch to attend for, or null for tokens 0..n-1. max_keys: a
 // bound on the keys that any of them sees (the block table's width in tokens will do); part:
 // n * nq * pyre_attn_generic_spans(max_keys) * (hd + 2) floats of scratch when that is more than one span.

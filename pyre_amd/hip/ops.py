@@ -537,6 +537,22 @@ def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.T
          out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
 
 
+def gemm_mid_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
+    from pyre_amd.hip.lib import lib
+
+    return bool(lib().pyre_gemm_mid_supports(m, n, k, ldx, ldw))
+
+
+def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int) -> None:
+    """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 256."""
+    _skinny_common(x, w, m)
+    n = w.shape[0]
+    if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() < ksplit * m * n or not out.is_cuda:
+        raise KernelError("gemm_mid: out must be contiguous float32 [ksplit, m, N] on the GPU")
+    call("pyre_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), m, n,
+         w.shape[1], ksplit, _stream())
+
+
 def read_bandwidth(device: str = "cuda:0", gib: float = 2.0, blocks: int = 4096, repeats: int = 10) -> float:
     """Measured streaming-read bandwidth in GB/s (a buffer larger than every cache)."""
     import time

@@ -20,6 +20,9 @@ SKINNY_MAX_ROWS = 64
 SKINNY_MAX_KSPLIT = 12
 #: up to this many rows the gate/up product and the SiLU-gate are one kernel
 FUSED_SILU_MAX_ROWS = 64
+#: most rows of the kernel between the two, which keeps a step's rows against 64 rows of the weights
+MID_MAX_ROWS = 256
+MID_MAX_KSPLIT = 12
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
@@ -47,6 +50,20 @@ def skinny_ksplit(m: int, n_out: int, k: int) -> int:
         if best_cost is None or cost < best_cost - 1e-9:
             best, best_cost = ks, cost
     return best
+
+
+def mid_ksplit(n_out: int, k: int) -> int:
+    """Into how many parts of k the kernel for 65 to 256 rows splits a product, or 0 if it is not
+    the one to take. A block has 64 rows of the weights; the kernel is at its best when the blocks
+    of all parts fill the 256 compute units in one round, and beats the BLAS library where that
+    takes at least two parts of 256 k or more (measured on the 1.5B, 7B and 32B shapes: q/k/v, the
+    attention output and the feed-forward's way down take 9 to 20 us where the library takes 19
+    to 31, and 60 against 100 at 7B's way down; the wide gate/up product stays with the library)."""
+    blocks = -(-n_out // 64)
+    ks = min(256 // blocks, k // 256, MID_MAX_KSPLIT)
+    while ks > 1 and (ks - 1) * (-(-(-(-k // ks)) // 32) * 32) >= k:
+        ks -= 1  # would leave a part empty
+    return ks if ks >= 2 else 0
 
 
 #: products whose library result is kept in float32 instead of being rounded to 16 bits:
@@ -82,6 +99,12 @@ def linear(lin, ctx, x, n, out):
         buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
         ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
         return Partials(buf, lin.bias)
+    if out is None and SKINNY_MAX_ROWS < n <= MID_MAX_ROWS and rt.options.get("mid_gemm", True):
+        ks = mid_ksplit(n_out, k)
+        if ks and ops.gemm_mid_supports(n, n_out, k, x.stride(0), lin.weight.stride(0)):
+            buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
+            ops.gemm_mid_bf16(x, lin.weight, buf, n, ks)
+            return Partials(buf, lin.bias)
     if not library:
         return None
     if out is not None:

@@ -804,6 +804,42 @@ def test_gemm_skinny(m, n, k, ksplit):
     assert torch.allclose(out.double().sum(0), want, atol=1e-3 * math.sqrt(k), rtol=1e-4)
 
 
+@pytest.mark.parametrize("m", [1, 65, 100, 128, 129, 200, 256])
+@pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (1536, 1536, 6), (1000, 136, 2), (131, 8, 1), (3584, 18944, 4),
+                                        (2048, 1000, 3), (70, 4096, 12)])
+def test_gemm_mid(m, n, k, ksplit):
+    """The products of a decode step of 65 to 256 rows: sizes that are no multiple of the tiles
+    (64 rows of the weights, 32 of the input, stages of 32 k), k in parts; and a row's result is
+    bit for bit the same whatever rows share the step and however many they are."""
+    ops = _ops()
+    assert ops.gemm_mid_supports(m, n, k, k, k)
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd(n, k, dtype=torch.bfloat16, seed=2)
+    out = torch.full((ksplit, m, n), float("nan"), device=DEV)
+    ops.gemm_mid_bf16(x, w, out, m, ksplit)
+    want = x.double() @ w.double().T
+    assert torch.allclose(out.double().sum(0), want, atol=1e-3 * math.sqrt(k), rtol=1e-4)
+    rows = sorted({0, m // 2, m - 1})
+    few = torch.full((ksplit, len(rows), n), float("nan"), device=DEV)
+    ops.gemm_mid_bf16(x[rows].contiguous(), w, few, len(rows), ksplit)
+    assert torch.equal(few, out[:, rows])
+    wide = torch.zeros(m, k + 16, dtype=torch.bfloat16, device=DEV)      # rows that are further apart
+    wide[:, 8:k + 8] = x
+    again = torch.full_like(out, float("nan"))
+    ops.gemm_mid_bf16(wide[:, 8:k + 8], w, again, m, ksplit)
+    assert torch.equal(again, out)
+
+
+def test_gemm_mid_refuses_what_it_cannot_take():
+    ops = _ops()
+    x, w = rnd(300, 64, dtype=torch.bfloat16), rnd(48, 64, dtype=torch.bfloat16)
+    assert not ops.gemm_mid_supports(300, 48, 64, 64, 64) and not ops.gemm_mid_supports(100, 48, 60, 60, 60)
+    with pytest.raises(Exception, match="not supported"):
+        ops.gemm_mid_bf16(x, w, torch.empty(1, 300, 48, device=DEV), 300, 1)
+    with pytest.raises(Exception, match="empty"):
+        ops.gemm_mid_bf16(x[:100], w, torch.empty(3, 100, 48, device=DEV), 100, 3)
+
+
 @pytest.mark.parametrize("m", [1, 8, 40])
 @pytest.mark.parametrize("inter,k", [(176, 64), (18944, 3584), (250, 96)])
 def test_gemm_skinny_silu(m, inter, k):

@@ -178,3 +178,20 @@ def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():
         assert "grow" in str(e)
     else:
         raise AssertionError("a frozen workspace must not grow")
+
+
+def test_mid_ksplit_fills_one_round_and_leaves_no_part_empty():
+    """The kernel for 65 to 256 rows is chosen where at least two parts of 256 k or more fill the
+    256 compute units in one round of blocks of 64 output columns."""
+    from pyre_amd.parts.fast import MID_MAX_KSPLIT, mid_ksplit
+
+    assert mid_ksplit(1536, 8960) == 10 and mid_ksplit(3584, 18944) == 4 and mid_ksplit(4608, 3584) == 3
+    assert mid_ksplit(37888, 3584) == 0 and mid_ksplit(17920, 1536) == 0 and mid_ksplit(152064, 3584) == 0
+    assert mid_ksplit(96, 64) == 0 and mid_ksplit(64, 500) == 0
+    for n_out in (1, 64, 65, 700, 2048, 8192, 9000):
+        for k in (8, 256, 511, 512, 1000, 4096, 20000):
+            ks = mid_ksplit(n_out, k)
+            if ks:
+                blocks = -(-n_out // 64)
+                kper = -(-(-(-k // ks)) // 32) * 32
+                assert 2 <= ks <= MID_MAX_KSPLIT and blocks * ks <= 256 and k // ks >= 256 and (ks - 1) * kper < k
