@@ -33,7 +33,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int BN = 64;   // rows of W per block
-constexpr int BK = 32;   // k per stage: rows of 64 bytes
+constexpr int BK = 64;   // k per stage: rows of 128 bytes
 
 // 16 bytes per lane from global memory straight into LDS: lane x's piece lands at
 // lds_addr + 16 x. The compiler does not know of these loads; whoever reads the bytes
@@ -47,75 +47,71 @@ __device__ inline void wait_loads() {
 }
 __device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 0u, 0u};
 
-// SW, SX: stages in the rings of W and of X. The weights come from memory (about 2 us away), the
-// rows of X from L2 (well under 1 us): W is loaded by a fifth wave of its own, whose loads
-// can then run far ahead without holding up the others' (a wave's loads finish in order).
-template <int CW, int SW, int SX>
-__global__ __launch_bounds__(320, 2) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
-                                                          const bf16* __restrict__ W, size_t ldw,
-                                                          float* __restrict__ out, int M, int N, int K, int kper) {
-  constexpr int BM = 128 * CW, WSTAGE = BN * 64, XSTAGE = BM * 64;
-  constexpr int PERW = BN / 16;      // loads of 16 rows per stage of W, all by the loading wave
-  constexpr int PERX = BM / 16 / 4;  // and of X, per multiplying wave
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[SW * WSTAGE + SX * XSTAGE];
+#ifndef PYRE_MID_NL2
+#define PYRE_MID_NL2 10
+#define PYRE_MID_NL1 6
+#endif
+constexpr int kLoaders2 = PYRE_MID_NL2, kLoaders1 = PYRE_MID_NL1;  // loading waves for 256 and for 128 rows of X
+
+// NL loading waves beside the four that multiply, S stages in the ring. What a wave can have
+// loaded per microsecond is limited (about 9 GB/s from L2, whatever the pattern and however many
+// loads it has on their way), so the loads of a stage are dealt to several waves that do
+// nothing else; a stage is the 64 rows of W, then the BM rows of X.
+template <int CW, int NL, int S>
+__global__ __launch_bounds__(256 + 64 * NL) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
+                                                                 const bf16* __restrict__ W, size_t ldw,
+                                                                 float* __restrict__ out, int M, int N, int K,
+                                                                 int kper) {
+  constexpr int BM = 128 * CW, ROWS = BN + BM, STAGE = ROWS * 128;
+  constexpr int PER = ROWS / 8 / NL;  // loads of 8 rows per loading wave and stage
+  static_assert(ROWS / 8 % NL == 0, "the loads of a stage divide evenly over the loading waves");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[S * STAGE];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int c = lane & 31, half = lane >> 5;
   const int ks = blockIdx.y, kbeg = ks * kper, kend = min(K, kbeg + kper);
   const int stages = (kend - kbeg + BK - 1) / BK;
-  const unsigned lds_base = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds)));
-  const bf16* zero = reinterpret_cast<const bf16*>(kZeroPiece);
-  // A load of 16 rows: the piece that lands at row lane / 4 of them, place lane % 4, is piece
-  // (place ^ swizzle of the row) of the row's 32 k. Rows past the end are zeros.
-  const int place_row = lane >> 2;
 
-  if (wave == 4) {
-    // ---- the loading wave: 64 rows of W per stage.
-    const bf16* src[PERW];
-    int kofs[PERW];
+  if (wave >= 4) {
+    // ---- a loading wave: of load j = l + NL i (rows 8 j .. 8 j + 7 of the stage) this lane
+    // brings the piece that lands at row 8 j + lane / 8, place lane % 8, which is piece
+    // (place ^ swizzle of the row) of the row's 64 k. Rows past the end are zeros.
+    const int l = wave - 4;
+    const unsigned lds_base = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds)));
+    const bf16* zero = reinterpret_cast<const bf16*>(kZeroPiece);
+    const bf16* src[PER];
+    int kofs[PER];
 #pragma unroll
-    for (int i = 0; i < PERW; ++i) {
-      const int row = 16 * i + place_row;
-      kofs[i] = 8 * ((lane & 3) ^ ((row >> 2) & 3));
-      const int n = blockIdx.x * BN + row;
-      src[i] = n < N ? W + static_cast<size_t>(n) * ldw + kbeg + kofs[i] : nullptr;
+    for (int i = 0; i < PER; ++i) {
+      const int row = 8 * (l + NL * i) + (lane >> 3);
+      kofs[i] = 8 * ((lane & 7) ^ ((row >> 1) & 7));
+      const bf16* base = nullptr;
+      if (row < BN) {
+        if (blockIdx.x * BN + row < N) base = W + static_cast<size_t>(blockIdx.x * BN + row) * ldw;
+      } else if (row - BN < M) {
+        base = X + static_cast<size_t>(row - BN) * ldx;
+      }
+      src[i] = base ? base + kbeg + kofs[i] : nullptr;
     }
     auto issue = [&](int st, int slot) {
       const int left = st < stages ? kend - kbeg - BK * st : 0;  // k of this part from the stage's start on
 #pragma unroll
-      for (int i = 0; i < PERW; ++i)
-        load_to_lds(src[i] && kofs[i] < left ? src[i] + BK * st : zero, lds_base + slot * WSTAGE + i * 1024);
+      for (int i = 0; i < PER; ++i)
+        load_to_lds(src[i] && kofs[i] < left ? src[i] + BK * st : zero, lds_base + slot * STAGE + (l + NL * i) * 1024);
     };
 #pragma unroll
-    for (int st = 0; st < SW - 1; ++st) issue(st, st);
+    for (int st = 0; st < S - 1; ++st) issue(st, st);
     int slot = 0;
     for (int st = 0; st < stages; ++st) {
-      wait_loads<PERW * (SW - 2)>();  // loads finish in the order of issue: stage st is there
-      __syncthreads();                // the others know, and have multiplied stage st - 1
-      issue(st + SW - 1, slot == 0 ? SW - 1 : slot - 1);
-      slot = slot + 1 == SW ? 0 : slot + 1;
+      wait_loads<PER * (S - 2)>();  // loads finish in the order of issue: this wave's share of stage st is there
+      __syncthreads();              // everyone knows, and stage st - 1 has been multiplied
+      issue(st + S - 1, slot == 0 ? S - 1 : slot - 1);
+      slot = slot + 1 == S ? 0 : slot + 1;
     }
     wait_loads<0>();  // the loads past the end
     return;
   }
 
-  // ---- the multiplying waves: wave w loads a quarter of the rows of X and multiplies its own
-  // 32 CW rows of them against the block's 64 rows of W.
-  const bf16* src[PERX];
-  int kofs[PERX];
-#pragma unroll
-  for (int i = 0; i < PERX; ++i) {
-    const int row = 16 * (wave + 4 * i) + place_row;
-    kofs[i] = 8 * ((lane & 3) ^ ((row >> 2) & 3));
-    src[i] = row < M ? X + static_cast<size_t>(row) * ldx + kbeg + kofs[i] : nullptr;
-  }
-  const unsigned x_base = lds_base + SW * WSTAGE;
-  auto issue = [&](int st, int slot) {
-    const int left = st < stages ? kend - kbeg - BK * st : 0;
-#pragma unroll
-    for (int i = 0; i < PERX; ++i)
-      load_to_lds(src[i] && kofs[i] < left ? src[i] + BK * st : zero, x_base + slot * XSTAGE + (wave + 4 * i) * 1024);
-  };
-
+  // ---- a multiplying wave: its own 32 CW rows of X against the block's 64 rows of W.
   f32x16 acc[2][CW];
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt)
@@ -124,35 +120,37 @@ __global__ __launch_bounds__(320, 2) void gemm_mid_kernel(const bf16* __restrict
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[rt][ct][i] = 0.f;
 
-  const int swz = (c >> 2) & 3;
-  const int xrow0 = 32 * CW * wave + c;  // this lane's row of X, for tile 0
-#pragma unroll
-  for (int st = 0; st < SX - 1; ++st) issue(st, st);
-  int wslot = 0, xslot = 0;
+  const int swz = (c >> 1) & 7;
+  const int xrow0 = BN + 32 * CW * wave + c;  // this lane's row of X in the stage, for tile 0
+  int slot = 0;
   for (int st = 0; st < stages; ++st) {
-    wait_loads<PERX * (SX - 2)>();  // this wave's share of stage st of X is there
-    __syncthreads();                // and everyone's, and stage st of W; and everyone has multiplied stage st - 1
-    issue(st + SX - 1, xslot == 0 ? SX - 1 : xslot - 1);
-    const unsigned char* wb = lds + wslot * WSTAGE;
-    const unsigned char* xb = lds + SW * WSTAGE + xslot * XSTAGE;
+    __syncthreads();  // stage st is there; and everyone has multiplied stage st - 1
+    const unsigned char* sb = lds + slot * STAGE;
+    // The operands of step kk + 1 are read from LDS while step kk is multiplied.
+    bf16x8 a[2], b[CW], an[2], bn[CW];
+    auto read = [&](int kk, bf16x8 (&ra)[2], bf16x8 (&rb)[CW]) {
+      const int piece = 16 * ((2 * kk + half) ^ swz);
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) ra[rt] = *reinterpret_cast<const bf16x8*>(sb + (32 * rt + c) * 128 + piece);
+#pragma unroll
+      for (int ct = 0; ct < CW; ++ct) rb[ct] = *reinterpret_cast<const bf16x8*>(sb + (xrow0 + 32 * ct) * 128 + piece);
+    };
+    read(0, a, b);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
-      const int piece = 16 * ((2 * kk + half) ^ swz);
-      bf16x8 a[2], b[CW];
-#pragma unroll
-      for (int rt = 0; rt < 2; ++rt) a[rt] = *reinterpret_cast<const bf16x8*>(wb + (32 * rt + c) * 64 + piece);
-#pragma unroll
-      for (int ct = 0; ct < CW; ++ct) b[ct] = *reinterpret_cast<const bf16x8*>(xb + (xrow0 + 32 * ct) * 64 + piece);
+      if (kk + 1 < BK / 16) read(kk + 1, an, bn);
 #pragma unroll
       for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
         for (int ct = 0; ct < CW; ++ct)
           acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[rt], b[ct], acc[rt][ct], 0, 0, 0);
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) a[rt] = an[rt];
+#pragma unroll
+      for (int ct = 0; ct < CW; ++ct) b[ct] = bn[ct];
     }
-    wslot = wslot + 1 == SW ? 0 : wslot + 1;
-    xslot = xslot + 1 == SX ? 0 : xslot + 1;
+    slot = slot + 1 == S ? 0 : slot + 1;
   }
-  wait_loads<0>();  // the loads past the end
 
   // acc[rt][ct][4 q + j]: row 32 rt + 8 q + 4 half + j of the block's tile of W, row
   // 32 (CW wave + ct) + c of X.
@@ -205,10 +203,10 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
   if (M > 128) {
-    hipLaunchKernelGGL((gemm_mid_kernel<2, 7, 3>), grid, dim3(320), 0, stream, x, static_cast<size_t>(ldx), w,
+    hipLaunchKernelGGL((gemm_mid_kernel<2, kLoaders2, 3>), grid, dim3(256 + 64 * kLoaders2), 0, stream, x, static_cast<size_t>(ldx), w,
                        static_cast<size_t>(ldw), out, M, N, K, kper);
   } else {
-    hipLaunchKernelGGL((gemm_mid_kernel<1, 8, 4>), grid, dim3(320), 0, stream, x, static_cast<size_t>(ldx), w,
+    hipLaunchKernelGGL((gemm_mid_kernel<1, kLoaders1, 4>), grid, dim3(256 + 64 * kLoaders1), 0, stream, x, static_cast<size_t>(ldx), w,
                        static_cast<size_t>(ldw), out, M, N, K, kper);
   }
   return check_launch("gemm_mid_bf16");

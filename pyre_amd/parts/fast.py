@@ -56,12 +56,13 @@ def mid_ksplit(n_out: int, k: int) -> int:
     """Into how many parts of k the kernel for 65 to 256 rows splits a product, or 0 if it is not
     the one to take. A block has 64 rows of the weights; the kernel is at its best when the blocks
     of all parts fill the 256 compute units in one round, and beats the BLAS library where that
-    takes at least two parts of 256 k or more (measured on the 1.5B, 7B and 32B shapes: q/k/v, the
+    takes at least two parts of 384 k or more (shorter parts gain nothing and cost the consumer
+    another addend; measured on the 1.5B, 7B and 32B shapes: q/k/v, the
     attention output and the feed-forward's way down take 9 to 20 us where the library takes 19
     to 31, and 60 against 100 at 7B's way down; the wide gate/up product stays with the library)."""
     blocks = -(-n_out // 64)
-    ks = min(256 // blocks, k // 256, MID_MAX_KSPLIT)
-    while ks > 1 and (ks - 1) * (-(-(-(-k // ks)) // 32) * 32) >= k:
+    ks = min(256 // blocks, k // 384, MID_MAX_KSPLIT)
+    while ks > 1 and (ks - 1) * (-(-(-(-k // ks)) // 64) * 64) >= k:
         ks -= 1  # would leave a part empty
     return ks if ks >= 2 else 0
 

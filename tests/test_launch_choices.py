@@ -181,7 +181,7 @@ def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():
 
 
 def test_mid_ksplit_fills_one_round_and_leaves_no_part_empty():
-    """The kernel for 65 to 256 rows is chosen where at least two parts of 256 k or more fill the
+    """The kernel for 65 to 256 rows is chosen where at least two parts of 384 k or more fill the
     256 compute units in one round of blocks of 64 output columns."""
     from pyre_amd.parts.fast import MID_MAX_KSPLIT, mid_ksplit
 
@@ -193,5 +193,5 @@ def test_mid_ksplit_fills_one_round_and_leaves_no_part_empty():
             ks = mid_ksplit(n_out, k)
             if ks:
                 blocks = -(-n_out // 64)
-                kper = -(-(-(-k // ks)) // 32) * 32
-                assert 2 <= ks <= MID_MAX_KSPLIT and blocks * ks <= 256 and k // ks >= 256 and (ks - 1) * kper < k
+                kper = -(-(-(-k // ks)) // 64) * 64
+                assert 2 <= ks <= MID_MAX_KSPLIT and blocks * ks <= 256 and k // ks >= 384 and (ks - 1) * kper < k
