@@ -100,8 +100,11 @@ def linear(lin, ctx, x, n, out):
         buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
         ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
         return Partials(buf, lin.bias)
-    if out is None and SKINNY_MAX_ROWS < n <= MID_MAX_ROWS and rt.options.get("mid_gemm", True):
+    mid = rt.options.get("mid_gemm", True)
+    if out is None and SKINNY_MAX_ROWS < n <= MID_MAX_ROWS and mid:
         ks = mid_ksplit(n_out, k)
+        if not ks and int(mid) == 2:  # tests: also where it does not pay, as with a tiny model
+            ks = 2 if k > 64 else 1
         if ks and ops.gemm_mid_supports(n, n_out, k, x.stride(0), lin.weight.stride(0)):
             buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
             ops.gemm_mid_bf16(x, lin.weight, buf, n, ks)

@@ -239,13 +239,15 @@ def test_decode_steps_of_requests_of_very_different_lengths(others, graphs, mode
         assert eng.graph_replays >= 7
 
 
-@pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
-                                                ("tiny-b", "float32", True)])
-def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, model_dirs, plain_models):
+@pytest.mark.parametrize("model,dtype,graphs,mid", [("tiny-c", "bfloat16", True, 1), ("tiny-c", "bfloat16", False, 1),
+                                                    ("tiny-b", "float32", True, 1), ("tiny-c", "bfloat16", True, 2),
+                                                    ("tiny-a", "bfloat16", False, 2)])
+def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, mid, model_dirs, plain_models):
     """200, 150, 100 and 70 live requests: decode steps whose products go to the BLAS library
-    (more than 64 rows), captured at 256, 192, 128 and 96 rows and replayed several times,
-    each replay against the plain implementation (a library call that records a clearing of
-    memory into the graph would be right once and wrong afterwards)."""
+    (more than 64 rows) or, with mid = 2, all to the kernel for 65 to 256 rows, which a tiny
+    model's sizes would not choose; captured at 256, 192, 128 and 96 rows and replayed several
+    times, each replay against the plain implementation (a library call that records a clearing
+    of memory into the graph would be right once and wrong afterwards)."""
     plain = plain_models[model]
     vocab = plain[0]["vocab_size"]
     prompt = [2 + (13 * i) % 37 for i in range(200)]
@@ -253,6 +255,7 @@ def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, 
     want = _expected(plain, reqs, dtype)
     eng = make_engine(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=200, max_cached_tokens=200 * 64,
                       max_num_batched_tokens=2048)
+    eng.runtime.options["mid_gemm"] = mid
     steps = [([(i, reqs[i][:prompt[i]], []) for i in range(lo, lo + 50)], []) for lo in range(0, 200, 50)]
     live, counts = list(range(200)), (200, 200, 200, 150, 150, 150, 100, 100, 100, 70, 70, 70)
     for k, keep in enumerate(counts):
