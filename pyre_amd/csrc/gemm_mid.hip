@@ -47,59 +47,67 @@ __device__ inline void wait_loads() {
 }
 __device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 0u, 0u};
 
-#ifndef PYRE_MID_NL2
-#define PYRE_MID_NL2 10
-#define PYRE_MID_NL1 6
-#endif
-constexpr int kLoaders2 = PYRE_MID_NL2, kLoaders1 = PYRE_MID_NL1;  // loading waves for 256 and for 128 rows of X
+enum Epilogue { kPartials = 0, kSiluMul = 1 };
 
-// NL loading waves beside the four that multiply, S stages in the ring. What a wave can have
-// loaded per microsecond is limited (about 9 GB/s from L2, whatever the pattern and however many
-// loads it has on their way), so the loads of a stage are dealt to several waves that do
-// nothing else; a stage is the 64 rows of W, then the BM rows of X.
-template <int CW, int NL, int S>
-__global__ __launch_bounds__(256 + 64 * NL) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
-                                                                 const bf16* __restrict__ W, size_t ldw,
-                                                                 float* __restrict__ out, int M, int N, int K,
-                                                                 int kper) {
-  constexpr int BM = 128 * CW, ROWS = BN + BM, STAGE = ROWS * 128;
-  constexpr int PER = ROWS / 8 / NL;  // loads of 8 rows per loading wave and stage
-  static_assert(ROWS / 8 % NL == 0, "the loads of a stage divide evenly over the loading waves");
+// RW groups of four multiplying waves, each group on 64 rows of W, and NL waves that only load; S
+// stages in the ring. What a wave can have loaded per microsecond is limited (about 9 GB/s from
+// L2, whatever the pattern and however many loads it has on their way; a compute unit takes
+// about 84 GB/s), so the loads of a stage are dealt to all waves, and there are more waves than
+// multiply; a stage is the 64 RW rows of W, then the BM rows of X. kSiluMul: a group's 64 rows are 32 gate rows and the up rows of the same features, so
+// that a lane holds both for its elements; out is bfloat16 [M][N / 2].
+template <int CW, int RW, int EPI, int NL, int S>
+__global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
+                                                                      const bf16* __restrict__ W, size_t ldw,
+                                                                      void* __restrict__ out, int M, int N, int K,
+                                                                      int kper) {
+  constexpr int BM = 128 * CW, BW = BN * RW, ROWS = BW + BM, STAGE = ROWS * 128;
+  constexpr int NWAVES = 4 * RW + NL;
+  constexpr int PER = ROWS / 8 / NWAVES;  // loads of 8 rows per wave and stage
+  static_assert(ROWS / 8 % NWAVES == 0, "the loads of a stage divide evenly over the waves");
   __shared__ __attribute__((aligned(1024))) unsigned char lds[S * STAGE];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int c = lane & 31, half = lane >> 5;
   const int ks = blockIdx.y, kbeg = ks * kper, kend = min(K, kbeg + kper);
   const int stages = (kend - kbeg + BK - 1) / BK;
+  const int inter = N / 2;
 
-  if (wave >= 4) {
-    // ---- a loading wave: of load j = l + NL i (rows 8 j .. 8 j + 7 of the stage) this lane
-    // brings the piece that lands at row 8 j + lane / 8, place lane % 8, which is piece
-    // (place ^ swizzle of the row) of the row's 64 k. Rows past the end are zeros.
-    const int l = wave - 4;
-    const unsigned lds_base = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds)));
-    const bf16* zero = reinterpret_cast<const bf16*>(kZeroPiece);
-    const bf16* src[PER];
-    int kofs[PER];
+  // Every wave loads: of load j = wave + NWAVES i (rows 8 j .. 8 j + 7 of the stage) this lane
+  // brings the piece that lands at row 8 j + lane / 8, place lane % 8, which is piece
+  // (place ^ swizzle of the row) of the row's 64 k. Rows past the end are zeros.
+  const unsigned lds_base = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds)));
+  const bf16* zero = reinterpret_cast<const bf16*>(kZeroPiece);
+  const bf16* src[PER];
+  int kofs[PER];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int row = 8 * (l + NL * i) + (lane >> 3);
-      kofs[i] = 8 * ((lane & 7) ^ ((row >> 1) & 7));
-      const bf16* base = nullptr;
-      if (row < BN) {
-        if (blockIdx.x * BN + row < N) base = W + static_cast<size_t>(blockIdx.x * BN + row) * ldw;
-      } else if (row - BN < M) {
-        base = X + static_cast<size_t>(row - BN) * ldx;
+  for (int i = 0; i < PER; ++i) {
+    const int row = 8 * (wave + NWAVES * i) + (lane >> 3);
+    kofs[i] = 8 * ((lane & 7) ^ ((row >> 1) & 7));
+    const bf16* base = nullptr;
+    if (row < BW) {
+      int n;  // the row of W behind row `row` of the block's tile, or past the end
+      if (EPI == kSiluMul) {
+        const int f = blockIdx.x * (32 * RW) + 32 * (row >> 6) + (row & 31);
+        n = f < inter ? ((row >> 5) & 1) * inter + f : N;
+      } else {
+        n = blockIdx.x * BW + row;
       }
-      src[i] = base ? base + kbeg + kofs[i] : nullptr;
+      if (n < N) base = W + static_cast<size_t>(n) * ldw;
+    } else if (row - BW < M) {
+      base = X + static_cast<size_t>(row - BW) * ldx;
     }
-    auto issue = [&](int st, int slot) {
-      const int left = st < stages ? kend - kbeg - BK * st : 0;  // k of this part from the stage's start on
+    src[i] = base ? base + kbeg + kofs[i] : nullptr;
+  }
+  auto issue = [&](int st, int slot) {
+    const int left = st < stages ? kend - kbeg - BK * st : 0;  // k of this part from the stage's start on
 #pragma unroll
-      for (int i = 0; i < PER; ++i)
-        load_to_lds(src[i] && kofs[i] < left ? src[i] + BK * st : zero, lds_base + slot * STAGE + (l + NL * i) * 1024);
-    };
+    for (int i = 0; i < PER; ++i)
+      load_to_lds(src[i] && kofs[i] < left ? src[i] + BK * st : zero, lds_base + slot * STAGE + (wave + NWAVES * i) * 1024);
+  };
 #pragma unroll
-    for (int st = 0; st < S - 1; ++st) issue(st, st);
+  for (int st = 0; st < S - 1; ++st) issue(st, st);
+
+  if (wave >= 4 * RW) {
+    // ---- a wave that only loads
     int slot = 0;
     for (int st = 0; st < stages; ++st) {
       wait_loads<PER * (S - 2)>();  // loads finish in the order of issue: this wave's share of stage st is there
@@ -111,7 +119,8 @@ __global__ __launch_bounds__(256 + 64 * NL) void gemm_mid_kernel(const bf16* __r
     return;
   }
 
-  // ---- a multiplying wave: its own 32 CW rows of X against the block's 64 rows of W.
+  // ---- a multiplying wave: its own 32 CW rows of X against its group's 64 rows of W.
+  const int group = wave >> 2, quarter = wave & 3;
   f32x16 acc[2][CW];
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt)
@@ -121,17 +130,20 @@ __global__ __launch_bounds__(256 + 64 * NL) void gemm_mid_kernel(const bf16* __r
       for (int i = 0; i < 16; ++i) acc[rt][ct][i] = 0.f;
 
   const int swz = (c >> 1) & 7;
-  const int xrow0 = BN + 32 * CW * wave + c;  // this lane's row of X in the stage, for tile 0
+  const int wrow0 = 64 * group + c;                // this lane's row of W in the stage, for tile 0
+  const int xrow0 = BW + 32 * CW * quarter + c;    // and of X
   int slot = 0;
   for (int st = 0; st < stages; ++st) {
-    __syncthreads();  // stage st is there; and everyone has multiplied stage st - 1
+    wait_loads<PER * (S - 2)>();  // this wave's share of stage st is there
+    __syncthreads();              // and everyone's; and everyone has multiplied stage st - 1
+    issue(st + S - 1, slot == 0 ? S - 1 : slot - 1);
     const unsigned char* sb = lds + slot * STAGE;
     // The operands of step kk + 1 are read from LDS while step kk is multiplied.
     bf16x8 a[2], b[CW], an[2], bn[CW];
     auto read = [&](int kk, bf16x8 (&ra)[2], bf16x8 (&rb)[CW]) {
       const int piece = 16 * ((2 * kk + half) ^ swz);
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt) ra[rt] = *reinterpret_cast<const bf16x8*>(sb + (32 * rt + c) * 128 + piece);
+      for (int rt = 0; rt < 2; ++rt) ra[rt] = *reinterpret_cast<const bf16x8*>(sb + (wrow0 + 32 * rt) * 128 + piece);
 #pragma unroll
       for (int ct = 0; ct < CW; ++ct) rb[ct] = *reinterpret_cast<const bf16x8*>(sb + (xrow0 + 32 * ct) * 128 + piece);
     };
@@ -151,29 +163,57 @@ __global__ __launch_bounds__(256 + 64 * NL) void gemm_mid_kernel(const bf16* __r
     }
     slot = slot + 1 == S ? 0 : slot + 1;
   }
+  wait_loads<0>();  // the loads past the end
 
-  // acc[rt][ct][4 q + j]: row 32 rt + 8 q + 4 half + j of the block's tile of W, row
-  // 32 (CW wave + ct) + c of X.
-  float* o = out + static_cast<size_t>(ks) * M * N;
-  const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  // acc[rt][ct][4 q + j]: row 32 rt + 8 q + 4 half + j of the group's tile of W, row
+  // 32 (CW quarter + ct) + c of X.
+  if (EPI == kPartials) {
+    float* o = static_cast<float*>(out) + static_cast<size_t>(ks) * M * N;
+    const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 #pragma unroll
-  for (int ct = 0; ct < CW; ++ct) {
-    const int m = 32 * (CW * wave + ct) + c;
-    if (m >= M) continue;
+    for (int ct = 0; ct < CW; ++ct) {
+      const int m = 32 * (CW * quarter + ct) + c;
+      if (m >= M) continue;
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = blockIdx.x * BW + 64 * group + 32 * rt + 8 * q + 4 * half;
+          if (n >= N) continue;
+          float* dst = o + static_cast<size_t>(m) * N + n;
+          if (vec && n + 3 < N) {
+            *reinterpret_cast<f32x4*>(dst) =
+                f32x4{acc[rt][ct][4 * q], acc[rt][ct][4 * q + 1], acc[rt][ct][4 * q + 2], acc[rt][ct][4 * q + 3]};
+          } else {
+            for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = acc[rt][ct][4 * q + j];
+          }
+        }
+    }
+  } else {
+    bf16* o = static_cast<bf16*>(out);
+    const bool vec = (inter & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0;
+#pragma unroll
+    for (int ct = 0; ct < CW; ++ct) {
+      const int m = 32 * (CW * quarter + ct) + c;
+      if (m >= M) continue;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = blockIdx.x * BN + 32 * rt + 8 * q + 4 * half;
-        if (n >= N) continue;
-        float* dst = o + static_cast<size_t>(m) * N + n;
-        if (vec && n + 3 < N) {
-          *reinterpret_cast<f32x4*>(dst) =
-              f32x4{acc[rt][ct][4 * q], acc[rt][ct][4 * q + 1], acc[rt][ct][4 * q + 2], acc[rt][ct][4 * q + 3]};
+        const int f = blockIdx.x * (32 * RW) + 32 * group + 8 * q + 4 * half;
+        if (f >= inter) continue;
+        float y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float gate = acc[0][ct][4 * q + j], up = acc[1][ct][4 * q + j];
+          y[j] = gate / (1.f + __expf(-gate)) * up;
+        }
+        bf16* dst = o + static_cast<size_t>(m) * inter + f;
+        if (vec && f + 3 < inter) {
+          *reinterpret_cast<uint2*>(dst) = uint2{pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
         } else {
-          for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = acc[rt][ct][4 * q + j];
+          for (int j = 0; j < 4 && f + j < inter; ++j) dst[j] = from_float<bf16>(y[j]);
         }
       }
+    }
   }
 }
 
@@ -203,11 +243,33 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
   if (M > 128) {
-    hipLaunchKernelGGL((gemm_mid_kernel<2, kLoaders2, 3>), grid, dim3(256 + 64 * kLoaders2), 0, stream, x, static_cast<size_t>(ldx), w,
-                       static_cast<size_t>(ldw), out, M, N, K, kper);
+    hipLaunchKernelGGL((gemm_mid_kernel<2, 1, kPartials, 6, 3>), grid, dim3(64 * 10), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
   } else {
-    hipLaunchKernelGGL((gemm_mid_kernel<1, kLoaders1, 4>), grid, dim3(256 + 64 * kLoaders1), 0, stream, x, static_cast<size_t>(ldx), w,
-                       static_cast<size_t>(ldw), out, M, N, K, kper);
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 1, kPartials, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
   }
   return check_launch("gemm_mid_bf16");
+}
+
+// W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
+// A block takes 64 features (64 gate rows and 64 up rows, eight multiplying waves).
+extern "C" int pyre_gemm_mid_silu_blocks(int two_i) { return (two_i / 2 + 63) / 64; }
+
+extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
+                                       int two_i, int K, hipStream_t stream) {
+  if (int rc = check_mid("gemm_mid_silu_bf16", X, W, M, two_i, K, ldx, ldw)) return rc;
+  PYRE_REQUIRE(two_i % 2 == 0, "gemm_mid_silu_bf16: gate and up rows must be equally many");
+  const int kper = (K + BK - 1) / BK * BK;
+  const dim3 grid(pyre_gemm_mid_silu_blocks(two_i), 1);
+  const bf16* x = static_cast<const bf16*>(X);
+  const bf16* w = static_cast<const bf16*>(W);
+  if (M > 128) {
+    hipLaunchKernelGGL((gemm_mid_kernel<2, 2, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 2, kSiluMul, 8, 4>), grid, dim3(64 * 16), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  }
+  return check_launch("gemm_mid_silu_bf16");
 }

@@ -553,6 +553,23 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, k
          w.shape[1], ksplit, _stream())
 
 
+def gemm_mid_silu_blocks(two_i: int) -> int:
+    from pyre_amd.hip.lib import lib
+
+    return int(lib().pyre_gemm_mid_silu_blocks(two_i))
+
+
+def gemm_mid_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int) -> None:
+    """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up], 1 <= m <= 256."""
+    _skinny_common(x, w_gate_up, m)
+    two_i = w_gate_up.shape[0]
+    if (out.dtype != torch.bfloat16 or not out.is_contiguous() or not out.is_cuda or out.dim() != 2
+            or out.shape[1] * 2 != two_i or out.shape[0] < m):
+        raise KernelError("gemm_mid_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
+    call("pyre_gemm_mid_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+         out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
+
+
 def read_bandwidth(device: str = "cuda:0", gib: float = 2.0, blocks: int = 4096, repeats: int = 10) -> float:
     """Measured streaming-read bandwidth in GB/s (a buffer larger than every cache)."""
     import time

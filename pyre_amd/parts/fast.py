@@ -129,9 +129,21 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
     """silu(x gate^T) * (x up^T) in one kernel for a decode step's few rows."""
     from pyre_amd.hip import ops
 
-    if not _is_bf16(ctx, lin, x) or n > FUSED_SILU_MAX_ROWS or lin.bias is not None:
+    if not _is_bf16(ctx, lin, x) or lin.bias is not None:
         return False
-    if not ctx.runtime.options.get("skinny_gemm", True):
+    if FUSED_SILU_MAX_ROWS < n <= MID_MAX_ROWS:
+        # 65 to 256 rows: blocks of 64 features against all rows, where one round of blocks holds
+        # them (measured: 17 us against the library's product and the SiLU-gate kernel's 29 at up
+        # to 128 rows on the 1.5B shape, 28 against 30 at 256; the 7B shape's 296 blocks would
+        # take two rounds and stay with the library)
+        mid = ctx.runtime.options.get("mid_gemm", True)
+        if not mid or not ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):
+            return False
+        if ops.gemm_mid_silu_blocks(lin.out_features) > 256 and int(mid) != 2:
+            return False
+        ops.gemm_mid_silu_bf16(x, lin.weight, act, n)
+        return True
+    if n > FUSED_SILU_MAX_ROWS or not ctx.runtime.options.get("skinny_gemm", True):
         return False
     if not ops.gemm_skinny_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):
         return False

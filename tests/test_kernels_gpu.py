@@ -830,6 +830,23 @@ def test_gemm_mid(m, n, k, ksplit):
     assert torch.equal(again, out)
 
 
+@pytest.mark.parametrize("m", [65, 128, 129, 256])
+@pytest.mark.parametrize("inter,k", [(176, 64), (8960, 1536), (250, 96), (70, 520)])
+def test_gemm_mid_silu(m, inter, k):
+    ops = _ops()
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    out = torch.full((m, inter), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops.gemm_mid_silu_bf16(x, w, out, m)
+    gu = x.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    assert torch.allclose(out.double(), want, atol=2e-2, rtol=2e-2)
+    rows = sorted({0, m // 2, m - 1})
+    few = torch.full((len(rows), inter), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops.gemm_mid_silu_bf16(x[rows].contiguous(), w, few, len(rows))
+    assert torch.equal(few, out[rows])
+
+
 def test_gemm_mid_refuses_what_it_cannot_take():
     ops = _ops()
     x, w = rnd(300, 64, dtype=torch.bfloat16), rnd(48, 64, dtype=torch.bfloat16)
