@@ -6,21 +6,22 @@
 // all rows of X of a step against 64 rows of W and splits k over blocks instead.
 //
 // The product is computed transposed, out^T = W X^T, on MFMA 32x32x16: A = 32 rows of W, B = 32
-// rows of X, both read along k as they are stored. A block owns 64 rows of W and BM = 128 or
-// 256 rows of X: four multiplying waves (wave w the rows 32 CW w .. of X, CW = 1 or 2 tiles,
-// against both tiles of W) and a fifth that loads W. k is walked in stages of 32 through two
-// rings in LDS, one of W and one of X, that are filled by loads from memory straight into LDS
-// several stages ahead; a stage holds its rows as 64-byte rows whose four 16-byte pieces are
-// exchanged among themselves by the row's number, so that the operand reads of 32 lanes (32
-// rows, the same k) spread over all banks. One barrier per stage: it publishes the stage that
-// has landed and frees the one before it.
+// rows of X, both read along k as they are stored. A block owns 64 RW rows of W and BM = 128 or
+// 256 rows of X: RW groups of four multiplying waves (a group on 64 rows of W, its wave q on the
+// rows 32 CW q .. of X, CW = 1 or 2 tiles, against both tiles of W) and some waves that only
+// load. k is walked in stages of 64 through a ring in LDS that is filled by loads from memory
+// straight into LDS, S - 1 stages ahead; a stage holds its rows as 128-byte rows whose eight
+// 16-byte pieces are exchanged among themselves by the row's number, so that the operand reads
+// of 32 lanes (32 rows, the same k) spread over all banks. One barrier per stage: it publishes
+// the stage that has landed and frees the one before it.
 //
-// `ksplit` blocks share rows of W (grid.y); each writes a partial sum, float32 [ksplit][M][N],
-// that the consumer adds in the order 0..ksplit-1. The order of an element's sums is a
-// function of k alone: a row's result does not depend on the other rows of the step or on
-// their number. The time is set by how many bytes a block has on their way at once (the rows of
-// X come from L2 again for every 64 rows of W): it pays where ksplit can fill the chip in one
-// round of blocks, which the caller checks.
+// kPartials: `ksplit` blocks share rows of W (grid.y); each writes a partial sum, float32
+// [ksplit][M][N], that the consumer adds in the order 0..ksplit-1. kSiluMul (W = gate rows, then
+// up rows; ksplit = 1): bfloat16 silu(gate) * up, [M][N / 2]. The order of an element's sums
+// is a function of k alone: a row's result does not depend on the other rows of the step or on
+// their number. The time is set by the bytes a compute unit can take from L2 (the rows of X
+// come again for every block): it pays where the blocks fill the chip in one round, which the
+// caller checks.
 #include "pyre_api.h"
 #include "pyre_common.h"
 
