@@ -42,6 +42,10 @@ constexpr int BK = 64;   // k per stage: rows of 128 bytes
 __device__ inline void load_to_lds(const void* src, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
 }
+// The same for bytes that are read once (the weights): past the caches.
+__device__ inline void load_to_lds_once(const void* src, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(src), "s"(lds_addr) : "memory", "m0");
+}
 template <int N>
 __device__ inline void wait_loads() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -62,10 +66,12 @@ __global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16
                                                                       void* __restrict__ out, int M, int N, int K,
                                                                       int kper) {
   constexpr int BM = 128 * CW, BW = BN * RW, ROWS = BW + BM, STAGE = ROWS * 128;
-  constexpr int NWAVES = 4 * RW + NL;
-  constexpr int PER = ROWS / 8 / NWAVES;  // loads of 8 rows per wave and stage
-  static_assert(ROWS / 8 % NWAVES == 0, "the loads of a stage divide evenly over the waves");
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[S * STAGE];
+  constexpr int NWAVES = 4 * RW + NL, LOADS = ROWS / 8;
+  constexpr int PER = (LOADS + NWAVES - 1) / NWAVES;  // loads of 8 rows per wave and stage
+  // Where the loads of a stage do not divide evenly over the waves, the spare turns load zeros
+  // into a kilobyte behind the ring, so that every wave counts the same number of loads.
+  constexpr bool SPARE = LOADS % NWAVES != 0;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[S * STAGE + (SPARE ? 1024 : 0)];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int c = lane & 31, half = lane >> 5;
   const int ks = blockIdx.y, kbeg = ks * kper, kend = min(K, kbeg + kper);
@@ -84,7 +90,9 @@ __global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16
     const int row = 8 * (wave + NWAVES * i) + (lane >> 3);
     kofs[i] = 8 * ((lane & 7) ^ ((row >> 1) & 7));
     const bf16* base = nullptr;
-    if (row < BW) {
+    if (row >= ROWS) {
+      // a spare turn
+    } else if (row < BW) {
       int n;  // the row of W behind row `row` of the block's tile, or past the end
       if (EPI == kSiluMul) {
         const int f = blockIdx.x * (32 * RW) + 32 * (row >> 6) + (row & 31);
@@ -101,8 +109,13 @@ __global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16
   auto issue = [&](int st, int slot) {
     const int left = st < stages ? kend - kbeg - BK * st : 0;  // k of this part from the stage's start on
 #pragma unroll
-    for (int i = 0; i < PER; ++i)
-      load_to_lds(src[i] && kofs[i] < left ? src[i] + BK * st : zero, lds_base + slot * STAGE + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < PER; ++i) {
+      const int j = wave + NWAVES * i;  // rows 8 j .. of the stage: of W up to BW / 8
+      const bf16* from = src[i] && kofs[i] < left ? src[i] + BK * st : zero;
+      const unsigned to = j < LOADS ? lds_base + slot * STAGE + j * 1024 : lds_base + S * STAGE;
+      if (j < BW / 8) load_to_lds_once(from, to);
+      else load_to_lds(from, to);
+    }
   };
 #pragma unroll
   for (int st = 0; st < S - 1; ++st) issue(st, st);
@@ -254,19 +267,30 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
 }
 
 // W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
-// A block takes 64 features (64 gate rows and 64 up rows, eight multiplying waves).
-extern "C" int pyre_gemm_mid_silu_blocks(int two_i) { return (two_i / 2 + 63) / 64; }
+// A block takes 64 features (64 gate rows and 64 up rows, eight multiplying waves), or 96 with
+// twelve for up to 128 rows of X where one round of blocks would not hold them otherwise.
+namespace {
+int silu_features(int M, int two_i) { return M <= 128 && (two_i / 2 + 63) / 64 > 256 ? 96 : 64; }
+}  // namespace
+
+extern "C" int pyre_gemm_mid_silu_blocks(int M, int two_i) {
+  const int f = silu_features(M, two_i);
+  return (two_i / 2 + f - 1) / f;
+}
 
 extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
                                        int two_i, int K, hipStream_t stream) {
   if (int rc = check_mid("gemm_mid_silu_bf16", X, W, M, two_i, K, ldx, ldw)) return rc;
   PYRE_REQUIRE(two_i % 2 == 0, "gemm_mid_silu_bf16: gate and up rows must be equally many");
   const int kper = (K + BK - 1) / BK * BK;
-  const dim3 grid(pyre_gemm_mid_silu_blocks(two_i), 1);
+  const dim3 grid(pyre_gemm_mid_silu_blocks(M, two_i), 1);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
   if (M > 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 2, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (silu_features(M, two_i) == 96) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 3, kSiluMul, 4, 3>), grid, dim3(64 * 16), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 2, kSiluMul, 8, 4>), grid, dim3(64 * 16), 0, stream, x,

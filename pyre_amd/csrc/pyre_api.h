@@ -71,9 +71,9 @@ int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw,
 int pyre_gemm_mid_supports(int M, int N, int K, long ldx, long ldw);
 int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N, int K,
                        int ksplit, hipStream_t stream);
-// The second of them for up to 256 rows: a block takes 64 features (pyre_gemm_mid_silu_blocks of
-// them in all) against all rows of X; it pays where one round of blocks holds them.
-int pyre_gemm_mid_silu_blocks(int two_i);
+// The second of them for up to 256 rows: a block takes 64 or 96 features (pyre_gemm_mid_silu_blocks
+// blocks in all) against all rows of X; it pays where one round of blocks holds them.
+int pyre_gemm_mid_silu_blocks(int M, int two_i);
 int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i,
                             int K, hipStream_t stream);
 

@@ -553,10 +553,10 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, k
          w.shape[1], ksplit, _stream())
 
 
-def gemm_mid_silu_blocks(two_i: int) -> int:
+def gemm_mid_silu_blocks(m: int, two_i: int) -> int:
     from pyre_amd.hip.lib import lib
 
-    return int(lib().pyre_gemm_mid_silu_blocks(two_i))
+    return int(lib().pyre_gemm_mid_silu_blocks(m, two_i))
 
 
 def gemm_mid_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int) -> None:

@@ -23,6 +23,8 @@ FUSED_SILU_MAX_ROWS = 64
 #: most rows of the kernel between the two, which keeps a step's rows against 64 rows of the weights
 MID_MAX_ROWS = 256
 MID_MAX_KSPLIT = 12
+#: fewest rows at which that kernel takes the gate/up product with the SiLU-gate
+MID_SILU_MIN_ROWS = 65
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
@@ -131,18 +133,19 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
 
     if not _is_bf16(ctx, lin, x) or lin.bias is not None:
         return False
-    if FUSED_SILU_MAX_ROWS < n <= MID_MAX_ROWS:
-        # 65 to 256 rows: blocks of 64 features against all rows, where one round of blocks holds
-        # them (measured: 17 us against the library's product and the SiLU-gate kernel's 29 at up
-        # to 128 rows on the 1.5B shape, 28 against 30 at 256; the 7B shape's 296 blocks would
-        # take two rounds and stay with the library)
+    if MID_SILU_MIN_ROWS <= n <= MID_MAX_ROWS:
+        # blocks of 64 features (96 where that is what it takes, up to 128 rows) against all rows,
+        # where one round of blocks holds them. Measured on the 1.5B shape: 17 us against the
+        # library's product and the SiLU-gate kernel's 29 at 65 to 128 rows, 28 against 30 at 256;
+        # on the 7B shape 55 against 66 at 128, and at 256 rows, as on the 32B shape, two rounds of
+        # blocks: those stay with the library. At 64 rows and fewer the weight-streaming kernel,
+        # whose loads go past the caches, is the faster one in a step (7B, 64 rows: 6.08 ms a
+        # step against 6.24), though not where the same weights are read again and again.
         mid = ctx.runtime.options.get("mid_gemm", True)
-        if not mid or not ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):
-            return False
-        if ops.gemm_mid_silu_blocks(lin.out_features) > 256 and int(mid) != 2:
-            return False
-        ops.gemm_mid_silu_bf16(x, lin.weight, act, n)
-        return True
+        fits = mid and ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0))
+        if fits and (ops.gemm_mid_silu_blocks(n, lin.out_features) <= 256 or int(mid) == 2):
+            ops.gemm_mid_silu_bf16(x, lin.weight, act, n)
+            return True
     if n > FUSED_SILU_MAX_ROWS or not ctx.runtime.options.get("skinny_gemm", True):
         return False
     if not ops.gemm_skinny_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):

@@ -830,10 +830,13 @@ def test_gemm_mid(m, n, k, ksplit):
     assert torch.equal(again, out)
 
 
-@pytest.mark.parametrize("m", [65, 128, 129, 256])
-@pytest.mark.parametrize("inter,k", [(176, 64), (8960, 1536), (250, 96), (70, 520)])
+@pytest.mark.parametrize("m", [33, 65, 128, 129, 256])
+@pytest.mark.parametrize("inter,k", [(176, 64), (8960, 1536), (250, 96), (70, 520), (18944, 136), (16401, 64)])
 def test_gemm_mid_silu(m, inter, k):
+    """Blocks of 64 features, and of 96 for up to 128 rows where 64 would make more than 256
+    blocks (the last two sizes), whose loads do not divide evenly over the block's waves."""
     ops = _ops()
+    assert ops.gemm_mid_silu_blocks(m, 2 * inter) == -(-inter // (96 if m <= 128 and inter > 256 * 64 else 64))
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
     w = rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.1)
     out = torch.full((m, inter), float("nan"), device=DEV, dtype=torch.bfloat16)
