@@ -58,8 +58,9 @@ enum Epilogue { kPartials = 0, kSiluMul = 1 };
 // stages in the ring. What a wave can have loaded per microsecond is limited (about 9 GB/s from
 // L2, whatever the pattern and however many loads it has on their way; a compute unit takes
 // about 84 GB/s), so the loads of a stage are dealt to all waves, and there are more waves than
-// multiply; a stage is the 64 RW rows of W, then the BM rows of X. kSiluMul: a group's 64 rows are 32 gate rows and the up rows of the same features, so
-// that a lane holds both for its elements; out is bfloat16 [M][N / 2].
+// multiply; a stage is the 64 RW rows of W, then the BM rows of X. kSiluMul: a group's 64 rows
+// are 32 gate rows and the up rows of the same features, so that a lane holds both for its
+// elements; out is bfloat16 [M][N / 2].
 template <int CW, int RW, int EPI, int NL, int S>
 __global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
                                                                       const bf16* __restrict__ W, size_t ldw,
