@@ -7,7 +7,7 @@
 //
 // The product is computed transposed, out^T = W X^T, on MFMA 32x32x16: A = 32 rows of W, B = 32
 // rows of X, both read along k as they are stored. A block owns 64 RW rows of W and BM = 128 or
-// 256 rows of X: RW groups of four multiplying waves (a group on 64 rows of W, its wave q on the
+// 256 rows of X: RW groups of XW = 4 multiplying waves (a group on 64 rows of W, its wave q on the
 // rows 32 CW q .. of X, CW = 1 or 2 tiles, against both tiles of W) and some waves that only
 // load. k is walked in stages of 64 through a ring in LDS that is filled by loads from memory
 // straight into LDS, S - 1 stages ahead; a stage holds its rows as 128-byte rows whose eight
@@ -54,20 +54,20 @@ __device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 
 
 enum Epilogue { kPartials = 0, kSiluMul = 1 };
 
-// RW groups of four multiplying waves, each group on 64 rows of W, and NL waves that only load; S
+// RW groups of XW multiplying waves, each group on 64 rows of W, and NL waves that only load; S
 // stages in the ring. What a wave can have loaded per microsecond is limited (about 9 GB/s from
 // L2, whatever the pattern and however many loads it has on their way; a compute unit takes
 // about 84 GB/s), so the loads of a stage are dealt to all waves, and there are more waves than
 // multiply; a stage is the 64 RW rows of W, then the BM rows of X. kSiluMul: a group's 64 rows
 // are 32 gate rows and the up rows of the same features, so that a lane holds both for its
 // elements; out is bfloat16 [M][N / 2].
-template <int CW, int RW, int EPI, int NL, int S>
-__global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
+template <int CW, int XW, int RW, int EPI, int NL, int S>
+__global__ __launch_bounds__(64 * (XW * RW + NL)) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
                                                                       const bf16* __restrict__ W, size_t ldw,
                                                                       void* __restrict__ out, int M, int N, int K,
                                                                       int kper) {
-  constexpr int BM = 128 * CW, BW = BN * RW, ROWS = BW + BM, STAGE = ROWS * 128;
-  constexpr int NWAVES = 4 * RW + NL, LOADS = ROWS / 8;
+  constexpr int BM = 32 * CW * XW, BW = BN * RW, ROWS = BW + BM, STAGE = ROWS * 128;
+  constexpr int NWAVES = XW * RW + NL, LOADS = ROWS / 8;
   constexpr int PER = (LOADS + NWAVES - 1) / NWAVES;  // loads of 8 rows per wave and stage
   // Where the loads of a stage do not divide evenly over the waves, the spare turns load zeros
   // into a kilobyte behind the ring, so that every wave counts the same number of loads.
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16
 #pragma unroll
   for (int st = 0; st < S - 1; ++st) issue(st, st);
 
-  if (wave >= 4 * RW) {
+  if (wave >= XW * RW) {
     // ---- a wave that only loads
     int slot = 0;
     for (int st = 0; st < stages; ++st) {
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(64 * (4 * RW + NL)) void gemm_mid_kernel(const bf16
   }
 
   // ---- a multiplying wave: its own 32 CW rows of X against its group's 64 rows of W.
-  const int group = wave >> 2, quarter = wave & 3;
+  const int group = wave / XW, quarter = wave % XW;
   f32x16 acc[2][CW];
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt)
@@ -258,10 +258,10 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
   if (M > 128) {
-    hipLaunchKernelGGL((gemm_mid_kernel<2, 1, kPartials, 6, 3>), grid, dim3(64 * 10), 0, stream, x,
+    hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 1, kPartials, 6, 3>), grid, dim3(64 * 10), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
   } else {
-    hipLaunchKernelGGL((gemm_mid_kernel<1, 1, kPartials, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 1, kPartials, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
   }
   return check_launch("gemm_mid_bf16");
@@ -288,13 +288,13 @@ extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, l
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
   if (M > 128) {
-    hipLaunchKernelGGL((gemm_mid_kernel<2, 2, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
+    hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 2, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else if (silu_features(M, two_i) == 96) {
-    hipLaunchKernelGGL((gemm_mid_kernel<1, 3, kSiluMul, 4, 3>), grid, dim3(64 * 16), 0, stream, x,
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 3, kSiluMul, 4, 3>), grid, dim3(64 * 16), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else {
-    hipLaunchKernelGGL((gemm_mid_kernel<1, 2, kSiluMul, 8, 4>), grid, dim3(64 * 16), 0, stream, x,
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 2, kSiluMul, 8, 4>), grid, dim3(64 * 16), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   }
   return check_launch("gemm_mid_silu_bf16");
