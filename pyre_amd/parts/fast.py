@@ -24,7 +24,7 @@ FUSED_SILU_MAX_ROWS = 64
 MID_MAX_ROWS = 256
 MID_MAX_KSPLIT = 12
 #: fewest rows at which that kernel takes the gate/up product with the SiLU-gate
-MID_SILU_MIN_ROWS = 65
+MID_SILU_MIN_ROWS = 33
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
@@ -133,14 +133,14 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
 
     if not _is_bf16(ctx, lin, x) or lin.bias is not None:
         return False
-    if MID_SILU_MIN_ROWS <= n <= MID_MAX_ROWS:
+    if ctx.runtime.options.get("mid_silu_min_rows", MID_SILU_MIN_ROWS) <= n <= MID_MAX_ROWS:
         # blocks of 64 features (96 where that is what it takes, up to 128 rows) against all rows,
         # where one round of blocks holds them. Measured on the 1.5B shape: 17 us against the
         # library's product and the SiLU-gate kernel's 29 at 65 to 128 rows, 28 against 30 at 256;
         # on the 7B shape 55 against 66 at 128, and at 256 rows, as on the 32B shape, two rounds of
-        # blocks: those stay with the library. At 64 rows and fewer the weight-streaming kernel,
-        # whose loads go past the caches, is the faster one in a step (7B, 64 rows: 6.08 ms a
-        # step against 6.24), though not where the same weights are read again and again.
+        # blocks: those stay with the library. In a decode step of the 7B shape it is ahead of the
+        # weight-streaming kernel from 48 rows on (5.40 against 5.47 ms a step at 48, 5.97 against
+        # 6.13 at 64; at 32 rows 4.69 against 4.64), on the 1.5B shape by 2 % from 24 rows on.
         mid = ctx.runtime.options.get("mid_gemm", True)
         fits = mid and ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0))
         if fits and (ops.gemm_mid_silu_blocks(n, lin.out_features) <= 256 or int(mid) == 2):
