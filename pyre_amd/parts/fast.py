@@ -14,11 +14,12 @@ import torch
 
 from pyre_amd.hip.ops import Partials
 
-#: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the BLAS library
+#: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the kernel for 65 to
+#: 256 rows where it pays and else to the BLAS library
 SKINNY_MAX_ROWS = 64
 #: the most partial sums of a weight-streaming product
 SKINNY_MAX_KSPLIT = 12
-#: up to this many rows the gate/up product and the SiLU-gate are one kernel
+#: up to this many rows the gate/up product and the SiLU-gate are one weight-streaming kernel
 FUSED_SILU_MAX_ROWS = 64
 #: most rows of the kernel between the two, which keeps a step's rows against 64 rows of the weights
 MID_MAX_ROWS = 256
@@ -128,7 +129,8 @@ def linear(lin, ctx, x, n, out):
 
 
 def gate_up_silu(lin, ctx, x, n, act) -> bool:
-    """silu(x gate^T) * (x up^T) in one kernel for a decode step's few rows."""
+    """silu(x gate^T) * (x up^T) in one kernel: the weight-streaming kernel for a decode step's few
+    rows, the kernel that keeps all rows in a block for 33 to 256 where it pays."""
     from pyre_amd.hip import ops
 
     if not _is_bf16(ctx, lin, x) or lin.bias is not None:
