@@ -35,6 +35,31 @@ template <> struct Vec4<bf16> {
 
 __device__ inline float4 add4(float4 a, float4 b) { return float4{a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w}; }
 
+// The same loads and stores past the caches, for rows that are read and written once in a step of
+// many rows (more bytes than the caches hold).
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
+template <typename T> struct Stream4;
+template <> struct Stream4<float> {
+  static __device__ inline float4 load(const float* p) {
+    const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+    return float4{v[0], v[1], v[2], v[3]};
+  }
+  static __device__ inline void store(float* p, float4 v) {
+    __builtin_nontemporal_store(f32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4_t*>(p));
+  }
+};
+template <> struct Stream4<bf16> {
+  static __device__ inline float4 load(const bf16* p) {
+    const u32x2_t u = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
+    return float4{__uint_as_float(u[0] << 16), __uint_as_float(u[0] & 0xffff0000u), __uint_as_float(u[1] << 16),
+                  __uint_as_float(u[1] & 0xffff0000u)};
+  }
+  static __device__ inline void store(bf16* p, float4 v) {
+    __builtin_nontemporal_store(u32x2_t{pack_bf16x2(v.x, v.y), pack_bf16x2(v.z, v.w)}, reinterpret_cast<u32x2_t*>(p));
+  }
+};
+
 // p[0] + p[1] + ... + p[n - 1] (in that order) of the float4 at `src` in each of n partial sums that
 // lie `stride` elements apart. Up to kAtOnce loads are in flight together: a kernel that only
 // passes a few rows on spends its time waiting for loads, one round trip after the other.
@@ -68,7 +93,7 @@ constexpr int kNormMaxVec = 8;  // float4 per thread
 // reduced by the butterfly of wave_sum; the 16 results are added in ascending order).
 // The 256-thread variant then plays VIRT = 4 of those threads per thread: t = thread +
 // 256 j. A position's result therefore does not depend on how many rows share the step.
-template <typename TD, typename TG, typename TO, int THREADS, int VIRT>
+template <typename TD, typename TG, typename TO, int THREADS, int VIRT, bool STREAM>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, int n_partials, size_t partial_stride,
     const TG* __restrict__ gain, TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
@@ -84,11 +109,20 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
   for (int i = 0; i < kNormMaxVec; ++i) {
     const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) break;
-    float4 x = Vec4<float>::load(resid + in_off + 4 * c);
+    float4 x = STREAM ? Stream4<float>::load(resid + in_off + 4 * c) : Vec4<float>::load(resid + in_off + 4 * c);
     if (delta) {
-      const float4 d = sum_partials4<TD>(delta + in_off + 4 * c, partial_stride, n_partials);
+      float4 d;
+      if (STREAM) {  // the same sums in the same order
+        d = Stream4<TD>::load(delta + in_off + 4 * c);
+        for (int p = 1; p < n_partials; ++p) d = add4(d, Stream4<TD>::load(delta + p * partial_stride + in_off + 4 * c));
+      } else {
+        d = sum_partials4<TD>(delta + in_off + 4 * c, partial_stride, n_partials);
+      }
       x = add4(x, d);
-      if (!rows) Vec4<float>::store(resid + in_off + 4 * c, x);
+      if (!rows) {
+        if (STREAM) Stream4<float>::store(resid + in_off + 4 * c, x);
+        else Vec4<float>::store(resid + in_off + 4 * c, x);
+      }
     }
     v[i] = x;
     // explicit fused multiply-adds: the same roundings in every variant of the kernel
@@ -117,14 +151,16 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
     if (c >= nvec) break;
     const float4 gn = Vec4<TG>::load(gain + 4 * c);
     const float4 x = v[i];
-    Vec4<TO>::store(out + out_off + 4 * c, float4{x.x * inv * gn.x, x.y * inv * gn.y, x.z * inv * gn.z, x.w * inv * gn.w});
+    const float4 y{x.x * inv * gn.x, x.y * inv * gn.y, x.z * inv * gn.z, x.w * inv * gn.w};
+    if (STREAM) Stream4<TO>::store(out + out_off + 4 * c, y);
+    else Vec4<TO>::store(out + out_off + 4 * c, y);
   }
 }
 
 // ---------------------------------------------------------------------------
 // rotary + cache write, four pairs per item; grid (tokens, ceil(items / 256)).
 // ---------------------------------------------------------------------------
-template <typename TI, typename TC>
+template <typename TI, typename TC, bool STREAM>
 __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
     const TI* __restrict__ qkv, int n_partials, size_t partial_stride, const void* __restrict__ bias,
     int bias_dt, TC* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
@@ -141,7 +177,13 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
 
   auto value4 = [&](int col) {
-    float4 v = sum_partials4<TI>(qkv + in_row + col, partial_stride, n_partials);
+    float4 v;
+    if (STREAM) {  // the product's rows of a step of many tokens are read once: past the caches
+      v = Stream4<TI>::load(qkv + in_row + col);
+      for (int p = 1; p < n_partials; ++p) v = add4(v, Stream4<TI>::load(qkv + p * partial_stride + in_row + col));
+    } else {
+      v = sum_partials4<TI>(qkv + in_row + col, partial_stride, n_partials);
+    }
     if (bias) {  // col is a multiple of 4: one load of four
       v = add4(v, bias_dt == kF32 ? Vec4<float>::load(static_cast<const float*>(bias) + col)
                                   : Vec4<bf16>::load(static_cast<const bf16*>(bias) + col));
@@ -235,14 +277,17 @@ bool add_rmsnorm_vec(float* resid, const void* delta, int delta_dt, int n_partia
   // Which variant runs depends on the number of rows; what it computes does not (see the kernel).
   const bool wide = hidden > 1024;
   const bool few = n <= 128 && wide;  // a decode step: spread each row over more threads
-#define PYRE_NORM_LAUNCH(THREADS, VIRT)                                                                     \
-  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, THREADS, VIRT>), dim3(n), dim3(THREADS), 0, stream, \
-                     resid, static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),  \
+#define PYRE_NORM_LAUNCH(THREADS, VIRT, STREAM)                                                                      \
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, THREADS, VIRT, STREAM>), dim3(n), dim3(THREADS), 0, stream, \
+                     resid, static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),          \
                      static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps)
   PYRE_DISPATCH(delta_dt, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO, {
-    if (few) PYRE_NORM_LAUNCH(1024, 1);
-    else if (wide) PYRE_NORM_LAUNCH(256, 4);
-    else PYRE_NORM_LAUNCH(256, 1);
+    const bool many = n >= 512;  // more bytes than the caches keep for the next kernel
+    if (few) PYRE_NORM_LAUNCH(1024, 1, false);
+    else if (wide && many) PYRE_NORM_LAUNCH(256, 4, true);
+    else if (wide) PYRE_NORM_LAUNCH(256, 4, false);
+    else if (many) PYRE_NORM_LAUNCH(256, 1, true);
+    else PYRE_NORM_LAUNCH(256, 1, false);
   })));
 #undef PYRE_NORM_LAUNCH
   return true;
@@ -257,12 +302,19 @@ bool rope_kv_write_vec(const void* qkv, int qkv_dt, int n_partials, long partial
   const int items = (nq + nkv) * (hd / 8) + nkv * (hd / 4);
   const dim3 grid(n, (items + 255) / 256);
   if (grid.y > 65535) return false;
-  PYRE_DISPATCH(qkv_dt, TI, PYRE_DISPATCH(q_dt, TC,
-      hipLaunchKernelGGL((rope_kv_write_vec_kernel<TI, TC>), grid, dim3(256), 0, stream,
-                         static_cast<const TI*>(qkv), n_partials, static_cast<size_t>(partial_stride), bias,
-                         bias_dt, static_cast<TC*>(q_out), static_cast<TC*>(k_cache),
-                         static_cast<TC*>(v_cache), cos_t, sin_t, positions, slots, nq, nkv, hd, page_size,
-                         write_kv)));
+#define PYRE_ROPE_LAUNCH(STREAM)                                                                                   \
+  PYRE_DISPATCH(qkv_dt, TI, PYRE_DISPATCH(q_dt, TC,                                                               \
+      hipLaunchKernelGGL((rope_kv_write_vec_kernel<TI, TC, STREAM>), grid, dim3(256), 0, stream,                  \
+                         static_cast<const TI*>(qkv), n_partials, static_cast<size_t>(partial_stride), bias,      \
+                         bias_dt, static_cast<TC*>(q_out), static_cast<TC*>(k_cache),                             \
+                         static_cast<TC*>(v_cache), cos_t, sin_t, positions, slots, nq, nkv, hd, page_size,       \
+                         write_kv)))
+  if (n >= 512) {
+    PYRE_ROPE_LAUNCH(true);
+  } else {
+    PYRE_ROPE_LAUNCH(false);
+  }
+#undef PYRE_ROPE_LAUNCH
   return true;
 }
 
