@@ -17,15 +17,17 @@ generated so far (which it keeps). A request that could not fit the pool even
 alone is refused when it is added. (The reference lets ``MemoryError`` escape,
 `pyre/paged_cache.py:58-67`.)
 
-While every running request is decoding and no waiting request could be admitted
-(nobody waits, or as many run as may), the next step is put on
-the device before the host has seen this step's tokens: its batch is known (the same
-requests, one position further, minus those that reach their length), and the tokens
-are fed on the device from the sampler's ids. The host then reads this step's tokens
-while the next step runs. A request that turns out to have ended (its end-of-sequence
-token) has one surplus row in that next step, which is ignored. This needs an engine
-whose ``step`` takes ``fed_ids`` and a sampler with ``launch``/``collect``/``ids``;
-with others every step waits for its tokens as before.
+Where it can, the next step is put on the device before the host has seen this step's
+tokens: it is planned as if every request that this step samples for had one more token
+(those that reach their length aside, which are left out), and those tokens are fed on the
+device from the sampler's ids. The host then reads this step's tokens while the next step
+runs, and the device does not wait while the host plans. Portions of prompts and newly
+admitted requests ride in such a step like in any other; a place or pages that become free
+with this step's results are seen one step later. A request that turns out to have ended
+(its end-of-sequence token) has one surplus row in that next step, which is ignored. If
+the next step would have to preempt somebody it is planned with the tokens known, as
+usual. This needs an engine whose ``step`` takes ``fed_ids`` and a sampler with
+``launch``/``collect``/``ids``; with others every step waits for its tokens as before.
 
 This module needs neither torch nor a GPU: the engine and the sampler are passed in.
 """
@@ -48,6 +50,10 @@ class Request:
     num_computed: int = 0            #: tokens of prompt + generated that are in the cache
     finish_reason: str | None = None  #: "eos" | "length"
     preemptions: int = 0
+    #: while the next step is planned ahead of this step's tokens: one token more that is
+    #: on the device only / the request reaches its length with that token
+    pending: int = 0
+    ending: bool = False
 
     @property
     def tokens(self) -> list[int]:
@@ -64,7 +70,7 @@ class Request:
 
     @property
     def cur_len(self) -> int:        # pyre/scheduler.py:22-24
-        return len(self.prompt_ids) + len(self.generated)
+        return len(self.prompt_ids) + len(self.generated) + self.pending
 
     @property
     def done(self) -> bool:
@@ -144,9 +150,11 @@ class Scheduler:
 
     # ------------------------------------------------------------------ planning
 
-    def plan(self) -> StepPlan:
+    def plan(self, ahead: bool = False) -> StepPlan | None:
         """Decide the next batch. Changes queue membership (admission, preemption)
-        and frees preempted requests' pages; reserves nothing."""
+        and frees preempted requests' pages; reserves nothing. ``ahead``: requests marked
+        ``ending`` are left out, and None is returned, with nothing changed, if somebody
+        would have to be preempted."""
         budget = self.token_budget
         free = self.cache.free_pages()
         entries: list[PlannedEntry] = []
@@ -160,8 +168,13 @@ class Scheduler:
         i = 0
         while i < len(self.running) and budget > 0:
             r = self.running[i]
+            if ahead and r.ending:
+                i += 1
+                continue
             n = portion(r, budget)
             need = self.cache.pages_needed(r.seq_id, n)
+            if ahead and need > free:
+                return None
             while need > free:
                 victim = self.running[-1]
                 if victim is r and len(self.running) == 1:
@@ -182,12 +195,14 @@ class Scheduler:
 
         # 2. admit waiting requests, first come first served (pyre/scheduler.py:49-50)
         # Pages that running prompts will still take in later steps are spoken for.
-        planned = {e.request.seq_id: e.count for e in entries}
-        promised = sum(
-            self.cache.pages_needed(r.seq_id, r.cur_len - r.num_computed)
-            - self.cache.pages_needed(r.seq_id, planned.get(r.seq_id, 0)) for r in self.running)
+        promised = None
         while (self.waiting and not preempted and budget > 0 and len(self.running) < self.max_batch
                and self.cache.has_free_slot()):
+            if promised is None:  # worked out only when somebody waits and could be let in
+                planned = {e.request.seq_id: e.count for e in entries}
+                promised = sum(
+                    self.cache.pages_needed(r.seq_id, r.cur_len - r.num_computed)
+                    - self.cache.pages_needed(r.seq_id, planned.get(r.seq_id, 0)) for r in self.running)
             r = self.waiting[0]
             n = portion(r, budget)
             need_now = self.cache.pages_needed(None, n)
@@ -242,7 +257,7 @@ class Scheduler:
                   for r in sampling]
             if self.lookahead:
                 handle = self.sampler.launch(logits, temps, us)
-                self._ahead = self._run_ahead(plan, sampling)
+                self._ahead = self._run_ahead(sampling)
                 new = self.sampler.collect(handle)
             else:
                 new = self.sampler.sample(logits, temps, us)
@@ -263,23 +278,35 @@ class Scheduler:
             self.finished[r.seq_id] = r
         return out
 
-    def _run_ahead(self, plan: StepPlan, sampling: list[Request]):
-        """Put the next step on the device if it is known without this step's tokens:
-        all running requests have just been sampled for, no waiting request could join
-        them, and the pages are there. Returns (plan, logits) or None. The sampler's ids of this step must
-        already be on the stream."""
-        if len(sampling) != len(self.running) or len(plan.entries) != len(sampling):
-            return None
-        rows = [(i, r) for i, r in enumerate(sampling)
-                if not r.done and len(r.generated) + 1 < r.params.max_new_tokens]
-        if not rows or len(rows) > self.token_budget:
-            return None
-        if self.waiting and len(rows) < self.max_batch:
-            return None  # the next step may admit a waiting request: it has to be planned with this step's results
-        if sum(self.cache.pages_needed(r.seq_id, 1) for _, r in rows) > self.cache.free_pages():
-            return None
-        nxt = StepPlan([PlannedEntry(r, r.num_computed, 1, True) for _, r in rows], [], [])
-        entries = [Entry(r.seq_id, [0], [0], feed=i) for i, r in rows]
+    def _run_ahead(self, sampling: list[Request]):
+        """Plan the next step without this step's tokens and put it on the device. Returns
+        (plan, logits) or None. The sampler's ids of this step must already be on the stream."""
+        feed = {}
+        marked = []
+        for i, r in enumerate(sampling):
+            if r.done:
+                continue  # a surplus row of the step before
+            marked.append(r)
+            if len(r.generated) + 1 >= r.params.max_new_tokens:
+                r.ending = True
+            else:
+                r.pending = 1
+                feed[r.seq_id] = i
+        try:
+            nxt = self.plan(ahead=True)
+            if nxt is None or not nxt.entries:
+                return None
+            entries = []
+            for e in nxt.entries:
+                r = e.request
+                if r.pending and e.start + e.count == r.cur_len:
+                    assert e.count == 1, "a request that was sampled for has all but one token in the cache"
+                    entries.append(Entry(r.seq_id, [0], [0], feed=feed[r.seq_id]))
+                else:
+                    entries.append(Entry(r.seq_id, r.token_slice(e.start, e.count), [e.count - 1] if e.samples else []))
+        finally:
+            for r in marked:
+                r.pending, r.ending = 0, False
         logits = self.engine.step(entries, fed_ids=self.sampler.ids)
         return nxt, logits
 

@@ -202,12 +202,14 @@ class AheadEngine(FakeEngine):
         super().__init__(**kw)
         self.fed = {}  #: rid -> every token the engine has been given for it, in order
         self.ahead_steps = 0
+        self.mixed_ahead_steps = 0  #: of them, steps that also carry tokens the host knows (prompt portions)
 
     def step(self, entries, fed_ids=None):
         for e in entries:
             toks = [fed_ids[e.feed]] if e.feed is not None else list(e.tokens)
             self.fed.setdefault(e.rid, []).extend(toks)
         self.ahead_steps += any(e.feed is not None for e in entries)
+        self.mixed_ahead_steps += any(e.feed is not None for e in entries) and any(e.feed is None for e in entries)
         return super().step(entries)
 
 
@@ -262,8 +264,9 @@ def test_a_request_added_meanwhile_waits_one_step():
     a = s.add_request([1, 2, 3], 8)
     s.step(), s.step()                      # the second step has put a third one on the device
     b = s.add_request([9, 9], 4)
-    s.step()                                # consumes the step that ran ahead; b still waits
-    assert [r.seq_id for r in s.waiting] == [b]
+    s.step()                                # consumes the step that ran ahead, without b; the next one has it
+    assert len(eng.steps) == 4
+    assert b not in [rid for rid, _, _ in eng.steps[2]] and b in [rid for rid, _, _ in eng.steps[3]]
     out = s.run()
     assert out[a] == expected([1, 2, 3], 8) and out[b] == expected([9, 9], 4)
 
@@ -294,7 +297,35 @@ def test_running_ahead_while_others_wait_for_a_free_place():
     assert first_seen(eng1) == first_seen(eng0) == list(range(6))
 
 
-@pytest.mark.parametrize("seed", range(6))
+def test_steps_with_prompt_portions_run_ahead_too():
+    """Long prompts arrive while others decode: the steps that carry their portions, and the
+    steps that admit them, are put on the device before the tokens of the step before are
+    read; the tokens are those of a run that waits for every step."""
+    prompts = [[3, 1], [2] * 70, [9, 8, 7], [5] * 90, [6] * 40]
+    lens = [40, 10, 25, 6, 12]
+
+    def run(ahead):
+        eng = AheadEngine(pages=64, max_num_seqs=3, max_num_batched_tokens=24, prefill_chunk=16)
+        s = Scheduler(eng)
+        s.sampler = AheadSampler(s)
+        s.lookahead = ahead
+        ids = [s.add_request(p, n) for p, n in zip(prompts, lens)]
+        out = s.run()
+        eng.cache.check_invariants()
+        assert eng.cache.free_pages() == 64
+        return eng, [out[i] for i in ids]
+
+    eng0, plain = run(False)
+    eng1, ahead = run(True)
+    assert ahead == plain == [expected(p, n) for p, n in zip(prompts, lens)]
+    assert eng1.mixed_ahead_steps >= 10
+    for step in eng1.steps:   # the budget and the number of requests hold in steps that ran ahead as well
+        assert sum(n for _, n, _ in step) <= 24 and len(step) <= 3
+    for rid, (p, g) in enumerate(zip(prompts, ahead)):
+        assert eng1.fed[rid] == p + g[:-1]   # no end token here: nothing surplus
+
+
+@pytest.mark.parametrize("seed", range(12))
 @pytest.mark.parametrize("ahead", [False, True])
 def test_random_workloads_give_every_request_its_own_tokens(seed, ahead):
     """Random prompts, lengths and end tokens, requests arriving while others run, a pool
