@@ -251,15 +251,25 @@ def test_cli_generates(model_dirs, tmp_path, capsys):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_running_one_step_ahead_changes_no_token(dtype, model_dirs):
     """Staggered requests of different lengths, some sampled with a temperature, one
-    ending early by its end-of-sequence token, on few pages: the tokens with decode steps
-    put on the device one step ahead (tokens fed there) are those of a scheduler that
-    waits for every step."""
+    ending early by its end-of-sequence token, on few pages: the tokens with steps put on
+    the device one step ahead (tokens fed there), prompt portions and admissions among
+    them, are those of a scheduler that waits for every step."""
     from pyre_amd.api import Scheduler
 
     eng = _load(model_dirs["tiny-c"], dtype, use_graphs=True, max_cached_tokens=640)
     vocab = eng.vocab_size
     prompts = [random_ids(vocab, n, seed=100 + n) for n in (5, 40, 17, 64, 9, 33)]
     lens = [30, 12, 44, 20, 37, 25]
+
+    mixed_ahead = [0]
+    real_step = eng.step
+
+    def counting_step(entries, fed_ids=None):
+        # a step that ran ahead (a token fed on the device) and carries a prompt portion too
+        mixed_ahead[0] += any(e.feed is not None for e in entries) and any(len(e.tokens) > 1 for e in entries)
+        return real_step(entries, fed_ids=fed_ids)
+
+    eng.step = counting_step
 
     def run(ahead, eos):
         s = Scheduler(eng, max_batch=4)
@@ -276,8 +286,10 @@ def test_running_one_step_ahead_changes_no_token(dtype, model_dirs):
     base, _ = run(False, None)
     eos = base[2][10]                     # request 2 will now end at the first occurrence of this token
     want, s0 = run(False, eos)
+    assert mixed_ahead[0] == 0
     got, s1 = run(True, eos)
     assert got == want
+    assert mixed_ahead[0] >= 3            # prompts in portions of 32 rode in steps that ran ahead
     assert len(want[2]) <= 11 and want[2][-1] == eos
     assert s1.lookahead and not s0.lookahead
     # the steps that ran ahead are fewer host round trips, not fewer engine steps
