@@ -6,9 +6,9 @@
 // all rows of X of a step against 64 rows of W and splits k over blocks instead.
 //
 // The product is computed transposed, out^T = W X^T, on MFMA 32x32x16: A = 32 rows of W, B = 32
-// rows of X, both read along k as they are stored. A block owns 64 RW rows of W and BM = 128 or
-// 256 rows of X: RW groups of XW = 4 multiplying waves (a group on 64 rows of W, its wave q on the
-// rows 32 CW q .. of X, CW = 1 or 2 tiles, against both tiles of W) and some waves that only
+// rows of X, both read along k as they are stored. A block owns 64 RW rows of W and BM = 128, 192
+// or 256 rows of X: RW groups of XW = 3 or 4 multiplying waves (a group on 64 rows of W, its wave q
+// on the rows 32 CW q .. of X, CW = 1 or 2 tiles, against both tiles of W) and some waves that only
 // load. k is walked in stages of 64 through a ring in LDS that is filled by loads from memory
 // straight into LDS, S - 1 stages ahead; a stage holds its rows as 128-byte rows whose eight
 // 16-byte pieces are exchanged among themselves by the row's number, so that the operand reads
@@ -257,8 +257,11 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
   const dim3 grid((N + BN - 1) / BN, ksplit);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
-  if (M > 128) {
+  if (M > 192) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 1, kPartials, 6, 3>), grid, dim3(64 * 10), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+  } else if (M > 128) {
+    hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 1, kPartials, 6, 4>), grid, dim3(64 * 9), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
   } else {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 1, kPartials, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
@@ -269,7 +272,10 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
 
 // W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
 // A block takes 64 features (64 gate rows and 64 up rows, eight multiplying waves), or 96 with
-// twelve for up to 128 rows of X where one round of blocks would not hold them otherwise.
+// twelve for up to 128 rows of X where one round of blocks would not hold them otherwise. The
+// rows of X that a block multiplies are 64, 96 (with 96 features), 128, 192 or 256, whichever
+// holds M: fewer rows are fewer multiplying waves, fewer loads and a deeper ring (measured on the
+// 7B shape, weights from memory: 49 us at 64 rows, 57 at 96, 63 at 128).
 namespace {
 int silu_features(int M, int two_i) { return M <= 128 && (two_i / 2 + 63) / 64 > 256 ? 96 : 64; }
 }  // namespace
@@ -287,8 +293,20 @@ extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, l
   const dim3 grid(pyre_gemm_mid_silu_blocks(M, two_i), 1);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
-  if (M > 128) {
+  if (M > 192) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 2, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M > 128) {
+    hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 2, kSiluMul, 8, 3>), grid, dim3(64 * 14), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 64 && silu_features(M, two_i) == 96) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 3, kSiluMul, 8, 4>), grid, dim3(64 * 14), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 64) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 2, kSiluMul, 8, 5>), grid, dim3(64 * 12), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 96 && silu_features(M, two_i) == 96) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 3, 3, kSiluMul, 6, 4>), grid, dim3(64 * 15), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else if (silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 3, kSiluMul, 4, 3>), grid, dim3(64 * 16), 0, stream, x,

@@ -138,7 +138,7 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
     if ctx.runtime.options.get("mid_silu_min_rows", MID_SILU_MIN_ROWS) <= n <= MID_MAX_ROWS:
         # blocks of 64 features (96 where that is what it takes, up to 128 rows) against all rows,
         # where one round of blocks holds them. Measured on the 1.5B shape: 17 us against the
-        # library's product and the SiLU-gate kernel's 29 at 65 to 128 rows, 28 against 30 at 256;
+        # library's product and the SiLU-gate kernel's 29 at 65 to 128 rows, 26 against 30 at 192, 28 at 256;
         # on the 7B shape 55 against 66 at 128, and at 256 rows, as on the 32B shape, two rounds of
         # blocks: those stay with the library. In a decode step of the 7B shape it is ahead of the
         # weight-streaming kernel from 48 rows on (5.40 against 5.47 ms a step at 48, 5.97 against
