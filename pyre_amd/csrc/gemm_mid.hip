@@ -263,6 +263,12 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
   } else if (M > 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 1, kPartials, 6, 4>), grid, dim3(64 * 9), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+  } else if (M <= 32) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 1, kPartials, 8, 6>), grid, dim3(64 * 9), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+  } else if (M <= 64) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 1, kPartials, 8, 5>), grid, dim3(64 * 10), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
   } else {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 1, kPartials, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
@@ -298,6 +304,12 @@ extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, l
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else if (M > 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 2, kSiluMul, 8, 3>), grid, dim3(64 * 14), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 32 && silu_features(M, two_i) == 96) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 3, kSiluMul, 8, 5>), grid, dim3(64 * 11), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 32) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 2, kSiluMul, 8, 6>), grid, dim3(64 * 10), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else if (M <= 64 && silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 3, kSiluMul, 8, 4>), grid, dim3(64 * 14), 0, stream, x,

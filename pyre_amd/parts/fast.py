@@ -19,13 +19,14 @@ from pyre_amd.hip.ops import Partials
 SKINNY_MAX_ROWS = 64
 #: the most partial sums of a weight-streaming product
 SKINNY_MAX_KSPLIT = 12
-#: up to this many rows the gate/up product and the SiLU-gate are one weight-streaming kernel
+#: up to this many rows the gate/up product and the SiLU-gate can be one weight-streaming kernel
+#: (shapes whose features one round of the other kernel's blocks does not hold: the 32B shape's)
 FUSED_SILU_MAX_ROWS = 64
 #: most rows of the kernel between the two, which keeps a step's rows against 64 rows of the weights
 MID_MAX_ROWS = 256
 MID_MAX_KSPLIT = 12
 #: fewest rows at which that kernel takes the gate/up product with the SiLU-gate
-MID_SILU_MIN_ROWS = 33
+MID_SILU_MIN_ROWS = 1
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
@@ -92,6 +93,15 @@ def linear(lin, ctx, x, n, out):
     skinny = rt.options.get("skinny_gemm", True) and ops.gemm_skinny_supports(
         min(n, SKINNY_MAX_ROWS), n_out, k, x.stride(0), lin.weight.stride(0))
     library = rt.options.get("library_gemm", True)
+    mid_from = SKINNY_MAX_ROWS + 1
+    if skinny and out is None and n <= SKINNY_MAX_ROWS and rt.options.get("mid_gemm", True) and mid_ksplit(n_out, k):
+        # A product so small that the weight-streaming kernel's blocks do not fill the compute units
+        # (the 1.5B shape's: 96, 72 and 240 blocks) is latency all the way, and the other kernel,
+        # whose loads go straight into a ring in LDS, starts sooner: 1.7 % of a step of 8 requests
+        # of that shape, 3 % at 32, 4 % at 64. Where the blocks fill the chip (7B: 504) it is 3 %
+        # slower at 8 rows and the same at 33 to 64.
+        if -(-n_out // 64) * skinny_ksplit(n, n_out, k) < 256 and rt.options.get("mid_small", True):
+            skinny, mid_from = False, 1
     if skinny and (n <= SKINNY_MAX_ROWS or (out is not None and not library)):
         if out is not None:
             # float32 results wanted in place (the head's logits): no split, 64 rows at a time
@@ -104,7 +114,7 @@ def linear(lin, ctx, x, n, out):
         ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
         return Partials(buf, lin.bias)
     mid = rt.options.get("mid_gemm", True)
-    if out is None and SKINNY_MAX_ROWS < n <= MID_MAX_ROWS and mid:
+    if out is None and mid_from <= n <= MID_MAX_ROWS and mid:
         ks = mid_ksplit(n_out, k)
         if not ks and int(mid) == 2:  # tests: also where it does not pay, as with a tiny model
             ks = 2 if k > 64 else 1
@@ -129,8 +139,9 @@ def linear(lin, ctx, x, n, out):
 
 
 def gate_up_silu(lin, ctx, x, n, act) -> bool:
-    """silu(x gate^T) * (x up^T) in one kernel: the weight-streaming kernel for a decode step's few
-    rows, the kernel that keeps all rows in a block for 33 to 256 where it pays."""
+    """silu(x gate^T) * (x up^T) in one kernel: the kernel that keeps all rows in a block for up to
+    256 rows where one round of blocks holds the features, else the weight-streaming kernel for a
+    decode step's few rows."""
     from pyre_amd.hip import ops
 
     if not _is_bf16(ctx, lin, x) or lin.bias is not None:
@@ -140,9 +151,10 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
         # where one round of blocks holds them. Measured on the 1.5B shape: 17 us against the
         # library's product and the SiLU-gate kernel's 29 at 65 to 128 rows, 26 against 30 at 192, 28 at 256;
         # on the 7B shape 55 against 66 at 128, and at 256 rows, as on the 32B shape, two rounds of
-        # blocks: those stay with the library. In a decode step of the 7B shape it is ahead of the
-        # weight-streaming kernel from 48 rows on (5.40 against 5.47 ms a step at 48, 5.97 against
-        # 6.13 at 64; at 32 rows 4.69 against 4.64), on the 1.5B shape by 2 % from 24 rows on.
+        # blocks: those stay with the library. With blocks of 32 and 64 rows of X for steps that
+        # small it is ahead of the weight-streaming kernel at every size: on the 7B shape 3.20
+        # against 3.23 ms a step at one request, 3.44 against 3.49 at 8, 3.77 against 3.87 at 16,
+        # 4.46 against 4.56 at 32, 5.87 against 6.13 at 64; on the 1.5B shape by 1 to 4 %.
         mid = ctx.runtime.options.get("mid_gemm", True)
         fits = mid and ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0))
         if fits and (ops.gemm_mid_silu_blocks(n, lin.out_features) <= 256 or int(mid) == 2):

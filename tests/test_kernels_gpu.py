@@ -805,7 +805,7 @@ def test_gemm_skinny(m, n, k, ksplit):
     assert torch.allclose(out.double().sum(0), want, atol=1e-3 * math.sqrt(k), rtol=1e-4)
 
 
-@pytest.mark.parametrize("m", [1, 65, 100, 128, 129, 192, 193, 256])
+@pytest.mark.parametrize("m", [1, 32, 33, 64, 65, 100, 128, 129, 192, 193, 256])
 @pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (1536, 1536, 6), (1000, 136, 2), (131, 8, 1), (3584, 18944, 4),
                                         (2048, 1000, 3), (70, 4096, 10)])
 def test_gemm_mid(m, n, k, ksplit):
@@ -831,7 +831,7 @@ def test_gemm_mid(m, n, k, ksplit):
     assert torch.equal(again, out)
 
 
-@pytest.mark.parametrize("m", [33, 64, 65, 96, 97, 128, 129, 192, 193, 256])
+@pytest.mark.parametrize("m", [1, 8, 32, 33, 64, 65, 96, 97, 128, 129, 192, 193, 256])
 @pytest.mark.parametrize("inter,k", [(176, 64), (8960, 1536), (250, 96), (70, 520), (18944, 136), (16401, 64)])
 def test_gemm_mid_silu(m, inter, k):
     """Blocks of 64 features, and of 96 for up to 128 rows where 64 would make more than 256

@@ -136,13 +136,16 @@ def test_mixed_with_page_reuse(model, dtype, page, engines, plain_models):
     assert eng.cache.page_groups[0].allocator.num_used == 0
 
 
-@pytest.mark.parametrize("model,dtype,graphs", [("tiny-c", "bfloat16", True), ("tiny-c", "bfloat16", False),
-                                                ("tiny-c", "float32", True), ("tiny-b", "bfloat16", True),
-                                                ("tiny-d", "float32", True)])
-def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_models):
+@pytest.mark.parametrize("model,dtype,graphs,mid", [
+    ("tiny-c", "bfloat16", True, 1), ("tiny-c", "bfloat16", False, 1), ("tiny-c", "float32", True, 1),
+    ("tiny-b", "bfloat16", True, 1), ("tiny-d", "float32", True, 1), ("tiny-c", "bfloat16", True, 0),
+    ("tiny-b", "bfloat16", False, 0)])
+def test_decode_steps_of_many_requests(model, dtype, graphs, mid, model_dirs, plain_models):
     """64 live requests, one token each per step, shrinking to 49, 33, 24 and 17 as requests
     end: every row of every step against the plain implementation. Captured steps run at
-    padded sizes (49 as 64, 33 as 48, 17 as 24); their padding rows must change nothing."""
+    padded sizes (49 as 64, 33 as 48, 17 as 24); their padding rows must change nothing.
+    ``mid = 0``: all products of these steps in the weight-streaming kernels, which otherwise
+    leave the gate/up product of a model this small to the kernel that keeps all rows in a block."""
     plain = plain_models[model]
     vocab = plain[0]["vocab_size"]
     prompt = [2 + (13 * i) % 61 for i in range(64)]                 # 2 to 62 tokens: page ends fall everywhere
@@ -150,6 +153,7 @@ def test_decode_steps_of_many_requests(model, dtype, graphs, model_dirs, plain_m
     want = _expected(plain, reqs, dtype)
     eng = make_engine(model_dirs[model], dtype, use_graphs=graphs, max_num_seqs=64, max_cached_tokens=64 * 80,
                       max_num_batched_tokens=1024)
+    eng.runtime.options["mid_gemm"] = mid
     steps = [([(i, reqs[i][:prompt[i]], [prompt[i] - 1]) for i in range(lo, min(lo + 16, 64))], []) for lo in range(0, 64, 16)]
     live = list(range(64))
     for k, keep in enumerate((64, 64, 64, 49, 49, 33, 33, 24, 17, 17)):
