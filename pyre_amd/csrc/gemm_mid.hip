@@ -1,13 +1,13 @@
-// out[m, n] = sum_k X[m, k] W[n, k] for 65 to 256 rows of X in bfloat16: the matrix products of
-// a decode step of many requests (pyre/model.py:315-319,338-342 at the batch sizes of
-// pyre/scheduler.py), where every weight is still read once but the arithmetic is no longer
+// out[m, n] = sum_k X[m, k] W[n, k] for up to 256 rows of X in bfloat16: the matrix products of
+// a decode step (pyre/model.py:315-319,338-342 at the batch sizes of pyre/scheduler.py), above all
+// of many requests, where every weight is still read once but the arithmetic is no longer
 // free. For products with few output columns (q/k/v, the attention output, the feed-forward's
 // way down) the BLAS library's kernels take 19 us or more whatever the size; this kernel keeps
 // all rows of X of a step against 64 rows of W and splits k over blocks instead.
 //
 // The product is computed transposed, out^T = W X^T, on MFMA 32x32x16: A = 32 rows of W, B = 32
-// rows of X, both read along k as they are stored. A block owns 64 RW rows of W and BM = 128, 192
-// or 256 rows of X: RW groups of XW = 3 or 4 multiplying waves (a group on 64 rows of W, its wave q
+// rows of X, both read along k as they are stored. A block owns 64 RW rows of W and BM = 32 to 256
+// rows of X: RW groups of XW = 1 to 4 multiplying waves (a group on 64 rows of W, its wave q
 // on the rows 32 CW q .. of X, CW = 1 or 2 tiles, against both tiles of W) and some waves that only
 // load. k is walked in stages of 64 through a ring in LDS that is filled by loads from memory
 // straight into LDS, S - 1 stages ahead; a stage holds its rows as 128-byte rows whose eight

@@ -14,8 +14,8 @@ import torch
 
 from pyre_amd.hip.ops import Partials
 
-#: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the kernel for 65 to
-#: 256 rows where it pays and else to the BLAS library
+#: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the kernel that keeps
+#: up to 256 rows in a block where it pays and else to the BLAS library
 SKINNY_MAX_ROWS = 64
 #: the most partial sums of a weight-streaming product
 SKINNY_MAX_KSPLIT = 12
@@ -57,8 +57,8 @@ def skinny_ksplit(m: int, n_out: int, k: int) -> int:
 
 
 def mid_ksplit(n_out: int, k: int) -> int:
-    """Into how many parts of k the kernel for 65 to 256 rows splits a product, or 0 if it is not
-    the one to take. A block has 64 rows of the weights; the kernel is at its best when the blocks
+    """Into how many parts of k the kernel that keeps a step's rows in a block (up to 256) splits a
+    product, or 0 if it is not the one to take. A block has 64 rows of the weights; the kernel is at its best when the blocks
     of all parts fill the 256 compute units in one round, and beats the BLAS library where that
     takes at least two parts of 384 k or more (shorter parts gain nothing and cost the consumer
     another addend; measured on the 1.5B, 7B and 32B shapes: q/k/v, the

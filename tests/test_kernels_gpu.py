@@ -809,7 +809,7 @@ def test_gemm_skinny(m, n, k, ksplit):
 @pytest.mark.parametrize("n,k,ksplit", [(48, 64, 1), (1536, 1536, 6), (1000, 136, 2), (131, 8, 1), (3584, 18944, 4),
                                         (2048, 1000, 3), (70, 4096, 10)])
 def test_gemm_mid(m, n, k, ksplit):
-    """The products of a decode step of 65 to 256 rows: sizes that are no multiple of the tiles
+    """The products of a decode step of up to 256 rows: sizes that are no multiple of the tiles
     (64 rows of the weights, 32 of the input, stages of 64 k), k in parts; and a row's result is
     bit for bit the same whatever rows share the step and however many they are."""
     ops = _ops()

@@ -181,7 +181,7 @@ def test_workspace_hands_out_the_same_memory_until_a_buffer_grows():
 
 
 def test_mid_ksplit_fills_one_round_and_leaves_no_part_empty():
-    """The kernel for 65 to 256 rows is chosen where at least two parts of 384 k or more fill the
+    """The kernel that keeps up to 256 rows in a block is chosen where at least two parts of 384 k or more fill the
     256 compute units in one round of blocks of 64 output columns."""
     from pyre_amd.parts.fast import MID_MAX_KSPLIT, mid_ksplit
 

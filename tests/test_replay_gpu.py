@@ -248,7 +248,7 @@ def test_decode_steps_of_requests_of_very_different_lengths(others, graphs, mode
                                                     ("tiny-a", "bfloat16", False, 2)])
 def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, mid, model_dirs, plain_models):
     """200, 150, 100 and 70 live requests: decode steps whose products go to the BLAS library
-    (more than 64 rows) or, with mid = 2, all to the kernel for 65 to 256 rows, which a tiny
+    (more than 64 rows) or, with mid = 2, all to the kernel that keeps a step's rows in a block, which a tiny
     model's sizes would not choose; captured at 256, 192, 128 and 96 rows and replayed several
     times, each replay against the plain implementation (a library call that records a clearing
     of memory into the graph would be right once and wrong afterwards)."""
