@@ -122,3 +122,49 @@ def test_captured_decode_steps_with_library_products_at_the_7b_shape(layers_7b):
     assert len(got) == 600 and eng.graph_replays == 5
     bad, worst = first_bad(got, want, TOL["bfloat16"])
     assert bad is None, bad
+
+
+def test_decode_steps_of_few_requests_at_the_1p5b_shape():
+    """Two layers of the Qwen2.5-1.5B shape (width 1536, 12 query / 2 key-value heads, feed-forward
+    8960, tied head): its products are so small that the weight-streaming kernel's blocks would
+    not fill the chip, and the kernel that keeps the step's rows in a block takes them at every
+    size, in blocks of 32 and 64 rows. Steps of 40, 8 and 1 requests from HIP graphs, twice."""
+    from pyre_amd.config import preset
+    from pyre_amd.parts.fast import mid_ksplit, skinny_ksplit
+    from pyre_amd.weights import model_tensor_specs, random_state
+
+    cfg = preset("qwen2.5-1.5b", num_hidden_layers=2)
+    h, inter = cfg.hidden_size, cfg.intermediate_size
+    for n_out, k in ((h + 2 * cfg.num_key_value_heads * cfg.head_dim, h), (h, h), (h, inter)):
+        assert mid_ksplit(n_out, k) and -(-n_out // 64) * skinny_ksplit(8, n_out, k) < 256   # the rule of parts/fast.py
+    state = random_state(model_tensor_specs(cfg), seed=6, std=0.02, gain_std=0.1, dtype="bfloat16", device=DEV)
+    plain_cfg = {k: getattr(cfg, k) for k in ("hidden_size", "intermediate_size", "num_hidden_layers",
+                                              "num_attention_heads", "num_key_value_heads", "vocab_size",
+                                              "rms_norm_eps", "rope_theta", "tie_word_embeddings", "head_dim")}
+    plain = (plain_cfg, {n: t.to(torch.float64) for n, t in state.items()})
+    plain[1].setdefault("lm_head.weight", plain[1]["model.embed_tokens.weight"])    # the tied head, as the plain loader has it
+    vocab = cfg.vocab_size
+    lengths = [4 + (11 * i) % 27 for i in range(40)]
+    reqs = {i: random_ids(vocab, n + 6, 700 + i) for i, n in enumerate(lengths)}
+    want = _want(plain, reqs, "bfloat16")
+    eng = make_engine_from_state(cfg, state, "bfloat16", use_graphs=True, max_cached_tokens=40 * 48, max_num_seqs=40,
+                                 max_num_batched_tokens=2048)
+    steps = [([(i, reqs[i][:lengths[i]], []) for i in range(40)], [])]
+    live = list(range(40))
+    for k, keep in enumerate((40, 40, 8, 8, 1, 1)):
+        live = live[:keep]
+        steps.append(([(i, [reqs[i][lengths[i] + k]], [0]) for i in live], []))
+    got = replay(eng, steps)
+    assert len(got) == 2 * (40 + 8 + 1) and eng.graph_replays == 3
+    bad, worst = first_bad(got, want, TOL["bfloat16"])
+    assert bad is None, bad
+    # the same steps with the weight-streaming kernel for the narrow products, run eagerly
+    eng2 = make_engine_from_state(cfg, state, "bfloat16", use_graphs=False, max_cached_tokens=40 * 48, max_num_seqs=40,
+                                  max_num_batched_tokens=2048)
+    eng2.runtime.options["mid_small"] = False
+    got2 = replay(eng2, steps)
+    bad, worst = first_bad(got2, want, TOL["bfloat16"])
+    assert bad is None, bad
+    plain[1].clear()
+    state.clear()
+    torch.cuda.empty_cache()
