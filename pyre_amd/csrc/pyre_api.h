@@ -66,11 +66,11 @@ int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw,
                                int two_i, int K, hipStream_t stream);
 
 // The first of them for up to 256 rows (a decode step of many requests), for products with few
-// output columns: a block keeps all rows of X against 64 rows of W, and ksplit blocks share
-// them. out: float32 [ksplit][M][N].
+// output columns: a block keeps all rows of X against 64 rows of W (128 with `wide`, for up to 64
+// rows of X), and ksplit blocks share them. out: float32 [ksplit][M][N].
 int pyre_gemm_mid_supports(int M, int N, int K, long ldx, long ldw);
 int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N, int K,
-                       int ksplit, hipStream_t stream);
+                       int ksplit, int wide, hipStream_t stream);
 // The second of them for up to 256 rows: a block takes 64 or 96 features (pyre_gemm_mid_silu_blocks
 // blocks in all) against all rows of X; it pays where one round of blocks holds them.
 int pyre_gemm_mid_silu_blocks(int M, int two_i);

@@ -10,7 +10,7 @@ char* error_buffer() {
 }  // namespace pyre
 
 extern "C" const char* pyre_last_error() { return pyre::error_buffer(); }
-extern "C" int pyre_abi_version() { return 13; }
+extern "C" int pyre_abi_version() { return 14; }
 
 // ---------------------------------------------------------------------------
 // A plain streaming read of `bytes` (a multiple of 16) for measuring what the

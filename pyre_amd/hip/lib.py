@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 
 class KernelError(RuntimeError):
@@ -44,7 +44,7 @@ _SIGNATURES = {
     "pyre_gemm_skinny_bf16": [P, L, P, L, P, I, I, I, I, P],
     "pyre_gemm_skinny_silu_bf16": [P, L, P, L, P, I, I, I, P],
     "pyre_gemm_mid_supports": [I, I, I, L, L],
-    "pyre_gemm_mid_bf16": [P, L, P, L, P, I, I, I, I, P],
+    "pyre_gemm_mid_bf16": [P, L, P, L, P, I, I, I, I, I, P],
     "pyre_gemm_mid_silu_blocks": [I, I],
     "pyre_gemm_mid_silu_bf16": [P, L, P, L, P, I, I, I, P],
     "pyre_sample": [P, L, P, P, P, I, I, P],

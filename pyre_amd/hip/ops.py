@@ -543,14 +543,15 @@ def gemm_mid_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
     return bool(lib().pyre_gemm_mid_supports(m, n, k, ldx, ldw))
 
 
-def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int) -> None:
-    """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 256."""
+def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int, wide: bool = False) -> None:
+    """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 256. ``wide``
+    (m <= 64): a block takes 128 rows of w instead of 64."""
     _skinny_common(x, w, m)
     n = w.shape[0]
     if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() < ksplit * m * n or not out.is_cuda:
         raise KernelError("gemm_mid: out must be contiguous float32 [ksplit, m, N] on the GPU")
     call("pyre_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), m, n,
-         w.shape[1], ksplit, _stream())
+         w.shape[1], ksplit, int(wide), _stream())
 
 
 def gemm_mid_silu_blocks(m: int, two_i: int) -> int:

@@ -27,6 +27,9 @@ MID_MAX_ROWS = 256
 MID_MAX_KSPLIT = 12
 #: fewest rows at which that kernel takes the gate/up product with the SiLU-gate
 MID_SILU_MIN_ROWS = 1
+#: fewest rows at which its form with 128 rows of the weights a block takes a narrow product
+#: (just above a size at which decode steps are captured, so that an eager step and its replay agree)
+MID_WIDE_MIN_ROWS = 25
 
 
 def skinny_ksplit(m: int, n_out: int, k: int) -> int:
@@ -56,7 +59,7 @@ def skinny_ksplit(m: int, n_out: int, k: int) -> int:
     return best
 
 
-def mid_ksplit(n_out: int, k: int) -> int:
+def mid_ksplit(n_out: int, k: int, block_rows: int = 64) -> int:
     """Into how many parts of k the kernel that keeps a step's rows in a block (up to 256) splits a
     product, or 0 if it is not the one to take. A block has 64 rows of the weights; the kernel is at its best when the blocks
     of all parts fill the 256 compute units in one round, and beats the BLAS library where that
@@ -64,7 +67,7 @@ def mid_ksplit(n_out: int, k: int) -> int:
     another addend; measured on the 1.5B, 7B and 32B shapes: q/k/v, the
     attention output and the feed-forward's way down take 9 to 20 us where the library takes 19
     to 31, and 60 against 100 at 7B's way down; the wide gate/up product stays with the library)."""
-    blocks = -(-n_out // 64)
+    blocks = -(-n_out // block_rows)
     ks = min(256 // blocks, k // 384, MID_MAX_KSPLIT)
     while ks > 1 and (ks - 1) * (-(-(-(-k // ks)) // 64) * 64) >= k:
         ks -= 1  # would leave a part empty
@@ -83,6 +86,45 @@ def _is_bf16(ctx, lin, x) -> bool:
             and x.dtype == torch.bfloat16)
 
 
+def narrow_kernel(n: int, n_out: int, k: int, options: dict | None = None) -> tuple[str, int, bool]:
+    """Which of our kernels takes a 16-bit product of ``n`` rows whose result is handed on as partial
+    sums: ("stream", parts of k, False) for the weight-streaming kernel, ("block", parts, wide) for the
+    kernel that keeps the step's rows in a block (``wide``: 128 rows of the weights a block instead
+    of 64), ("", 0, False) for neither (the BLAS library then). A function of the sizes alone; the
+    thresholds in rows lie just above sizes at which decode steps are captured, so that an eager step
+    and its replay at the padded size agree."""
+    opt = options or {}
+    block = opt.get("mid_gemm", True)
+    if n <= SKINNY_MAX_ROWS and opt.get("skinny_gemm", True):
+        if block and n >= opt.get("mid_wide_min_rows", MID_WIDE_MIN_ROWS):
+            # From 25 rows on the weight-streaming kernel slows down (64 activations come from L2
+            # once per 128 rows of weights, and four times the LDS reads and MFMAs sit between a
+            # run's arrival and the next run's request); the kernel with a ring in LDS and 128
+            # rows of the weights a block does not, where its blocks fill three quarters of the
+            # chip at least. Measured in steps of the 7B shape: 4.43 against 4.47 ms at 32
+            # requests, 5.20 against 5.29 at 48, 5.74 against 5.88 at 64 (at 8 and 16: 3.46 against
+            # 3.44, 3.79 against 3.77); of the 32B shape 35.5 against 36.2 at 64.
+            ks = mid_ksplit(n_out, k, 128)
+            if ks and -(-n_out // 128) * ks >= 192:
+                return "block", ks, True
+        ks = skinny_ksplit(n, n_out, k)
+        if block and opt.get("mid_small", True) and -(-n_out // 64) * ks < 256 and mid_ksplit(n_out, k):
+            # A product so small that the weight-streaming kernel's blocks do not fill the compute
+            # units (the 1.5B shape's: 96, 72 and 240 blocks) is latency all the way, and the other
+            # kernel, whose loads go straight into a ring in LDS, starts sooner: 1.7 % of a step of
+            # 8 requests of that shape, 3 % at 32, 4 % at 64. Where the blocks fill the chip (7B:
+            # 504) it is 3 % slower at 8 rows.
+            return "block", mid_ksplit(n_out, k), False
+        return "stream", ks, False
+    if n <= MID_MAX_ROWS and block:
+        ks = mid_ksplit(n_out, k)
+        if not ks and int(block) == 2:  # tests: also where it does not pay, as with a tiny model
+            ks = 2 if k > 64 else 1
+        if ks:
+            return "block", ks, False
+    return "", 0, False
+
+
 def linear(lin, ctx, x, n, out):
     from pyre_amd.hip import ops
 
@@ -90,45 +132,34 @@ def linear(lin, ctx, x, n, out):
     if not _is_bf16(ctx, lin, x):
         return None
     k, n_out = lin.in_features, lin.out_features
-    skinny = rt.options.get("skinny_gemm", True) and ops.gemm_skinny_supports(
+    streams = rt.options.get("skinny_gemm", True) and ops.gemm_skinny_supports(
         min(n, SKINNY_MAX_ROWS), n_out, k, x.stride(0), lin.weight.stride(0))
     library = rt.options.get("library_gemm", True)
-    mid_from = SKINNY_MAX_ROWS + 1
-    if skinny and out is None and n <= SKINNY_MAX_ROWS and rt.options.get("mid_gemm", True) and mid_ksplit(n_out, k):
-        # A product so small that the weight-streaming kernel's blocks do not fill the compute units
-        # (the 1.5B shape's: 96, 72 and 240 blocks) is latency all the way, and the other kernel,
-        # whose loads go straight into a ring in LDS, starts sooner: 1.7 % of a step of 8 requests
-        # of that shape, 3 % at 32, 4 % at 64. Where the blocks fill the chip (7B: 504) it is 3 %
-        # slower at 8 rows and the same at 33 to 64.
-        if -(-n_out // 64) * skinny_ksplit(n, n_out, k) < 256 and rt.options.get("mid_small", True):
-            skinny, mid_from = False, 1
-    if skinny and (n <= SKINNY_MAX_ROWS or (out is not None and not library)):
-        if out is not None:
-            # float32 results wanted in place (the head's logits): no split, 64 rows at a time
+    if out is not None:
+        # float32 results wanted in place (the head's logits)
+        if streams and (n <= SKINNY_MAX_ROWS or not library):  # no split, 64 rows at a time
             for r0 in range(0, n, SKINNY_MAX_ROWS):
                 rows = min(SKINNY_MAX_ROWS, n - r0)
                 ops.gemm_skinny_bf16(x[r0:r0 + rows], lin.weight, out[r0:r0 + rows], rows, 1)
-            return Partials(out.view(1, n, n_out), lin.bias)
-        ks = skinny_ksplit(n, n_out, k)
+        elif library:  # many rows (a large decode step, or every row of a portion): one pass over the weights
+            torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out_dtype=torch.float32, out=out)
+        else:
+            return None
+        return Partials(out.view(1, n, n_out), lin.bias)
+    kernel, ks, wide = narrow_kernel(n, n_out, k, rt.options)
+    if kernel == "stream" and not streams:
+        kernel = ""
+    if kernel == "block" and not ops.gemm_mid_supports(n, n_out, k, x.stride(0), lin.weight.stride(0)):
+        kernel, ks = ("stream", skinny_ksplit(n, n_out, k)) if streams and n <= SKINNY_MAX_ROWS else ("", 0)
+    if kernel:
         buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
-        ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
+        if kernel == "stream":
+            ops.gemm_skinny_bf16(x, lin.weight, buf, n, ks)
+        else:
+            ops.gemm_mid_bf16(x, lin.weight, buf, n, ks, wide=wide)
         return Partials(buf, lin.bias)
-    mid = rt.options.get("mid_gemm", True)
-    if out is None and mid_from <= n <= MID_MAX_ROWS and mid:
-        ks = mid_ksplit(n_out, k)
-        if not ks and int(mid) == 2:  # tests: also where it does not pay, as with a tiny model
-            ks = 2 if k > 64 else 1
-        if ks and ops.gemm_mid_supports(n, n_out, k, x.stride(0), lin.weight.stride(0)):
-            buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
-            ops.gemm_mid_bf16(x, lin.weight, buf, n, ks)
-            return Partials(buf, lin.bias)
     if not library:
         return None
-    if out is not None:
-        # many rows of float32 results in place (the head's logits of a large decode step, or of
-        # every row of a portion): one pass over the weights in the library
-        torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out_dtype=torch.float32, out=out)
-        return Partials(out.view(1, n, n_out), lin.bias)
     if lin.role in rt.options.get("library_f32_roles", LIBRARY_F32_ROLES):
         buf = ctx.workspace.get(f"linear32.{lin.role}", (n, n_out), torch.float32)
         torch.mm(x if n == x.shape[0] else x[:n], lin.weight.t(), out_dtype=torch.float32, out=buf)

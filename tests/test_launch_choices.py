@@ -195,3 +195,32 @@ def test_mid_ksplit_fills_one_round_and_leaves_no_part_empty():
                 blocks = -(-n_out // 64)
                 kper = -(-(-(-k // ks)) // 64) * 64
                 assert 2 <= ks <= MID_MAX_KSPLIT and blocks * ks <= 256 and k // ks >= 384 and (ks - 1) * kper < k
+
+
+def test_which_kernel_takes_a_product_is_a_function_of_its_sizes():
+    """The choice between the weight-streaming kernel, the kernel that keeps a step's rows in a
+    block (with 64 or 128 rows of the weights a block) and the BLAS library, for the shapes it was
+    measured on; within the row counts between two sizes at which decode steps are captured the
+    answer does not change, so that an eager step and its replay run the same kernels."""
+    from pyre_amd.engine.batch import DECODE_ROW_BUCKETS
+    from pyre_amd.parts.fast import MID_MAX_ROWS, narrow_kernel
+
+    qkv7, down7 = (4608, 3584), (3584, 18944)
+    assert narrow_kernel(8, *qkv7) == ("stream", 7, False) and narrow_kernel(24, *down7) == ("stream", 9, False)
+    assert narrow_kernel(25, *qkv7) == narrow_kernel(64, *qkv7) == ("block", 7, True)       # 36 x 7 blocks of 128 rows
+    assert narrow_kernel(48, *down7) == ("block", 9, True)
+    assert narrow_kernel(65, *qkv7) == narrow_kernel(256, *qkv7) == ("block", 3, False)     # 72 x 3 blocks of 64 rows
+    assert narrow_kernel(257, *qkv7) == ("", 0, False)
+    assert narrow_kernel(64, 5120, 27648) == ("block", 6, True)                             # the 32B shape's way down
+    # the 1.5B shape: too few blocks either way, the kernel with the ring in LDS from one row on
+    assert narrow_kernel(1, 2048, 1536) == narrow_kernel(64, 2048, 1536) == ("block", 4, False)
+    assert narrow_kernel(8, 1536, 8960) == ("block", 10, False)
+    assert narrow_kernel(8, 1536, 8960, {"mid_small": False})[0] == "stream"
+    # a tiny model: the weight-streaming kernel, then the library; for tests the other kernel if asked for
+    assert narrow_kernel(8, 96, 64)[0] == "stream" and narrow_kernel(100, 96, 64) == ("", 0, False)
+    assert narrow_kernel(100, 96, 64, {"mid_gemm": 2}) == ("block", 1, False)
+    assert narrow_kernel(8, *qkv7, {"mid_gemm": 0}) == ("stream", 7, False) and narrow_kernel(100, *qkv7, {"mid_gemm": 0})[0] == ""
+    edges = [0] + [b for b in DECODE_ROW_BUCKETS if b <= MID_MAX_ROWS]
+    for shape in (qkv7, down7, (3584, 3584), (2048, 1536), (1536, 8960), (7168, 5120), (5120, 27648), (96, 64), (1000, 4096)):
+        for lo, hi in zip(edges, edges[1:]):
+            assert len({narrow_kernel(n, *shape) for n in range(lo + 1, hi + 1)}) == 1, (shape, lo, hi)
