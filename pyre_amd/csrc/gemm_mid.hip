@@ -252,23 +252,32 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
                                   int K, int ksplit, int wide, hipStream_t stream) {
   if (int rc = check_mid("gemm_mid_bf16", X, W, M, N, K, ldx, ldw)) return rc;
   PYRE_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_mid_bf16: ksplit=%d", ksplit);
-  PYRE_REQUIRE(!wide || M <= 64, "gemm_mid_bf16: blocks of 128 rows of W take up to 64 rows of X, not %d", M);
   const int kper = ((K + ksplit - 1) / ksplit + BK - 1) / BK * BK;
   PYRE_REQUIRE(static_cast<long>(ksplit - 1) * kper < K, "gemm_mid_bf16: a part of k would be empty (K=%d, ksplit=%d)", K, ksplit);
   const dim3 grid((N + BN - 1) / BN, ksplit);
   const bf16* x = static_cast<const bf16*>(X);
   const bf16* w = static_cast<const bf16*>(W);
   if (wide) {
-    // Few rows of X: a stage's bytes are mostly W's, and with twice the rows of W a stage (and the
-    // barrier that goes with it) carries twice the bytes. Measured on the 7B shape's way down,
-    // weights from memory: 25.6 us at 64 rows of X where 64 rows of W a block take 29.8 and the
-    // weight-streaming kernel 31.9.
+    // Twice the rows of W a block, over half as much of k where the caller splits k further: a
+    // block's bytes (its rows of W and all rows of X, over its part of k) are fewest where the two
+    // are equally many, and at few rows of X a stage (and the barrier that goes with it) carries
+    // twice the bytes. Measured on the 7B shape's way down, weights from memory: 25.6 us at 64
+    // rows of X where 64 rows of W a block take 29.8 and the weight-streaming kernel 31.9.
     const dim3 grid2((N + 2 * BN - 1) / (2 * BN), ksplit);
     if (M <= 32) {
       hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 2, kPartials, 8, 6>), grid2, dim3(64 * 10), 0, stream, x,
                          static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
-    } else {
+    } else if (M <= 64) {
       hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 2, kPartials, 8, 5>), grid2, dim3(64 * 12), 0, stream, x,
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+    } else if (M <= 128) {
+      hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 2, kPartials, 8, 4>), grid2, dim3(64 * 16), 0, stream, x,
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+    } else if (M <= 192) {
+      hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 2, kPartials, 8, 3>), grid2, dim3(64 * 14), 0, stream, x,
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+    } else {
+      hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 2, kPartials, 8, 3>), grid2, dim3(64 * 16), 0, stream, x,
                          static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
     }
   } else if (M > 192) {

@@ -66,8 +66,8 @@ int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw,
                                int two_i, int K, hipStream_t stream);
 
 // The first of them for up to 256 rows (a decode step of many requests), for products with few
-// output columns: a block keeps all rows of X against 64 rows of W (128 with `wide`, for up to 64
-// rows of X), and ksplit blocks share them. out: float32 [ksplit][M][N].
+// output columns: a block keeps all rows of X against 64 rows of W (128 with `wide`), and ksplit
+// blocks share them. out: float32 [ksplit][M][N].
 int pyre_gemm_mid_supports(int M, int N, int K, long ldx, long ldw);
 int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N, int K,
                        int ksplit, int wide, hipStream_t stream);

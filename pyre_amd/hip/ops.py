@@ -544,8 +544,8 @@ def gemm_mid_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
 
 
 def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, ksplit: int, wide: bool = False) -> None:
-    """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 256. ``wide``
-    (m <= 64): a block takes 128 rows of w instead of 64."""
+    """out[s] (float32 [ksplit, m, N]) = partial sums over k of x[0:m] @ w.T, 1 <= m <= 256. ``wide``:
+    a block takes 128 rows of w instead of 64."""
     _skinny_common(x, w, m)
     n = w.shape[0]
     if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() < ksplit * m * n or not out.is_cuda:

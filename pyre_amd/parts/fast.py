@@ -95,18 +95,22 @@ def narrow_kernel(n: int, n_out: int, k: int, options: dict | None = None) -> tu
     and its replay at the padded size agree."""
     opt = options or {}
     block = opt.get("mid_gemm", True)
+    if block and opt.get("mid_wide_min_rows", MID_WIDE_MIN_ROWS) <= n <= MID_MAX_ROWS:
+        # With 128 rows of the weights a block, where such blocks fill three quarters of the chip at
+        # least: a block's bytes are the step's rows of X and its rows of W, over its part of k, and
+        # with as many of the one as of the other they are fewest (at few rows of X a stage, and the
+        # barrier that goes with it, carries twice the bytes). From 25 rows on the weight-streaming
+        # kernel slows down (64 activations come from L2 once per 128 rows of weights, and four
+        # times the LDS reads and MFMAs sit between a run's arrival and the next run's request),
+        # this one does not. Measured in steps of the 7B shape against the weight-streaming kernel:
+        # 4.43 against 4.47 ms at 32 requests, 5.20 against 5.29 at 48, 5.74 against 5.88 at 64 (at 8
+        # and 16: 3.46 against 3.44, 3.79 against 3.77); of the 32B shape 35.5 against 36.2 at 64.
+        # Against 64 rows of the weights a block: 7.78 against 7.94 ms at 96 requests, 8.86 against
+        # 8.90 at 128, 12.56 against 12.63 at 192, 15.25 against 15.34 at 256.
+        ks = mid_ksplit(n_out, k, 128)
+        if ks and -(-n_out // 128) * ks >= 192:
+            return "block", ks, True
     if n <= SKINNY_MAX_ROWS and opt.get("skinny_gemm", True):
-        if block and n >= opt.get("mid_wide_min_rows", MID_WIDE_MIN_ROWS):
-            # From 25 rows on the weight-streaming kernel slows down (64 activations come from L2
-            # once per 128 rows of weights, and four times the LDS reads and MFMAs sit between a
-            # run's arrival and the next run's request); the kernel with a ring in LDS and 128
-            # rows of the weights a block does not, where its blocks fill three quarters of the
-            # chip at least. Measured in steps of the 7B shape: 4.43 against 4.47 ms at 32
-            # requests, 5.20 against 5.29 at 48, 5.74 against 5.88 at 64 (at 8 and 16: 3.46 against
-            # 3.44, 3.79 against 3.77); of the 32B shape 35.5 against 36.2 at 64.
-            ks = mid_ksplit(n_out, k, 128)
-            if ks and -(-n_out // 128) * ks >= 192:
-                return "block", ks, True
         ks = skinny_ksplit(n, n_out, k)
         if block and opt.get("mid_small", True) and -(-n_out // 64) * ks < 256 and mid_ksplit(n_out, k):
             # A product so small that the weight-streaming kernel's blocks do not fill the compute

@@ -209,7 +209,8 @@ def test_which_kernel_takes_a_product_is_a_function_of_its_sizes():
     assert narrow_kernel(8, *qkv7) == ("stream", 7, False) and narrow_kernel(24, *down7) == ("stream", 9, False)
     assert narrow_kernel(25, *qkv7) == narrow_kernel(64, *qkv7) == ("block", 7, True)       # 36 x 7 blocks of 128 rows
     assert narrow_kernel(48, *down7) == ("block", 9, True)
-    assert narrow_kernel(65, *qkv7) == narrow_kernel(256, *qkv7) == ("block", 3, False)     # 72 x 3 blocks of 64 rows
+    assert narrow_kernel(65, *qkv7) == narrow_kernel(256, *qkv7) == ("block", 7, True)
+    assert narrow_kernel(65, 2048, 1536) == narrow_kernel(256, 2048, 1536) == ("block", 4, False)   # 32 x 4 blocks of 64 rows
     assert narrow_kernel(257, *qkv7) == ("", 0, False)
     assert narrow_kernel(64, 5120, 27648) == ("block", 6, True)                             # the 32B shape's way down
     # the 1.5B shape: too few blocks either way, the kernel with the ring in LDS from one row on
