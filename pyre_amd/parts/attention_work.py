@@ -19,6 +19,10 @@ DECODE_UNITS = 256
 #: keys per chunk of the decode kernel, and the fewest chunks a block is given if its request has them
 DECODE_CHUNK = 32
 DECODE_MIN_CHUNKS_PER_BLOCK = 8
+#: the same when the blocks take several rounds anyway: every block has a start and an end worth
+#: several chunks' time, and nothing is idle that more blocks could fill (measured in the serving
+#: workload of 256 requests: 2.73 ms a captured step with 16, 2.77 with 8, 2.75 with 24, 2.80 with 32)
+DECODE_MIN_CHUNKS_MANY_ROUNDS = 16
 #: the most blocks that share one request (the kernel's limit)
 DECODE_MAX_BLOCKS_PER_REQUEST = 64
 
@@ -56,8 +60,9 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
 
     A request of c chunks of 32 keys gets ceil(c / size) blocks of four waves and deals its
     chunks evenly to them. The chip runs ``slots`` blocks per key/value item at once. If all
-    blocks can run in one round, ``size`` is the smallest at which they do: the step then
-    takes as long as one block. Otherwise (or if that is slower) ``size`` is half of what a
+    blocks can run in one round, ``size`` is the smallest at which they do (but not so small
+    that joining a request's blocks takes longer than the blocks): the step then takes as long
+    as one block. Otherwise (or if that is slower) ``size`` is half of what a
     slot has to work off in all, and the list starts with the longest requests, so that the
     rounds stay full to the end. Row 0 is (blocks, 0, 0, 0), row 1 + i is (token, block of its
     request + 65536 * blocks of its request, chunks per wave, first partial slot of the
@@ -73,6 +78,7 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
     slots = _decode_slots(rows, nq, nkv)
     if size is None:
         size = -(-total // (2 * slots))  # many rounds: half a slot's share
+        least = DECODE_MIN_CHUNKS_MANY_ROUNDS
         if n + padding <= slots:
             a, b = 1, longest  # the smallest block size at which one round holds all blocks
             while a < b:
@@ -82,8 +88,10 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
                 else:
                     a = mid + 1
             if a <= 3 * size:  # one round of blocks of a, against total / slots + size for many rounds
-                size = a
-        size = max(size, DECODE_MIN_CHUNKS_PER_BLOCK)
+                # The block that joins a request's blocks takes about half a chunk's time for each
+                # of them: size + chunks / (2 size) is least at sqrt(chunks / 2).
+                size, least = max(a, math.isqrt(longest // 2)), DECODE_MIN_CHUNKS_PER_BLOCK
+        size = max(size, least)
     size = max(size, -(-longest // DECODE_MAX_BLOCKS_PER_REQUEST))
     nb = -(-chunks // size)
     per = -(-chunks // (4 * nb))

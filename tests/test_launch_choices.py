@@ -99,12 +99,17 @@ def test_decode_work_of_known_shapes():
     for n in (96, 256):                                                # two blocks a unit: whole requests again
         w = decode_work(tok(n), pos(n, 4096), n, 0, 28, 4)
         assert w[0, 0] == n and (w[1:, 2] == 33).all()
+    # one request of 16,384 tokens: 513 chunks in blocks of sqrt(513 / 2) = 16, not of the 9 that 64 blocks would hold
+    w = decode_work(tok(1), pos(1, 16384), 1, 0, 28, 4)
+    assert w[0, 0] == 33 and (w[1:, 2] == 4).all()
     # 256 requests of very different lengths on two key/value heads: the long ones are cut
     rng = np.random.default_rng(0)
     p = np.exp(rng.uniform(np.log(16), np.log(2560), 256)).astype(np.int32)
     w = decode_work(tok(256), p, 256, 0, 12, 2)
     assert w[1, 1] // 65536 >= 4 and w[1, 0] == int(np.argmax(p))
     assert 4 * w[1:, 2].max() * 32 <= p.sum() // 256 + 256             # a block is about half a slot's share
+    chunks_of = dict(zip(range(256), (p // 32 + 1).tolist()))
+    assert all(nb == 1 for t, nb in zip(w[1:, 0].tolist(), (w[1:, 1] // 65536).tolist()) if chunks_of[t] <= 16)   # and 16 chunks at least
 
 
 def test_prefill_work_lists_cover_every_chunk_once():
