@@ -301,12 +301,20 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
 
 // W = [gate rows; up rows] (two_i x K); out: bfloat16 [M][two_i / 2] = silu(X gate^T) * (X up^T).
 // A block takes 64 features (64 gate rows and 64 up rows, eight multiplying waves), or 96 with
-// twelve for up to 128 rows of X where one round of blocks would not hold them otherwise. The
+// twelve for up to 128 rows of X (128 for 25 to 64 rows) where one round of blocks would not hold
+// them otherwise. The
 // rows of X that a block multiplies are 64, 96 (with 96 features), 128, 192 or 256, whichever
 // holds M: fewer rows are fewer multiplying waves, fewer loads and a deeper ring (measured on the
 // 7B shape, weights from memory: 49 us at 64 rows, 57 at 96, 63 at 128).
 namespace {
-int silu_features(int M, int two_i) { return M <= 128 && (two_i / 2 + 63) / 64 > 256 ? 96 : 64; }
+int silu_features(int M, int two_i) {
+  const int inter = two_i / 2;
+  if ((inter + 63) / 64 <= 256 || M > 128) return 64;
+  // 128 features: the 32B shape's 27,648 in 216 blocks, for 25 to 64 rows of X (measured in its
+  // decode steps against the weight-streaming kernel: 34.2 against 35.0 ms at 64 requests, 22.7
+  // against 22.9 at 32, the same at 8, 13.0 against 12.7 at one)
+  return M >= 25 && M <= 64 && (inter + 95) / 96 > 256 ? 128 : 96;
+}
 }  // namespace
 
 extern "C" int pyre_gemm_mid_silu_blocks(int M, int two_i) {
@@ -327,6 +335,12 @@ extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, l
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else if (M > 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 2, kSiluMul, 8, 3>), grid, dim3(64 * 14), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 32 && silu_features(M, two_i) == 128) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 4, kSiluMul, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+  } else if (M <= 64 && silu_features(M, two_i) == 128) {
+    hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 4, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
                        static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
   } else if (M <= 32 && silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 3, kSiluMul, 8, 5>), grid, dim3(64 * 11), 0, stream, x,

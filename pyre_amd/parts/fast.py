@@ -20,7 +20,8 @@ SKINNY_MAX_ROWS = 64
 #: the most partial sums of a weight-streaming product
 SKINNY_MAX_KSPLIT = 12
 #: up to this many rows the gate/up product and the SiLU-gate can be one weight-streaming kernel
-#: (shapes whose features one round of the other kernel's blocks does not hold: the 32B shape's)
+#: (shapes whose features one round of the other kernel's blocks does not hold: the 32B shape's
+#: at up to 24 rows)
 FUSED_SILU_MAX_ROWS = 64
 #: most rows of the kernel between the two, which keeps a step's rows against 64 rows of the weights
 MID_MAX_ROWS = 256

@@ -832,13 +832,15 @@ def test_gemm_mid(m, n, k, ksplit):
 
 
 @pytest.mark.parametrize("m", [1, 8, 32, 33, 64, 65, 96, 97, 128, 129, 192, 193, 256])
-@pytest.mark.parametrize("inter,k", [(176, 64), (8960, 1536), (250, 96), (70, 520), (18944, 136), (16401, 64)])
+@pytest.mark.parametrize("inter,k", [(176, 64), (8960, 1536), (250, 96), (70, 520), (18944, 136), (16401, 64), (24600, 72)])
 def test_gemm_mid_silu(m, inter, k):
     """Blocks of 64 features, and of 96 for up to 128 rows where 64 would make more than 256
-    blocks (the last two sizes), whose loads do not divide evenly over the block's waves; the
+    blocks (or of 128 for 25 to 64 rows where 96 still would: the last size), whose loads do not
+    divide evenly over the block's waves; the
     row counts lie on both sides of every size of block (64, 96, 128, 192, 256 rows)."""
     ops = _ops()
-    assert ops.gemm_mid_silu_blocks(m, 2 * inter) == -(-inter // (96 if m <= 128 and inter > 256 * 64 else 64))
+    features = 64 if m > 128 or inter <= 256 * 64 else 128 if 25 <= m <= 64 and inter > 256 * 96 else 96
+    assert ops.gemm_mid_silu_blocks(m, 2 * inter) == -(-inter // features)
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
     w = rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.1)
     out = torch.full((m, inter), float("nan"), device=DEV, dtype=torch.bfloat16)
