@@ -1,8 +1,9 @@
 """The cache manager: page pools, block tables, state slots.
 
-Every entry of a model's layer order declares what it keeps
-(:class:`~pyre_amd.parts.base.PagedCacheSpec`, :class:`~pyre_amd.parts.base.StateCacheSpec`
-or nothing). Entries with the same needs form a *group*:
+Every entry of a model's layer order declares what it keeps: a list of cache descriptions
+(:class:`~pyre_amd.parts.base.PagedCacheSpec`, :class:`~pyre_amd.parts.base.StateCacheSpec`),
+one per cache of the entry's layer (none, one for a layer with one mixer, more for a layer with
+several). A *cell* is (entry, index in that list). Cells with the same needs form a *group*:
 
 * a **page group** has a pool of pages of its own and, for each request, a block
   table of its own. One page id addresses that page in every layer of the group
@@ -11,7 +12,9 @@ or nothing). Entries with the same needs form a *group*:
   description says (the mixer's choice); the manager allocates
   ``[layers, pages, *page_shape]`` for each and knows nothing of their meaning.
   A group with a window gives a page back as soon as no later query can see it.
-  All groups share one page size.
+  All groups share one page size, the engine's; a description that names another
+  (``PagedCacheSpec.page_size``: a mixer whose kernels need pages of a particular size) is
+  refused when the manager is made.
 * a **state group** has one fixed-size state per (layer, slot).
 
 A request holds one *slot* from admission to its end; the slot indexes the state
@@ -44,30 +47,39 @@ from pyre_amd.parts.base import PagedCacheSpec, StateCacheSpec
 RELEASED = -1  #: block-table entry of a page that a window has passed
 
 
+class _Cells:
+    """The cells (entry of the layer order, index among that entry's caches) of a group, in order."""
+
+    cells: list
+
+    @property
+    def entries(self) -> list[int]:
+        """Positions in the layer order, ascending (an entry with two cells of this group twice)."""
+        return [entry for entry, _ in self.cells]
+
+    def layer_index(self, entry: int, k: int = 0) -> int:
+        """Where cell (entry, k) lies along the first axis of the group's tensors."""
+        return self.cells.index((entry, k))
+
+
 @dataclass
-class PageGroup:
+class PageGroup(_Cells):
     index: int
     spec: PagedCacheSpec
-    entries: list[int]               #: positions in the layer order, ascending
+    cells: list[tuple[int, int]]
     page_size: int
     num_pages: int
     allocator: PageAllocator
-    #: name -> [len(entries), num_pages, *page_shape] for every tensor of the description
+    #: name -> [len(cells), num_pages, *page_shape] for every tensor of the description
     tensors: dict = field(default_factory=dict)
-
-    def layer_index(self, entry: int) -> int:
-        return self.entries.index(entry)
 
 
 @dataclass
-class StateGroup:
+class StateGroup(_Cells):
     index: int
     spec: StateCacheSpec
-    entries: list[int]
-    tensor: object = None            #: [len(entries), num_slots, *shape]
-
-    def layer_index(self, entry: int) -> int:
-        return self.entries.index(entry)
+    cells: list[tuple[int, int]]
+    tensor: object = None            #: [len(cells), num_slots, *shape]
 
 
 @dataclass
@@ -84,7 +96,8 @@ class _Request:
 class CacheManager:
     def __init__(self, cache_specs: list, page_size: int, num_pages: int, max_num_seqs: int,
                  max_model_len: int, fill=None, poison: bool = False):
-        """``cache_specs[i]`` is what entry i of the layer order keeps (or None)."""
+        """``cache_specs[i]`` is what entry i of the layer order keeps: a list of descriptions
+        (a single description or None stand for a list of one or of none)."""
         self.fill = fill
         self.poison = poison
         if page_size <= 0 or num_pages <= 0 or max_num_seqs <= 0:
@@ -95,28 +108,44 @@ class CacheManager:
         self.max_pages_per_seq = -(-max_model_len // page_size)
         self.page_groups: list[PageGroup] = []
         self.state_groups: list[StateGroup] = []
-        #: entry -> ("paged" | "state", group index) for entries that keep something
-        self.group_of_entry: dict[int, tuple[str, int]] = {}
+        #: (entry, index among the entry's caches) -> ("paged" | "state", group index)
+        self.group_of_cell: dict[tuple[int, int], tuple[str, int]] = {}
         by_spec: dict[object, object] = {}
-        for entry, spec in enumerate(cache_specs):
-            if spec is None:
-                continue
-            grp = by_spec.get(spec)
-            if grp is None:
-                if isinstance(spec, PagedCacheSpec):
-                    grp = PageGroup(len(self.page_groups), spec, [], page_size, num_pages,
-                                    PageAllocator(num_pages))
-                    self.page_groups.append(grp)
-                elif isinstance(spec, StateCacheSpec):
-                    grp = StateGroup(len(self.state_groups), spec, [])
-                    self.state_groups.append(grp)
-                else:
-                    raise TypeError(f"entry {entry}: unknown cache description {spec!r}")
-                by_spec[spec] = grp
-            grp.entries.append(entry)
-            self.group_of_entry[entry] = ("paged" if isinstance(grp, PageGroup) else "state", grp.index)
+        for entry, kept in enumerate(cache_specs):
+            specs = [] if kept is None else list(kept) if isinstance(kept, (list, tuple)) else [kept]
+            for k, spec in enumerate(specs):
+                grp = by_spec.get(spec)
+                if grp is None:
+                    if isinstance(spec, PagedCacheSpec):
+                        if spec.page_size not in (None, page_size):
+                            raise ValueError(f"entry {entry} of the layer order keeps a cache whose kernels need pages "
+                                             f"of {spec.page_size} tokens; the engine is set to pages of {page_size}, "
+                                             "and all page groups share one size: set page_size to that")
+                        grp = PageGroup(len(self.page_groups), spec, [], page_size, num_pages,
+                                        PageAllocator(num_pages))
+                        self.page_groups.append(grp)
+                    elif isinstance(spec, StateCacheSpec):
+                        grp = StateGroup(len(self.state_groups), spec, [])
+                        self.state_groups.append(grp)
+                    else:
+                        raise TypeError(f"entry {entry}: unknown cache description {spec!r}")
+                    by_spec[spec] = grp
+                grp.cells.append((entry, k))
+                self.group_of_cell[(entry, k)] = ("paged" if isinstance(grp, PageGroup) else "state", grp.index)
+        self._caches_of_entry: dict[int, int] = {}
+        for entry, _ in self.group_of_cell:
+            self._caches_of_entry[entry] = self._caches_of_entry.get(entry, 0) + 1
         self.slots = PageAllocator(max_num_seqs, what="slot")
         self._requests: dict[object, _Request] = {}
+
+    @property
+    def group_of_entry(self) -> dict[int, tuple[str, int]]:
+        """entry -> ("paged" | "state", group index) of the entry's first cache."""
+        return {entry: where for (entry, k), where in self.group_of_cell.items() if k == 0}
+
+    def caches_of_entry(self, entry: int) -> int:
+        """How many caches entry ``entry`` of the layer order keeps."""
+        return self._caches_of_entry.get(entry, 0)
 
     # ------------------------------------------------------------------ tensors
 
@@ -125,7 +154,7 @@ class CacheManager:
         import torch
 
         for g in self.page_groups:
-            n = len(g.entries)
+            n = len(g.cells)
             for t in g.spec.tensors:
                 dt = torch.float32 if t.dtype == "float32" else dtype
                 g.tensors[t.name] = torch.zeros((n, g.num_pages, *t.page_shape(g.page_size)), device=device, dtype=dt)
@@ -133,7 +162,7 @@ class CacheManager:
         for g in self.state_groups:
             dt = torch.float32 if g.spec.dtype == "float32" else dtype
             # one slot more than requests: padding rows of a captured step write there
-            g.tensor = torch.zeros((len(g.entries), self.max_num_seqs + 1, *g.spec.shape), device=device, dtype=dt)
+            g.tensor = torch.zeros((len(g.cells), self.max_num_seqs + 1, *g.spec.shape), device=device, dtype=dt)
             if self.poison:
                 self._fill(g.tensor, list(range(self.max_num_seqs)), float("nan"))
 
@@ -153,7 +182,7 @@ class CacheManager:
             self._fill(t, pages, float("nan"))
 
     def bytes_per_page(self, dtype_bytes: int) -> int:
-        return sum(len(g.entries) * t.elements_per_token() * g.page_size * (4 if t.dtype == "float32" else dtype_bytes)
+        return sum(len(g.cells) * t.elements_per_token() * g.page_size * (4 if t.dtype == "float32" else dtype_bytes)
                    for g in self.page_groups for t in g.spec.tensors)
 
     # ------------------------------------------------------------------ requests

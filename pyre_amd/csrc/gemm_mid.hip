@@ -308,12 +308,12 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
 // 7B shape, weights from memory: 49 us at 64 rows, 57 at 96, 63 at 128).
 namespace {
 int silu_features(int M, int two_i) {
-  const int inter = two_i / 2;
-  if ((inter + 63) / 64 <= 256 || M > 128) return 64;
+  const int inter = two_i / 2, units = compute_units();
+  if ((inter + 63) / 64 <= units || M > 128) return 64;
   // 128 features: the 32B shape's 27,648 in 216 blocks, for 25 to 64 rows of X (measured in its
   // decode steps against the weight-streaming kernel: 34.2 against 35.0 ms at 64 requests, 22.7
   // against 22.9 at 32, the same at 8, 13.0 against 12.7 at one)
-  return M >= 25 && M <= 64 && (inter + 95) / 96 > 256 ? 128 : 96;
+  return M >= 25 && M <= 64 && (inter + 95) / 96 > units ? 128 : 96;
 }
 }  // namespace
 

@@ -307,7 +307,8 @@ int launch_skinny(int mt, dim3 grid, hipStream_t stream, const bf16* X, size_t l
 // stages X again. The fastest had about 1.6 blocks per compute unit (or, with fewer tiles
 // than that, three waves): that is the rule.
 int silu_waves(int tiles) {
-  constexpr double kUnits = 256.0, kBlocksPerUnit = 1.6;
+  const double kUnits = compute_units();
+  constexpr double kBlocksPerUnit = 1.6;
   int best = 3;
   double best_dist = 1e30;
   for (int w = 3; w <= 6; ++w) {

@@ -10,6 +10,12 @@ extern "C" {
 
 const char* pyre_last_error();
 int pyre_abi_version();
+// Compute units of the current device (256 where there is no device to ask): the kernels whose
+// blocks are meant to fill the chip in one round shape their launches by it, and so must
+// whoever plans work for them on the host.
+int pyre_compute_units();
+// A digest of the sources this library was compiled from, as the build wrote it in.
+const char* pyre_sources_digest();
 
 // Streams `bytes` of device memory through the chip and writes (almost) nothing:
 // a measurement of achievable read bandwidth.
@@ -155,8 +161,12 @@ int pyre_argmax(const float* logits, long row_stride, int* out, void* scratch, i
 // refused with an error. The caller makes the GPU of `stream`, `logits` and `out` the current
 // device. Same kernels and same results as pyre_argmax. All calls on one GPU share that GPU's
 // array: calls that may overlap there (two streams, two threads) race; put them on one stream
-// or use pyre_argmax with scratch of their own.
+// or use pyre_argmax with scratch of their own. The first call on a device looks the array's
+// address up (hipGetSymbolAddress), which must not happen while a stream is capturing: a caller
+// that captures calls pyre_argmax_static_init() on that device beforehand (it launches nothing
+// and may be called any number of times).
 #define PYRE_ARGMAX_STATIC_MAX_ROWS 256
+int pyre_argmax_static_init();
 int pyre_argmax_static(const float* logits, long row_stride, int* out, int m, int vocab,
                        hipStream_t stream);
 

@@ -114,6 +114,11 @@ __device__ inline float block_max(float v, float* scratch) {
 // The last error of this thread, returned to Python by pyre_last_error().
 char* error_buffer();
 
+// Compute units of the current device (runtime.hip); launch shapes that are made to fill the
+// chip in one round of blocks follow it.
+constexpr int kDefaultUnits = 256;  // an MI355X
+int compute_units();
+
 inline int fail(const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);

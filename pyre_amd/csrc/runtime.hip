@@ -1,16 +1,45 @@
-// The library's small host-side state: the per-thread error message.
+// The library's small host-side state: the per-thread error message, the number of compute
+// units of each device, the digest of the sources it was built from.
+#include <atomic>
+
 #include "pyre_api.h"
 #include "pyre_common.h"
+
+#ifndef PYRE_SOURCES_DIGEST
+#define PYRE_SOURCES_DIGEST "unknown"
+#endif
 
 namespace pyre {
 char* error_buffer() {
   static thread_local char buf[512] = "";
   return buf;
 }
+
+// Compute units of the current device, asked for once per device; kDefaultUnits where there
+// is no device to ask (launch plans made on a machine without one).
+int compute_units() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> known[kMaxDevices];
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    (void)hipGetLastError();
+    return kDefaultUnits;
+  }
+  int n = known[device].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return kDefaultUnits;
+  }
+  known[device].store(n, std::memory_order_relaxed);
+  return n;
+}
 }  // namespace pyre
 
 extern "C" const char* pyre_last_error() { return pyre::error_buffer(); }
-extern "C" int pyre_abi_version() { return 14; }
+extern "C" int pyre_abi_version() { return 15; }
+extern "C" int pyre_compute_units() { return pyre::compute_units(); }
+extern "C" const char* pyre_sources_digest() { return PYRE_SOURCES_DIGEST; }
 
 // ---------------------------------------------------------------------------
 // A plain streaming read of `bytes` (a multiple of 16) for measuring what the

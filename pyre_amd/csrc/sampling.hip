@@ -194,7 +194,22 @@ int static_scratch_of(int device, void** ptr) {
   return 0;
 }
 
+// The current device's copy of `scratch`, looked up at the first call on that device.
+int static_scratch_here(void** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  PYRE_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+  PYRE_REQUIRE(device >= 0 && device < kMaxDevices, "argmax_static: device %d is beyond the %d this entry point knows",
+               device, kMaxDevices);
+  return static_scratch_of(device, ptr);
+}
+
 }  // namespace
+
+extern "C" int pyre_argmax_static_init() {
+  void* base = nullptr;
+  return static_scratch_here(&base);
+}
 
 extern "C" int pyre_argmax_static(const float* logits, long row_stride, int* out, int m, int vocab,
                                   hipStream_t stream) {
@@ -203,13 +218,8 @@ extern "C" int pyre_argmax_static(const float* logits, long row_stride, int* out
                "argmax_static: %d rows; the built-in scratch holds %d (use pyre_argmax with scratch of your own)", m,
                PYRE_ARGMAX_STATIC_MAX_ROWS);
   if (m <= 0) return 0;
-  int device = -1;
-  hipError_t e = hipGetDevice(&device);
-  PYRE_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
-  PYRE_REQUIRE(device >= 0 && device < kMaxDevices, "argmax_static: device %d is beyond the %d this entry point knows",
-               device, kMaxDevices);
   void* base = nullptr;
-  if (int rc = static_scratch_of(device, &base)) return rc;
+  if (int rc = static_scratch_here(&base)) return rc;
   // Nothing has to start at zero: the first stage writes all 64 slices of every row before
   // the second stage reads them, whatever an earlier (larger) call left behind.
   float* pv = static_cast<float*>(base);

@@ -197,7 +197,8 @@ def prepare_step(entries: list[Entry], cache, vocab_size: int, graph_max_rows: i
             cache.reserve(e.rid, len(e.tokens))
             reserved.append(e.rid)
         n_tokens = sum(len(e.tokens) for e in entries)
-        pages = max((len(cache.block_table(e.rid, 0)) for e in entries), default=0) if cache.page_groups else 0
+        # the widest table of the step (the groups share a page size, so their tables are equally long)
+        pages = max((len(cache.block_table(e.rid, g)) for e in entries for g in range(len(cache.page_groups))), default=0)
         graphable = (n_tokens == len(entries) and n_tokens <= graph_max_rows and all(len(e.want) == 1 for e in entries))
         if graphable:
             rows, width = round_decode_shape(n_tokens, pages)

@@ -63,10 +63,17 @@ class Runtime:
     max_positions: int               #: rows of position tables (the longest request)
     workspace: Workspace = None
     options: dict = field(default_factory=dict)
+    #: compute units of the device, read once: launch plans whose shape decides the order of a
+    #: sum go by this number for as long as the engine lives (None: asked of the device)
+    compute_units: int | None = None
 
     def __post_init__(self) -> None:
         if self.workspace is None:
             self.workspace = Workspace(self.device)
+        if self.compute_units is None:
+            from pyre_amd.hip import ops
+
+            self.compute_units = ops.compute_units(self.device)
 
     @property
     def true_fp32(self) -> bool:

@@ -48,7 +48,8 @@ class Engine:
         # The model's own limit is the default, not a bound: the reference reads
         # max_position_embeddings and never consults it (`pyre/config.py:60`).
         self.max_model_len = ec.max_model_len or spec.max_positions
-        self.runtime = Runtime(self.device, self.dtype, self.max_model_len)
+        with torch.cuda.device(self.device):
+            self.runtime = Runtime(self.device, self.dtype, self.max_model_len)
         specs = model.cache_specs()
         probe = CacheManager(specs, ec.page_size, 1, ec.max_num_seqs, self.max_model_len)
         num_pages = self._choose_num_pages(probe)
@@ -99,19 +100,22 @@ class Engine:
 
     @classmethod
     def from_state(cls, config: ModelConfig, state: dict[str, torch.Tensor],
-                   engine_config: EngineConfig | None = None) -> "Engine":
-        """Tensors already in memory (random weights made on the device, tests)."""
+                   engine_config: EngineConfig | None = None, consume: bool = False) -> "Engine":
+        """Tensors already in memory (random weights made on the device, tests). ``consume``:
+        ``state`` is emptied, so that the tensors which the parts copy (fused weights) are free
+        as soon as they have been copied and not when the caller lets go of its dictionary."""
         ec = engine_config or EngineConfig()
         model = LayeredModel(get_architecture(config.architecture).build(config))
         tensors = adopt_state(state, model.tensor_specs(), torch.device(ec.device), TORCH_DTYPES[ec.dtype])
+        if consume:
+            state.clear()
         return cls._finish(model, config, ec, tensors)
 
     @classmethod
     def _finish(cls, model, config, ec, tensors) -> "Engine":
         with torch.cuda.device(torch.device(ec.device)):
             rt = Runtime(torch.device(ec.device), TORCH_DTYPES[ec.dtype], 0)
-            model.bind(tensors, rt)
-            tensors.clear()
+            model.bind(tensors, rt)  # takes the tensors out of the dictionary one by one
             return cls(model, config, ec)
 
     def tune_library_gemms(self, rows) -> int:
@@ -162,7 +166,7 @@ class Engine:
     def has(self, rid) -> bool:
         return rid in self.cache
 
-    def step(self, entries: list[Entry], fed_ids: torch.Tensor | None = None) -> torch.Tensor | None:
+    def step(self, entries: list[Entry], fed_ids: torch.Tensor | None = None, tap=None) -> torch.Tensor | None:
         """Run one batch. Requests not seen before are admitted (a slot and empty
         block tables); pages for all the step's tokens are reserved first, lengths
         are committed afterwards. Returns float32 ``[sum(len(want)), vocab]`` on the
@@ -183,6 +187,10 @@ class Engine:
         the device, for instance the ids a sampler has just written) when the step
         runs on the device: the host can put the step on the stream without waiting
         for the previous step's result.
+
+        ``tap(pos, rows)``, a debugging aid, is called after every entry ``pos`` of the layer
+        order with a copy of the hidden rows ``[tokens, hidden]`` (float32) as they stand there;
+        such a step runs eagerly.
         """
         n_tokens = sum(len(e.tokens) for e in entries)
         ec = self.engine_config
@@ -190,13 +198,13 @@ class Engine:
             raise ValueError(f"step of {n_tokens} tokens exceeds max_num_batched_tokens={ec.max_num_batched_tokens}")
         if len(entries) > ec.max_num_seqs:
             raise ValueError(f"step of {len(entries)} requests exceeds max_num_seqs={ec.max_num_seqs}")
-        hb, graph_shape = prepare_step(entries, self.cache, self.vocab_size, GRAPH_MAX_ROWS if ec.use_graphs else 0,
-                                       fed_ids is not None)
+        hb, graph_shape = prepare_step(entries, self.cache, self.vocab_size,
+                                       GRAPH_MAX_ROWS if ec.use_graphs and tap is None else 0, fed_ids is not None)
         with torch.cuda.device(self.device):
             if graph_shape is not None:
                 logits = self._step_captured(hb, *graph_shape, fed_ids)
             else:
-                logits = self._run(hb, fed_ids)
+                logits = self._run(hb, fed_ids, tap)
         for e in entries:
             self.cache.commit(e.rid, len(e.tokens))
         self.steps_run += 1
@@ -222,19 +230,19 @@ class Engine:
             arrays={spec.name: views["x:" + spec.name] for spec in self.step_arrays})
         return ctx, self._layer_views(views)
 
-    def _forward(self, ctx, caches):
+    def _forward(self, ctx, caches, tap=None):
         """The model's kernels on torch's current stream, asked for once."""
         from pyre_amd.hip import ops
 
         ops.use_stream(torch.cuda.current_stream().cuda_stream)
         try:
-            return self.model.forward(ctx, caches)
+            return self.model.forward(ctx, caches, tap) if tap is not None else self.model.forward(ctx, caches)
         finally:
             ops.use_stream(None)
 
-    def _run(self, hb, fed_ids=None):
+    def _run(self, hb, fed_ids=None, tap=None):
         ctx, caches = self._context(hb.attach(self.step_arrays), fed_ids)
-        return self._forward(ctx, caches)
+        return self._forward(ctx, caches, tap)
 
     def _step_captured(self, hb, rows: int, width: int, fed_ids=None):
         """A decode step at a fixed size (``rows`` requests, tables ``width`` pages
@@ -269,25 +277,26 @@ class Engine:
         self.graph_replays += 1
         return logits[:live]
 
-    def _layer_views(self, views) -> list:
+    def _layer_views(self, views) -> list[list]:
+        """For every entry of the layer order the views of its caches (or of the entry's whose
+        caches it reads), in the order of the layer's descriptions."""
         cache = self.cache
         out = []
         for pos, call in enumerate(self.model.schedule):
             src = call.cache_from if call.cache_from is not None else pos
-            where = cache.group_of_entry.get(src)
-            if where is None:
-                out.append(None)
-                continue
-            kind, gi = where
-            if kind == "paged":
-                g = cache.page_groups[gi]
-                li = g.layer_index(src)
-                out.append(PagedLayerView({name: t[li] for name, t in g.tensors.items()}, views[f"table{gi}"],
-                                          views[f"slots{gi}"], g.page_size, g.spec.window,
-                                          writes=call.cache_from is None))
-            else:
-                g = cache.state_groups[gi]
-                out.append(StateLayerView(g.tensor[g.layer_index(src)], views["state_slots"]))
+            mine = []
+            for k in range(cache.caches_of_entry(src)):
+                kind, gi = cache.group_of_cell[(src, k)]
+                if kind == "paged":
+                    g = cache.page_groups[gi]
+                    li = g.layer_index(src, k)
+                    mine.append(PagedLayerView({name: t[li] for name, t in g.tensors.items()}, views[f"table{gi}"],
+                                               views[f"slots{gi}"], g.page_size, g.spec.window,
+                                               writes=call.cache_from is None))
+                else:
+                    g = cache.state_groups[gi]
+                    mine.append(StateLayerView(g.tensor[g.layer_index(src, k)], views["state_slots"]))
+            out.append(mine)
         return out
 
     def finish(self, rid) -> None:

@@ -34,6 +34,9 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--max-seqs", type=int, default=8, help="most requests that are live at a time")
     ap.add_argument("--poison", action="store_true",
                     help="debugging aid: freed cache pages and state slots are filled with NaN")
+    ap.add_argument("--graphs", action="store_true",
+                    help="capture steps of single tokens in HIP graphs and replay them, as generation does "
+                         "(the same kernels and the same bits either way)")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
     if args.page_size <= 0 or TOKEN_ROUNDING % args.page_size:
@@ -67,7 +70,7 @@ def main(argv: list[str] | None = None) -> int:
     ec = EngineConfig(dtype=args.dtype, device=args.device, page_size=args.page_size,
                       max_cached_tokens=max_tokens, max_num_seqs=args.max_seqs,
                       max_model_len=max(model_limit, max_tokens),
-                      max_num_batched_tokens=max(max_tokens, 4096), use_graphs=False, debug_poison=args.poison)
+                      max_num_batched_tokens=max(max_tokens, 4096), use_graphs=args.graphs, debug_poison=args.poison)
     note(f"loading {args.model} ({args.dtype}) ...")
     engine = Engine.from_folder(args.model, ec)
     note(f"ready: {engine.cache.page_groups[0].num_pages if engine.cache.page_groups else 0} pages of "

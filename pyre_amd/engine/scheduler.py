@@ -111,7 +111,12 @@ class Scheduler:
         self.sampler = sampler
         self.waiting: list[Request] = []
         self.running: list[Request] = []
+        #: finished requests that nobody has taken yet (:meth:`take_finished`), the oldest first;
+        #: at most ``max_finished_kept`` of them, so that a stream driven by ``step()`` whose
+        #: caller reads the tokens that ``step`` returns and never comes here does not grow
         self.finished: dict[int, Request] = {}
+        self.max_finished_kept = 4096
+        self.last_finished: list[Request] = []  #: the requests that the last step finished
         self._next_seq = 0
         self.steps = 0
         #: put the next decode step on the device before this step's tokens are read
@@ -232,6 +237,7 @@ class Scheduler:
 
     def step(self) -> list[tuple[int, int]]:
         """Plan, run and sample one batch; returns (seq_id, new token) pairs."""
+        self.last_finished = []
         ahead, self._ahead = self._ahead, None
         if ahead is not None and all(e.request.done for e in ahead[0].entries):
             ahead = None  # every request of the step that ran ahead has ended meanwhile
@@ -272,11 +278,19 @@ class Scheduler:
                     r.finish_reason = "eos"
                 elif len(r.generated) >= p.max_new_tokens:
                     r.finish_reason = "length"
-        for r in [r for r in self.running if r.done]:
+        self.last_finished = [r for r in self.running if r.done]
+        for r in self.last_finished:
             self.running.remove(r)
             self.engine.finish(r.seq_id)
             self.finished[r.seq_id] = r
+        while len(self.finished) > self.max_finished_kept:
+            del self.finished[next(iter(self.finished))]
         return out
+
+    def take_finished(self) -> dict[int, Request]:
+        """The requests that have finished since the last call, which the scheduler then forgets."""
+        done, self.finished = self.finished, {}
+        return done
 
     def _run_ahead(self, sampling: list[Request]):
         """Plan the next step without this step's tokens and put it on the device. Returns
@@ -307,12 +321,26 @@ class Scheduler:
         finally:
             for r in marked:
                 r.pending, r.ending = 0, False
-        logits = self.engine.step(entries, fed_ids=self.sampler.ids)
+        try:
+            logits = self.engine.step(entries, fed_ids=self.sampler.ids)
+        except (MemoryError, ValueError):
+            # The engine's step is all or nothing: the cache is as it was. The step that was to
+            # run ahead is given up (its admissions taken back); this step's tokens are
+            # collected as usual and the next step is planned with them.
+            for r in reversed(nxt.admitted):
+                self.running.remove(r)
+                if r.seq_id in self.cache:
+                    self.engine.finish(r.seq_id)
+                self.waiting.insert(0, r)
+            return None
         return nxt, logits
 
     def run(self) -> dict[int, list[int]]:
-        """Run until every request is finished: {seq_id: generated tokens}
-        (`pyre/scheduler.py:105-114`)."""
+        """Run until every request is finished: {seq_id: generated tokens} of the requests that
+        finished meanwhile (`pyre/scheduler.py:105-114`). They stay in ``finished`` until
+        :meth:`take_finished` (or the cap) removes them."""
+        results: dict[int, list[int]] = {sid: r.generated for sid, r in self.finished.items()}
         while self.has_work:
             self.step()
-        return {sid: r.generated for sid, r in sorted(self.finished.items())}
+            results.update((r.seq_id, r.generated) for r in self.last_finished)
+        return dict(sorted(results.items()))

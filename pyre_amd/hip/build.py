@@ -1,10 +1,13 @@
 """Compiles the HIP sources under ``pyre_amd/csrc`` into one shared library for gfx950.
 
-``ensure_built()`` returns the path of an up-to-date library, compiling what is
-missing or older than its source; ``build(force=True)`` compiles everything. The
-objects and the library live in ``pyre_amd/csrc/_build`` (or, when that folder
-cannot be written, in a per-user temporary folder). Progress goes to stderr so
-that a tool's stdout protocol stays clean.
+``ensure_built()`` returns the path of a library built from the sources as they are now,
+compiling what is missing or was compiled from other text; ``build(force=True)`` compiles
+everything. Nothing goes by file times: an object carries the digest of its source, the
+headers and the flags in a file beside it, and the library has the digest of all sources
+compiled in (``pyre_sources_digest()``), which the binding checks when it loads it. The
+objects and the library live in ``pyre_amd/csrc/_build`` (or, when that folder cannot be
+written, in a per-user temporary folder). Progress goes to stderr so that a tool's stdout
+protocol stays clean.
 """
 
 from __future__ import annotations
@@ -77,19 +80,48 @@ def build_dir() -> Path:
     return Path(tempfile.gettempdir()) / f"pyre_amd_build_{os.getuid()}_{tag}"
 
 
-def _stale(target: Path, deps: list[Path]) -> bool:
-    if not target.exists():
-        return True
-    t = target.stat().st_mtime
-    return any(d.stat().st_mtime > t for d in deps)
+def _digest(files: list[Path], extra: str = "") -> str:
+    h = hashlib.sha1(extra.encode())
+    for f in files:
+        h.update(f.name.encode() + b"\0" + f.read_bytes() + b"\0")
+    return h.hexdigest()
 
 
-def _compile_one(hipcc: str, src: Path, obj: Path) -> tuple[Path, float]:
+def sources_digest() -> str:
+    """A digest of every source, every header and the compiler's flags: what the library
+    answers from ``pyre_sources_digest()`` if it was built from this tree."""
+    return _digest([*sources(), *_headers()], " ".join(HIPCC_FLAGS))[:16]
+
+
+#: the source that has the digest of all of them compiled in
+_DIGEST_HOLDER = "runtime.hip"
+
+
+def _object_digest(src: Path, hdrs: list[Path], tree: str) -> str:
+    """What an object was compiled from: its source, the headers, the flags (and, for the
+    one source that holds it, the digest of the whole tree)."""
+    return _digest([src, *hdrs], " ".join(HIPCC_FLAGS) + (tree if src.name == _DIGEST_HOLDER else ""))
+
+
+def _stamp(path: Path) -> str:
+    try:
+        return path.with_name(path.name + ".sha1").read_text().strip()
+    except OSError:
+        return ""
+
+
+def _write_stamp(path: Path, digest: str) -> None:
+    path.with_name(path.name + ".sha1").write_text(digest + "\n")
+
+
+def _compile_one(hipcc: str, src: Path, obj: Path, digest: str, tree: str) -> tuple[Path, float]:
     t0 = time.time()
-    cmd = [hipcc, *HIPCC_FLAGS, f"-I{CSRC}", "-c", str(src), "-o", str(obj)]
+    define = [f'-DPYRE_SOURCES_DIGEST="{tree}"'] if src.name == _DIGEST_HOLDER else []
+    cmd = [hipcc, *HIPCC_FLAGS, *define, f"-I{CSRC}", "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise BuildError(f"hipcc failed on {src.name}:\n{proc.stderr[-4000:]}")
+    _write_stamp(obj, digest)
     return src, time.time() - t0
 
 
@@ -99,14 +131,16 @@ def build(force: bool = False, quiet: bool = False) -> Path:
     out.mkdir(parents=True, exist_ok=True)
     lib = out / LIB_NAME
     hdrs = _headers()
+    tree = sources_digest()
     todo = []
     objs = []
     for src in sources():
         obj = out / (src.stem + ".o")
         objs.append(obj)
-        if force or _stale(obj, [src, *hdrs]):
-            todo.append((src, obj))
-    if not todo and lib.exists() and not _stale(lib, objs):
+        digest = _object_digest(src, hdrs, tree)
+        if force or not obj.exists() or _stamp(obj) != digest:
+            todo.append((src, obj, digest))
+    if not todo and lib.exists() and _stamp(lib) == tree:
         return lib
     hipcc = _hipcc()
     if todo:
@@ -115,7 +149,7 @@ def build(force: bool = False, quiet: bool = False) -> Path:
         workers = max(1, min(len(todo), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16))
         t0 = time.time()
         with ThreadPoolExecutor(workers) as pool:
-            futures = [pool.submit(_compile_one, hipcc, s, o) for s, o in todo]
+            futures = [pool.submit(_compile_one, hipcc, s, o, d, tree) for s, o, d in todo]
             for i, fut in enumerate(futures):
                 src, dt = fut.result()
                 if not quiet:
@@ -126,16 +160,15 @@ def build(force: bool = False, quiet: bool = False) -> Path:
     if proc.returncode != 0:
         raise BuildError(f"link failed:\n{proc.stderr[-4000:]}")
     os.replace(tmp, lib)
+    _write_stamp(lib, tree)
     if not quiet:
         _log(f"linked {lib}")
     return lib
 
 
 def ensure_built() -> Path:
-    """Path of the library; compiles only when it is missing or out of date."""
-    out = build_dir()
-    lib = out / LIB_NAME
-    srcs = sources()
-    if lib.exists() and (not srcs or not _stale(lib, [*srcs, *_headers()])):
+    """Path of the library; compiles only when it is missing or was built from other sources."""
+    lib = build_dir() / LIB_NAME
+    if lib.exists() and (not sources() or _stamp(lib) == sources_digest()):
         return lib
     return build(force=False)

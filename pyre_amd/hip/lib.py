@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 
 class KernelError(RuntimeError):
@@ -40,6 +40,8 @@ _SIGNATURES = {
     "pyre_attn_prefill_work_bf16": [P, P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_argmax": [P, L, P, P, I, I, P],
     "pyre_argmax_static": [P, L, P, I, I, P],
+    "pyre_argmax_static_init": [],
+    "pyre_compute_units": [],
     "pyre_gemm_skinny_supports": [I, I, I, L, L],
     "pyre_gemm_skinny_bf16": [P, L, P, L, P, I, I, I, I, P],
     "pyre_gemm_skinny_silu_bf16": [P, L, P, L, P, I, I, I, P],
@@ -54,17 +56,29 @@ _SIGNATURES = {
 _lib = None
 
 
+def _open(path) -> ctypes.CDLL:
+    handle = ctypes.CDLL(str(path))
+    handle.pyre_last_error.restype = ctypes.c_char_p
+    handle.pyre_abi_version.restype = c_int
+    return handle
+
+
+def _fits(handle) -> bool:
+    """The library speaks this binding's ABI and was compiled from the sources of this tree."""
+    if handle.pyre_abi_version() != ABI_VERSION or not hasattr(handle, "pyre_sources_digest"):
+        return False
+    handle.pyre_sources_digest.restype = ctypes.c_char_p
+    return handle.pyre_sources_digest().decode() == _build.sources_digest()
+
+
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        path = _build.ensure_built()
-        handle = ctypes.CDLL(str(path))
-        handle.pyre_last_error.restype = ctypes.c_char_p
-        handle.pyre_abi_version.restype = c_int
-        if handle.pyre_abi_version() != ABI_VERSION:
-            # An older library from a previous checkout: rebuild once. The loader keeps the
-            # mapping of a path it has already opened, so the new build is opened under a
-            # name of its own.
+        handle = _open(_build.ensure_built())
+        if not _fits(handle):
+            # A library from other sources under a stamp that says otherwise (a copied build
+            # folder, an older checkout): rebuild once. The loader keeps the mapping of a path
+            # it has already opened, so the new build is opened under a name of its own.
             import os
             import shutil
 
@@ -72,14 +86,13 @@ def lib() -> ctypes.CDLL:
             fresh = path.with_name(f"{path.stem}.{os.getpid()}{path.suffix}")
             shutil.copyfile(path, fresh)
             try:
-                handle = ctypes.CDLL(str(fresh))
+                handle = _open(fresh)
             finally:
                 os.unlink(fresh)
-            handle.pyre_last_error.restype = ctypes.c_char_p
-            handle.pyre_abi_version.restype = c_int
-            if handle.pyre_abi_version() != ABI_VERSION:
-                raise KernelError(f"kernel library has ABI {handle.pyre_abi_version()}, the binding expects "
-                                  f"{ABI_VERSION}: sources and binding are out of step")
+            if not _fits(handle):
+                raise KernelError(f"kernel library has ABI {handle.pyre_abi_version()} and the binding expects "
+                                  f"{ABI_VERSION}, or it does not carry the digest of the sources it was built "
+                                  "from: sources and binding are out of step")
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.argtypes = argtypes

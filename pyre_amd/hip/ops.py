@@ -246,13 +246,28 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, ou
 
 F32_KSPLIT_MAX = 8
 
+#: compute units that launch plans are made for when nobody names a device (an MI355X)
+DEFAULT_UNITS = 256
 
-def gemm_f32_ksplit(n_out: int, k: int) -> int:
+
+def compute_units(device=None) -> int:
+    """Compute units of ``device`` (torch's current one if None), as the kernel library sees
+    them: its kernels that fill the chip in one round of blocks go by the same number."""
+    from pyre_amd.hip.lib import lib
+
+    if device is None:
+        return int(lib().pyre_compute_units())
+    with torch.cuda.device(device):
+        return int(lib().pyre_compute_units())
+
+
+def gemm_f32_ksplit(n_out: int, k: int, units: int = DEFAULT_UNITS) -> int:
     """Into how many parts of k the float32 product is split: enough blocks of 128 output
-    columns for the 256 compute units, parts of at least 512. A function of the weight's
-    shape alone, never of the rows, so that a row's result does not depend on its step."""
+    columns for the ``units`` compute units, parts of at least 512. A function of the weight's
+    shape (and the engine's device) alone, never of the rows, so that a row's result does not
+    depend on its step."""
     blocks = -(-n_out // 128)
-    return max(1, min(F32_KSPLIT_MAX, 256 // blocks, k // 512))
+    return max(1, min(F32_KSPLIT_MAX, units // blocks, k // 512))
 
 
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, m: int,
@@ -320,6 +335,10 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_ca
 
 
 ATTN_GENERIC_SCRATCH = 1 << 25   #: float32 elements of scratch that one launch of attn_generic may use
+#: the largest head that any attention kernel takes (attention_generic.hip's kMaxHead: a block of
+#: 256 threads holds one element each) and the most query heads of a launch (a grid dimension)
+ATTN_MAX_HEAD_DIM = 256
+ATTN_MAX_HEADS = 65535
 
 
 def _attn_generic_keys(table_width: int, page_size: int, window: int) -> int:
@@ -384,6 +403,17 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor | None
 
 
 ARGMAX_STATIC_MAX_ROWS = 256  #: rows that the library's built-in scratch holds
+
+
+def argmax_static_init(device=None) -> None:
+    """Look the built-in scratch's address up on ``device`` (torch's current one if None). The
+    first :func:`argmax_static` on a device does this by itself, which must not happen while a
+    stream is capturing: whoever captures calls this beforehand."""
+    if device is None:
+        call("pyre_argmax_static_init")
+    else:
+        with torch.cuda.device(device):
+            call("pyre_argmax_static_init")
 
 
 def argmax_static(logits: torch.Tensor, out: torch.Tensor) -> None:

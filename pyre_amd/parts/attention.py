@@ -10,7 +10,7 @@ from pyre_amd.hip import ops
 from pyre_amd.parts import attention_work as plan
 from pyre_amd.parts import fast
 from pyre_amd.parts.base import (AttentionSpec, Mixer, PagedCacheSpec, PagedTensorSpec, StepArraySpec, TensorSpec,
-                                 make_part)
+                                 make_part, take)
 from pyre_amd.parts.linear import Linear, linear_specs
 
 
@@ -60,9 +60,18 @@ class Attention(Mixer):
     """
 
     def __init__(self, spec: AttentionSpec):
-        if spec.num_heads % spec.num_kv_heads:
+        if spec.num_kv_heads <= 0 or spec.num_heads % spec.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
+        # what no attention kernel takes is refused when the model is built, not at its first step
+        if not (0 < spec.head_dim <= ops.ATTN_MAX_HEAD_DIM):
+            raise ValueError(f"attention: head_dim {spec.head_dim} is outside 1..{ops.ATTN_MAX_HEAD_DIM}, the sizes "
+                             "that the attention kernels take")
+        if spec.num_heads > ops.ATTN_MAX_HEADS:
+            raise ValueError(f"attention: {spec.num_heads} query heads are more than a launch holds ({ops.ATTN_MAX_HEADS})")
+        if spec.window < 0:
+            raise ValueError("attention: the window must not be negative")
         self.spec = spec
+        self.units = plan.DEFAULT_UNITS  #: compute units that the work lists are planned for; the engine's at bind
         self.position = make_part("position", spec.position)
         self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
         self.q_dim = spec.num_heads * spec.head_dim
@@ -84,17 +93,20 @@ class Attention(Mixer):
 
         def work(hb):
             return plan.decode_work(hb.arrays["attention.decode_tokens"], hb.positions, hb.decode_shape()[0],
-                                    s.window, s.num_heads, s.num_kv_heads)
+                                    s.window, s.num_heads, s.num_kv_heads, units=self.units)
 
         def portions(hb):
             return plan.prefill_work(hb.arrays["attention.prefill_tiles"], hb.positions, s.window,
-                                     plan.prefill_items(s.num_heads, s.num_kv_heads))
+                                     plan.prefill_items(s.num_heads, s.num_kv_heads), units=self.units)
 
-        return [*STEP_ARRAYS,
-                StepArraySpec(self.decode_work_name,
-                              lambda n_cap, s_cap: 4 * (1 + plan.decode_capacity(s_cap, s.num_heads, s.num_kv_heads)), work),
-                StepArraySpec(self.prefill_work_name,
-                              lambda n_cap, s_cap: 8 * (n_cap // TILE + s_cap + 2 * plan.DECODE_UNITS + 1), portions)]
+        def decode_cap(n_cap, s_cap):
+            return 4 * (1 + plan.decode_capacity(s_cap, s.num_heads, s.num_kv_heads, self.units))
+
+        def prefill_cap(n_cap, s_cap):
+            return 8 * plan.prefill_capacity(n_cap, s_cap, TILE, plan.prefill_items(s.num_heads, s.num_kv_heads), self.units)
+
+        return [*STEP_ARRAYS, StepArraySpec(self.decode_work_name, decode_cap, work),
+                StepArraySpec(self.prefill_work_name, prefill_cap, portions)]
 
     def linears(self) -> list:
         return [self.qkv, self.out]
@@ -108,12 +120,19 @@ class Attention(Mixer):
 
     def bind(self, tensors, runtime) -> None:
         p = self.spec.prefix
-        w = torch.cat([tensors[f"{p}.{n}_proj.weight"] for n in "qkv"], dim=0)
+        self.units = getattr(runtime, "compute_units", None) or plan.DEFAULT_UNITS
+        # the three weights are let go of one by one, so that at most one copy more than the
+        # fused matrix lives at any time
+        parts = []
+        for n in "qkv":
+            parts.append(take(tensors, f"{p}.{n}_proj.weight"))
+        w = torch.cat(parts, dim=0)
+        del parts
         b = None
         if self.spec.qkv_bias:
-            b = torch.cat([tensors[f"{p}.{n}_proj.bias"] for n in "qkv"], dim=0)
+            b = torch.cat([take(tensors, f"{p}.{n}_proj.bias") for n in "qkv"], dim=0)
         self.qkv.set(w, b)
-        self.out.set(tensors[f"{p}.o_proj.weight"], tensors.get(f"{p}.o_proj.bias") if self.spec.out_bias else None)
+        self.out.set(take(tensors, f"{p}.o_proj.weight"), take(tensors, f"{p}.o_proj.bias") if self.spec.out_bias else None)
 
     def forward(self, ctx, h, cache):
         s, n, ws = self.spec, ctx.n_tokens, ctx.workspace

@@ -14,8 +14,10 @@ import math
 
 import numpy as np
 
-#: compute units; a unit runs one block of the decode kernel at a time, or two
-DECODE_UNITS = 256
+#: compute units of the device that is planned for when nobody says (an MI355X). An engine reads
+#: its device's number once (``Runtime.compute_units``) and plans with it; a unit runs one block of
+#: the decode kernel at a time, or two
+DEFAULT_UNITS = 256
 #: keys per chunk of the decode kernel, and the fewest chunks a block is given if its request has them
 DECODE_CHUNK = 32
 DECODE_MIN_CHUNKS_PER_BLOCK = 8
@@ -32,27 +34,27 @@ def decode_items(nq: int, nkv: int) -> int:
     return nkv * -(-(nq // nkv) // 16)
 
 
-def decode_alone(rows: int, nq: int, nkv: int) -> bool:
+def decode_alone(rows: int, nq: int, nkv: int, units: int = DEFAULT_UNITS) -> bool:
     """Whether a step of ``rows`` single-token requests runs one block per compute unit: a
     block for every request and item then fits the chip at once. (Measured on the 7B heads:
     64 requests of 4,096 tokens take 79 us that way and 87 to 115 us with two blocks a unit,
     which the dispatcher does not spread evenly; 256 requests take 405 and 332 us.)"""
-    return rows * decode_items(nq, nkv) <= DECODE_UNITS
+    return rows * decode_items(nq, nkv) <= units
 
 
-def _decode_slots(rows: int, nq: int, nkv: int) -> int:
+def _decode_slots(rows: int, nq: int, nkv: int, units: int = DEFAULT_UNITS) -> int:
     """Blocks per item that run at once."""
-    at_once = DECODE_UNITS if decode_alone(rows, nq, nkv) else 2 * DECODE_UNITS
+    at_once = units if decode_alone(rows, nq, nkv, units) else 2 * units
     return max(1, at_once // decode_items(nq, nkv))
 
 
-def decode_capacity(rows: int, nq: int, nkv: int) -> int:
+def decode_capacity(rows: int, nq: int, nkv: int, units: int = DEFAULT_UNITS) -> int:
     """Blocks that the work list of a step with ``rows`` single-token requests can come to."""
-    return rows + 2 * _decode_slots(rows, nq, nkv) + 1
+    return rows + 2 * _decode_slots(rows, nq, nkv, units) + 1
 
 
 def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: int, nq: int, nkv: int,
-                size: int | None = None) -> np.ndarray:
+                size: int | None = None, units: int = DEFAULT_UNITS) -> np.ndarray:
     """The decode kernel's work list (int32 ``[1 + blocks, 4]``) for the single tokens
     ``tokens`` (flat indices) at ``positions``, planned as for ``rows`` requests (the rounded
     number: the missing ones count as requests of one chunk, which is what the padding of a
@@ -75,7 +77,7 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
     chunks = pos // DECODE_CHUNK - lo // DECODE_CHUNK + 1
     padding = max(0, rows - n)
     total, longest = int(chunks.sum()) + padding, int(chunks.max())
-    slots = _decode_slots(rows, nq, nkv)
+    slots = _decode_slots(rows, nq, nkv, units)
     if size is None:
         size = -(-total // (2 * slots))  # many rounds: half a slot's share
         least = DECODE_MIN_CHUNKS_MANY_ROUNDS
@@ -152,7 +154,8 @@ def _time_of(chunks: np.ndarray, size: int, slots: int) -> float:
     return float(loads.max())
 
 
-def prefill_work(tiles: np.ndarray, positions: np.ndarray, window: int, items: int, size: int | None = None) -> np.ndarray:
+def prefill_work(tiles: np.ndarray, positions: np.ndarray, window: int, items: int, size: int | None = None,
+                 units: int = DEFAULT_UNITS) -> np.ndarray:
     """The prompt-portion kernel's work list (int32 ``[blocks, 8]``) for ``tiles`` ([T, 2]:
     first token, count) at ``positions``; ``items`` blocks run per tile and chunk range.
 
@@ -174,7 +177,7 @@ def prefill_work(tiles: np.ndarray, positions: np.ndarray, window: int, items: i
     chunks = last - first + 1
     order = np.argsort(-chunks, kind="stable")
     n, longest = len(tiles), int(chunks.max())
-    slots = max(1, DECODE_UNITS // items)
+    slots = max(1, units // items)
     if size is None:
         size = longest
         if n < 4 * slots:  # with many tiles the units stay busy to the end anyway
@@ -201,6 +204,12 @@ def prefill_work(tiles: np.ndarray, positions: np.ndarray, window: int, items: i
     work[:, 3] = np.minimum(last[src], work[:, 2] + per[src] - 1)
     work[:, 4], work[:, 5], work[:, 6] = slot0, b, nb_sorted[which]
     return work
+
+
+def prefill_capacity(max_tokens: int, max_seqs: int, tile: int, items: int, units: int = DEFAULT_UNITS) -> int:
+    """Blocks that the work list of a step of up to ``max_tokens`` tokens in ``max_seqs`` requests can
+    come to: its tiles, and the two rounds of blocks more that :func:`prefill_work` allows itself."""
+    return max_tokens // tile + max_seqs + 2 * max(1, units // items) + 1
 
 
 def prefill_slots(work: np.ndarray) -> int:

@@ -23,8 +23,12 @@ Interfaces (duck-typed; the base classes document them):
 ``PositionEncoding``  ``rotary(runtime) -> (cos, sin, rotary_dim)`` tables indexed by
                   absolute position for mixers that rotate queries and keys, or
                   ``rotary_dim = 0`` for none.
-``Block``         ``forward(ctx, state, cache)`` arranges the four above around the
-                  residual stream.
+``Block``         ``forward(ctx, state, caches)`` arranges the four above around the
+                  residual stream; ``cache_specs()`` lists what the block keeps (one
+                  description per cache: a block with one mixer has its mixer's, a block
+                  with two has two, in the order in which ``forward`` receives their
+                  views) and ``step_arrays()`` what its parts want of every step. The
+                  model asks the block, never the parts inside it.
 """
 
 from __future__ import annotations
@@ -101,6 +105,10 @@ class PagedCacheSpec:
 
     tensors: tuple[PagedTensorSpec, ...]
     window: int = 0
+    #: tokens per page that this mixer's kernels need, if they need a particular number; None:
+    #: whatever the engine is set to. All page groups of an engine share one page size, so an
+    #: engine set to another size refuses the model when it is built.
+    page_size: int | None = None
 
     kind: ClassVar[str] = "paged"
 
@@ -110,6 +118,8 @@ class PagedCacheSpec:
             raise ValueError("a paged cache needs at least one tensor, each with a name of its own")
         if self.window < 0:
             raise ValueError("window must not be negative")
+        if self.page_size is not None and self.page_size <= 0:
+            raise ValueError("page_size must be positive")
 
 
 @dataclass(frozen=True)
@@ -121,6 +131,30 @@ class StateCacheSpec:
     dtype: str = "float32"
 
     kind: ClassVar[str] = "state"
+
+
+# --------------------------------------------------------------------------- the checkpoint's tensors at bind time
+
+
+class TensorBag(dict):
+    """The checkpoint's tensors while the parts take theirs. ``uses[name]`` counts the parts
+    that named the tensor in their ``tensor_specs``; :func:`take` hands a tensor out and, when
+    the last of them has come for it, drops it from the bag, so that a part which copies its
+    tensors (a fused weight) does not keep the originals alive until the whole model is bound."""
+
+    def __init__(self, tensors: dict, uses: dict[str, int]):
+        super().__init__(tensors)
+        self.uses = dict(uses)
+
+
+def take(tensors: dict, name: str):
+    """``tensors[name]``; out of the bag with it if nobody else is going to ask. With a plain
+    dictionary this is ``tensors[name]`` and nothing more."""
+    uses = getattr(tensors, "uses", None)
+    if uses is None or name not in uses:
+        return tensors[name]
+    uses[name] -= 1
+    return tensors.pop(name) if uses[name] <= 0 else tensors[name]
 
 
 # --------------------------------------------------------------------------- part classes
@@ -183,6 +217,21 @@ class Norm(Part):
 class PositionEncoding(Part):
     def rotary(self, runtime):
         return None, None, 0
+
+
+class Block(Part):
+    """A layer: parts arranged around the residual stream. ``forward`` receives one cache view
+    per description of ``cache_specs()``, in that order (or the views of the entry whose caches
+    this call reads, ``LayerCall.cache_from``)."""
+
+    def cache_specs(self) -> list:
+        return []
+
+    def step_arrays(self) -> list[StepArraySpec]:
+        return []
+
+    def forward(self, ctx, state, caches: list) -> None:
+        raise NotImplementedError
 
 
 # --------------------------------------------------------------------------- registry of parts

@@ -7,7 +7,7 @@ from dataclasses import dataclass
 import torch
 
 from pyre_amd.hip.ops import Partials
-from pyre_amd.parts.base import BlockSpec, Part, TensorSpec, make_part
+from pyre_amd.parts.base import Block, BlockSpec, TensorSpec, make_part
 
 
 @dataclass
@@ -19,7 +19,7 @@ class Hidden:
     pending: Partials | None = None
 
 
-class PreNormBlock(Part):
+class PreNormBlock(Block):
     """x += mixer(norm1(x)); x += feed_forward(norm2(x))."""
 
     def __init__(self, spec: BlockSpec):
@@ -42,9 +42,16 @@ class PreNormBlock(Part):
     def linears(self) -> list:
         return [lin for p in self.parts() for lin in p.linears()]
 
-    def forward(self, ctx, state: Hidden, cache) -> None:
+    def cache_specs(self) -> list:
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def step_arrays(self) -> list:
+        return self.mixer.step_arrays()
+
+    def forward(self, ctx, state: Hidden, caches: list) -> None:
         h = ctx.workspace.get("block.h", (ctx.n_tokens, state.resid.shape[1]), ctx.dtype)
         self.mixer_norm.forward(ctx, state.resid, state.pending, h)
-        mixed = self.mixer.forward(ctx, h, cache)
+        mixed = self.mixer.forward(ctx, h, caches[0] if caches else None)
         self.feed_forward_norm.forward(ctx, state.resid, mixed, h)
         state.pending = self.feed_forward.forward(ctx, h)

@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import torch
 
-from pyre_amd.hip.ops import Partials
+from pyre_amd.hip.ops import DEFAULT_UNITS, Partials
 
 #: most rows the weight-streaming MFMA kernel takes; above, 16-bit products go to the kernel that keeps
 #: up to 256 rows in a block where it pays and else to the BLAS library
@@ -33,14 +33,20 @@ MID_SILU_MIN_ROWS = 1
 MID_WIDE_MIN_ROWS = 25
 
 
-def skinny_ksplit(m: int, n_out: int, k: int) -> int:
+#: what the weight-streaming products reach while they stream, measured on the 7B shapes on an
+#: MI355X, in bytes per microsecond over the whole chip; the time of one run of 128 k of a block
+#: and of one more addend in the consumer, in microseconds
+STREAM_BYTES_PER_US, STREAM_RUN_US, STREAM_PART_US = 6.5e6, 0.9, 0.1
+
+
+def skinny_ksplit(m: int, n_out: int, k: int, units: int = DEFAULT_UNITS) -> int:
     """Into how many parts of k to split a weight-streaming product. A block (64 rows of the
     weights, 128 of wide ones) walks its part of k in dependent runs of 128, about 0.9 us
     each, and the blocks of a compute unit share its time: the product takes as long as the
     longest walk or as the unit with the most blocks needs for its bytes (6.5 TB/s over the
-    256 units, measured on the 7B shapes), whichever is more; every part costs its consumer
+    ``units`` compute units), whichever is more; every part costs its consumer
     one more addend. The split with the least of that is chosen, at least four runs a part."""
-    units, run_us, bytes_per_us, part_us = 256, 0.9, 6.5e6, 0.1
+    run_us, bytes_per_us, part_us = STREAM_RUN_US, STREAM_BYTES_PER_US, STREAM_PART_US
     tiles = -(-n_out // 16)
     row_blocks = -(-n_out // (128 if tiles >= 2048 else 64))
     runs = -(-k // 128)
@@ -60,16 +66,16 @@ def skinny_ksplit(m: int, n_out: int, k: int) -> int:
     return best
 
 
-def mid_ksplit(n_out: int, k: int, block_rows: int = 64) -> int:
+def mid_ksplit(n_out: int, k: int, block_rows: int = 64, units: int = DEFAULT_UNITS) -> int:
     """Into how many parts of k the kernel that keeps a step's rows in a block (up to 256) splits a
     product, or 0 if it is not the one to take. A block has 64 rows of the weights; the kernel is at its best when the blocks
-    of all parts fill the 256 compute units in one round, and beats the BLAS library where that
+    of all parts fill the ``units`` compute units in one round, and beats the BLAS library where that
     takes at least two parts of 384 k or more (shorter parts gain nothing and cost the consumer
     another addend; measured on the 1.5B, 7B and 32B shapes: q/k/v, the
     attention output and the feed-forward's way down take 9 to 20 us where the library takes 19
     to 31, and 60 against 100 at 7B's way down; the wide gate/up product stays with the library)."""
     blocks = -(-n_out // block_rows)
-    ks = min(256 // blocks, k // 384, MID_MAX_KSPLIT)
+    ks = min(units // blocks, k // 384, MID_MAX_KSPLIT)
     while ks > 1 and (ks - 1) * (-(-(-(-k // ks)) // 64) * 64) >= k:
         ks -= 1  # would leave a part empty
     return ks if ks >= 2 else 0
@@ -87,11 +93,13 @@ def _is_bf16(ctx, lin, x) -> bool:
             and x.dtype == torch.bfloat16)
 
 
-def narrow_kernel(n: int, n_out: int, k: int, options: dict | None = None) -> tuple[str, int, bool]:
+def narrow_kernel(n: int, n_out: int, k: int, options: dict | None = None,
+                  units: int = DEFAULT_UNITS) -> tuple[str, int, bool]:
     """Which of our kernels takes a 16-bit product of ``n`` rows whose result is handed on as partial
     sums: ("stream", parts of k, False) for the weight-streaming kernel, ("block", parts, wide) for the
     kernel that keeps the step's rows in a block (``wide``: 128 rows of the weights a block instead
-    of 64), ("", 0, False) for neither (the BLAS library then). A function of the sizes alone; the
+    of 64), ("", 0, False) for neither (the BLAS library then). A function of the sizes (and of the
+    device's compute units, which an engine reads once) alone; the
     thresholds in rows lie just above sizes at which decode steps are captured, so that an eager step
     and its replay at the padded size agree."""
     opt = options or {}
@@ -108,21 +116,21 @@ def narrow_kernel(n: int, n_out: int, k: int, options: dict | None = None) -> tu
         # and 16: 3.46 against 3.44, 3.79 against 3.77); of the 32B shape 35.5 against 36.2 at 64.
         # Against 64 rows of the weights a block: 7.78 against 7.94 ms at 96 requests, 8.86 against
         # 8.90 at 128, 12.56 against 12.63 at 192, 15.25 against 15.34 at 256.
-        ks = mid_ksplit(n_out, k, 128)
-        if ks and -(-n_out // 128) * ks >= 192:
+        ks = mid_ksplit(n_out, k, 128, units)
+        if ks and 4 * -(-n_out // 128) * ks >= 3 * units:
             return "block", ks, True
     if n <= SKINNY_MAX_ROWS and opt.get("skinny_gemm", True):
-        ks = skinny_ksplit(n, n_out, k)
-        if block and opt.get("mid_small", True) and -(-n_out // 64) * ks < 256 and mid_ksplit(n_out, k):
+        ks = skinny_ksplit(n, n_out, k, units)
+        if block and opt.get("mid_small", True) and -(-n_out // 64) * ks < units and mid_ksplit(n_out, k, 64, units):
             # A product so small that the weight-streaming kernel's blocks do not fill the compute
             # units (the 1.5B shape's: 96, 72 and 240 blocks) is latency all the way, and the other
             # kernel, whose loads go straight into a ring in LDS, starts sooner: 1.7 % of a step of
             # 8 requests of that shape, 3 % at 32, 4 % at 64. Where the blocks fill the chip (7B:
             # 504) it is 3 % slower at 8 rows.
-            return "block", mid_ksplit(n_out, k), False
+            return "block", mid_ksplit(n_out, k, 64, units), False
         return "stream", ks, False
     if n <= MID_MAX_ROWS and block:
-        ks = mid_ksplit(n_out, k)
+        ks = mid_ksplit(n_out, k, 64, units)
         if not ks and int(block) == 2:  # tests: also where it does not pay, as with a tiny model
             ks = 2 if k > 64 else 1
         if ks:
@@ -151,11 +159,11 @@ def linear(lin, ctx, x, n, out):
         else:
             return None
         return Partials(out.view(1, n, n_out), lin.bias)
-    kernel, ks, wide = narrow_kernel(n, n_out, k, rt.options)
+    kernel, ks, wide = narrow_kernel(n, n_out, k, rt.options, rt.compute_units)
     if kernel == "stream" and not streams:
         kernel = ""
     if kernel == "block" and not ops.gemm_mid_supports(n, n_out, k, x.stride(0), lin.weight.stride(0)):
-        kernel, ks = ("stream", skinny_ksplit(n, n_out, k)) if streams and n <= SKINNY_MAX_ROWS else ("", 0)
+        kernel, ks = ("stream", skinny_ksplit(n, n_out, k, rt.compute_units)) if streams and n <= SKINNY_MAX_ROWS else ("", 0)
     if kernel:
         buf = ctx.workspace.get(f"linear.{lin.role}.partials", (ks, n, n_out), torch.float32)
         if kernel == "stream":
@@ -193,7 +201,7 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
         # 4.46 against 4.56 at 32, 5.87 against 6.13 at 64; on the 1.5B shape by 1 to 4 %.
         mid = ctx.runtime.options.get("mid_gemm", True)
         fits = mid and ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0))
-        if fits and (ops.gemm_mid_silu_blocks(n, lin.out_features) <= 256 or int(mid) == 2):
+        if fits and (ops.gemm_mid_silu_blocks(n, lin.out_features) <= ctx.runtime.compute_units or int(mid) == 2):
             ops.gemm_mid_silu_bf16(x, lin.weight, act, n)
             return True
     if n > FUSED_SILU_MAX_ROWS or not ctx.runtime.options.get("skinny_gemm", True):
@@ -229,18 +237,25 @@ def attention(mixer, ctx, q, o, cache) -> bool:
         # number of requests, so that a step gives bit for bit the same result whether it runs
         # eagerly or as a replayed graph at those sizes.
         rows, _ = hb.decode_shape()
-        capacity = decode_capacity(rows, s.num_heads, s.num_kv_heads)
+        units = mixer.units
+        capacity = decode_capacity(rows, s.num_heads, s.num_kv_heads, units)
+        listed_blocks = int(hb.arrays[mixer.decode_work_name].reshape(-1)[0])
+        if listed_blocks > capacity:  # the kernel would leave the rest of the list undone, silently
+            raise RuntimeError(f"the decode attention's work list has {listed_blocks} blocks, its launch {capacity}")
         items = decode_items(s.num_heads, s.num_kv_heads)
         acc = ctx.workspace.get("attn.part_acc", (capacity, items, 16, s.head_dim), torch.float32)
         ml = ctx.workspace.get("attn.part_ml", (capacity, items, 16, 2), torch.float32)
         counters = ctx.workspace.get("attn.counters", (capacity, items), torch.int32, zeroed=True)
         ops.attn_decode_work_bf16(q, o, k_pages, v_pages, ctx.arrays[mixer.decode_work_name], capacity, ctx.positions,
                                   ctx.seq_of_token, cache.table, acc, ml, counters,
-                                  decode_alone(rows, s.num_heads, s.num_kv_heads), s.num_heads, s.num_kv_heads,
+                                  decode_alone(rows, s.num_heads, s.num_kv_heads, units), s.num_heads, s.num_kv_heads,
                                   s.head_dim, cache.page_size, mixer.scale, cache.window)
     if n_tiles and s.head_dim <= 128:
         work = hb.arrays[mixer.prefill_work_name]
         n_slots = prefill_slots(work)
+        if 8 * len(work) > ctx.arrays[mixer.prefill_work_name].numel():
+            raise RuntimeError(f"the prompt attention's work list has {len(work)} blocks, its step array holds "
+                               f"{ctx.arrays[mixer.prefill_work_name].numel() // 8}")
         per_slot = prefill_items(s.num_heads, s.num_kv_heads) * ops.attn_prefill_waves(s.num_heads, s.num_kv_heads)
         partials = counters = None
         if n_slots:

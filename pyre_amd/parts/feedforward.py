@@ -6,7 +6,7 @@ import torch
 
 from pyre_amd.hip import ops
 from pyre_amd.parts import fast
-from pyre_amd.parts.base import FeedForward, SwiGLUSpec, TensorSpec
+from pyre_amd.parts.base import FeedForward, SwiGLUSpec, TensorSpec, take
 from pyre_amd.parts.linear import Linear, linear_specs
 
 
@@ -26,8 +26,11 @@ class SwiGLU(FeedForward):
 
     def bind(self, tensors, runtime) -> None:
         p = self.spec.prefix
-        self.gate_up.set(torch.cat([tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]], dim=0))
-        self.down.set(tensors[f"{p}.down_proj.weight"])
+        halves = [take(tensors, f"{p}.gate_proj.weight"), take(tensors, f"{p}.up_proj.weight")]
+        fused = torch.cat(halves, dim=0)
+        del halves  # the two weights are free before the next layer makes its copy
+        self.gate_up.set(fused)
+        self.down.set(take(tensors, f"{p}.down_proj.weight"))
 
     def linears(self) -> list:
         return [self.gate_up, self.down]

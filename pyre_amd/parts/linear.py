@@ -41,7 +41,7 @@ class Linear:
         f32 = x.dtype == torch.float32 and self.weight.dtype == torch.float32
         if f32 and out is None:
             # the true 32-bit path: the matrix cores' float32 instruction, k split by the weight's shape alone
-            ks = ops.gemm_f32_ksplit(self.out_features, self.in_features)
+            ks = ops.gemm_f32_ksplit(self.out_features, self.in_features, ctx.runtime.compute_units)
             buf = ctx.workspace.get(f"linear.{self.role}", (ks, n, self.out_features), torch.float32)
             ops.gemm_f32(x, self.weight, None, buf if ks > 1 else buf[0], n, ks)
             return Partials(buf, self.bias)

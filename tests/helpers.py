@@ -13,6 +13,38 @@ import plain_qwen2 as P
 TOL = {"float32": 1e-5, "bfloat16": 2e-2}
 
 
+def depth_tol(dtype: str, layers: int) -> float:
+    """The bound for a model of ``layers`` layers, fixed before any run of such a model: the
+    bounds above are those of the tiny models (up to three layers); every layer adds rounding
+    noise of its own, independent of the others', so the bound grows with the square root of
+    the depth (28 layers: 3.1e-5 and 6.1e-2)."""
+    return TOL[dtype] * max(1.0, (layers / 3) ** 0.5)
+
+
+def layer_report(engine, plain, ids, rounding=None) -> list[tuple[int, float]]:
+    """(entry of the layer order, max |hidden - plain hidden| / scale of the plain rows) for one
+    request fed whole through ``engine`` (which must not know the request "__layers" yet), the
+    way `scripts/diagnose_parity.py:103-120` of the reference walks its layers."""
+    from pyre_amd.engine.batch import Entry
+
+    cfg, w = plain
+    _, hidden = P.forward(w, cfg, ids, rounding=rounding, return_hidden=True)
+    seen = {}
+    engine.step([Entry("__layers", list(ids), [])], tap=lambda pos, rows: seen.__setitem__(pos, rows.double().cpu()))
+    engine.finish("__layers")
+    out = []
+    for pos, ref in enumerate(hidden):
+        ref = ref.double().cpu()
+        out.append((pos, float((seen[pos] - ref).abs().max() / ref.abs().max().clamp_min(1e-30))))
+    return out
+
+
+def first_layer_off(report, tol: float) -> str:
+    """One line naming the first layer whose hidden rows leave ``tol``, and every layer's figure."""
+    bad = next((f"first layer outside {tol:.1e}: {pos}" for pos, d in report if not d <= tol), f"no layer is outside {tol:.1e}")
+    return bad + "; per layer: " + " ".join(f"{pos}:{d:.1e}" for pos, d in report)
+
+
 def random_ids(vocab: int, n: int, seed: int) -> list[int]:
     rng = random.Random(seed)
     return [rng.randrange(vocab) for _ in range(n)]
@@ -96,3 +128,20 @@ def cut(n: int, sizes: list[int]) -> list[int]:
         n -= s
         i += 1
     return out
+
+
+def check_greedy(plain, prompt: list[int], tokens: list[int], tol: float) -> int:
+    """Every generated token against the plain implementation's argmax given the tokens before
+    it. A token may differ only where the plain logits leave the choice to rounding (the two
+    within ``tol`` of the logit scale); returns how many did."""
+    cfg, w = plain
+    ids, near = list(prompt), 0
+    for k, tok in enumerate(tokens):
+        row = P.forward(w, cfg, ids)[-1]
+        twin = int(row.argmax())
+        if twin != tok:
+            margin = float((row[twin] - row[tok]) / row.abs().max())
+            assert margin < tol, f"token {k} is {tok}, the plain implementation gives {twin} (margin {margin:.2e})"
+            near += 1
+        ids.append(tok)
+    return near

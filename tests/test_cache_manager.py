@@ -143,6 +143,31 @@ def test_layers_with_the_same_needs_share_a_group():
     assert m.bytes_per_page(2) == 2 * (2 * 2 * 16 * 16 * 2) * 2
 
 
+def test_an_entry_may_keep_several_caches():
+    """A layer with two mixers keeps two caches: the entry's description is a list, and a cell
+    is (entry, place in that list)."""
+    state = StateCacheSpec((4, 8))
+    specs = [[FULL, state], [], [WIN], None, [FULL, FULL]]
+    m = CacheManager(specs, 16, 10, 4, 512)
+    assert [g.cells for g in m.page_groups] == [[(0, 0), (4, 0), (4, 1)], [(2, 0)]]
+    assert [g.cells for g in m.state_groups] == [[(0, 1)]]
+    assert [m.caches_of_entry(e) for e in range(5)] == [2, 0, 1, 0, 2]
+    assert m.group_of_cell[(4, 1)] == ("paged", 0) and m.page_groups[0].layer_index(4, 1) == 2
+    assert m.group_of_entry == {0: ("paged", 0), 2: ("paged", 1), 4: ("paged", 0)}
+    assert m.bytes_per_page(2) == (3 + 1) * (2 * 2 * 16 * 16 * 2)
+
+
+def test_a_cache_that_needs_pages_of_another_size_is_refused():
+    """All page groups share the engine's page size; a mixer whose kernels need another says so
+    in its description and is refused when the manager is made, not at its first step."""
+    needs_32 = PagedCacheSpec((PagedTensorSpec("k", (2, 16), token_axis=1),), page_size=32)
+    CacheManager([FULL, needs_32], 32, 10, 4, 512)
+    with pytest.raises(ValueError, match="pages of 32 tokens.*set to pages of 16"):
+        CacheManager([FULL, needs_32], 16, 10, 4, 512)
+    with pytest.raises(ValueError, match="positive"):
+        PagedCacheSpec((PagedTensorSpec("k", (2, 16)),), page_size=0)
+
+
 def test_a_window_gives_pages_back_once_passed():
     m = CacheManager([FULL, WIN], 16, 12, 2, 512)
     m.add_request("a")

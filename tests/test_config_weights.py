@@ -251,3 +251,41 @@ def test_model_spec_is_data():
     assert spec.head.tied_to is None
     assert get_architecture("Qwen2ForCausalLM").build(preset("tiny-a")).head.tied_to == "model.embed_tokens.weight"
     json.dumps(preset("tiny-a").to_dict())
+
+
+def test_sizes_that_no_kernel_takes_are_refused_when_the_model_is_built():
+    """A head of more than 256 elements is refused by the attention part's constructor, before
+    any weight is read (no attention kernel takes it), with a message that names the size."""
+    from pyre_amd.parts.model import LayeredModel
+
+    cfg = config_from_dict({"architectures": ["Qwen2ForCausalLM"], "hidden_size": 64, "intermediate_size": 32,
+                            "num_hidden_layers": 1, "num_attention_heads": 2, "vocab_size": 50, "head_dim": 288})
+    with pytest.raises(ValueError, match="head_dim 288 is outside 1..256"):
+        LayeredModel(get_architecture(cfg.architecture).build(cfg))
+    ok = config_from_dict({"architectures": ["Qwen2ForCausalLM"], "hidden_size": 64, "intermediate_size": 32,
+                           "num_hidden_layers": 1, "num_attention_heads": 2, "vocab_size": 50, "head_dim": 256})
+    assert LayeredModel(get_architecture(ok.architecture).build(ok)).cache_specs()[0][0].tensors[0].token_shape == (2, 256)
+
+
+def test_parts_take_their_tensors_and_let_the_originals_go():
+    """Binding empties the dictionary it is given, and a tensor that its part copies (the fused
+    q/k/v and gate/up weights) is dropped as soon as it has been copied: nothing but the model
+    holds the weights afterwards."""
+    import weakref
+
+    from pyre_amd.parts.base import TensorBag, take
+    from pyre_amd.parts.model import LayeredModel
+
+    cfg = preset("tiny-b")
+    model = LayeredModel(get_architecture(cfg.architecture).build(cfg))
+    state = random_state(model.tensor_specs(), 0, dtype="float32")
+    refs = {n: weakref.ref(t) for n, t in state.items()}
+    model.bind(state, None)
+    assert state == {}
+    fused = [n for n in refs if any(k in n for k in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj"))]
+    assert len(fused) == 3 * 8 and all(refs[n]() is None for n in fused)           # copied, then let go
+    assert refs["model.layers.0.mlp.down_proj.weight"]() is model.layers[0].feed_forward.down.weight
+    # a tensor that two parts name stays until the second has it
+    bag = TensorBag({"w": 1, "v": 2}, {"w": 2, "v": 1})
+    assert take(bag, "w") == 1 and "w" in bag and take(bag, "w") == 1 and "w" not in bag
+    assert take(bag, "v") == 2 and not bag and take({"x": 3}, "x") == 3

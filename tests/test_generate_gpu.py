@@ -234,18 +234,50 @@ def test_preemption_recomputes_and_gives_the_same_tokens(model_dirs):
     assert outs[0] == outs[1]
 
 
-def test_cli_generates(model_dirs, tmp_path, capsys):
+def test_cli_generates(model_dirs, plain_models, tmp_path, capsys):
+    """The command line's tokens are the plain implementation's greedy tokens."""
+    from helpers import check_greedy
     from pyre_amd.cli import main
 
     out = tmp_path / "res.json"
-    rc = main(["--model", str(model_dirs["tiny-a"]), "--dtype", "float32", "--prompt-ids", "5,17,3",
-               "--prompt-ids", "9", "--max-new-tokens", "5", "--max-batch", "4", "--num-blocks", "32",
+    rc = main(["--model", str(model_dirs["tiny-b"]), "--dtype", "float32", "--prompt-ids", "5,17,3",
+               "--prompt-ids", "9", "--max-new-tokens", "6", "--max-batch", "4", "--num-blocks", "32",
                "--out", str(out)])
     assert rc == 0
     import json
 
     res = json.loads(out.read_text())
-    assert [len(g) for g in res["generated"]] == [5, 5]
+    assert res["prompts"] == [[5, 17, 3], [9]] and [len(g) for g in res["generated"]] == [6, 6]
+    for prompt, tokens in zip(res["prompts"], res["generated"]):
+        assert check_greedy(plain_models["tiny-b"], prompt, tokens, 1e-5) == 0
+    printed = capsys.readouterr().out.splitlines()
+    assert printed[0] == "request 0: prompt of 3 tokens -> " + ",".join(map(str, res["generated"][0]))
+
+
+def test_the_generate_program_as_a_process(model_dirs, plain_models, tmp_path):
+    """``bin/pyre_generate`` as a user starts it: a process of its own, the reference's spellings
+    of the options (``--tokens``), a JSON result file; its tokens against the plain implementation."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from helpers import check_greedy
+
+    root = Path(__file__).resolve().parent.parent
+    out = tmp_path / "res.json"
+    proc = subprocess.run([sys.executable, str(root / "bin" / "pyre_generate"), "--model", str(model_dirs["tiny-c"]),
+                           "--dtype", "bfloat16", "--prompt-ids", "700,3,3,41,9,100,5", "--tokens", "5",
+                           "--num-blocks", "16", "--max-batch", "2", "--out", str(out)],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    res = json.loads(out.read_text())
+    assert res["dtype"] == "bfloat16" and len(res["generated"][0]) == 5
+    assert proc.stdout.splitlines()[0] == "request 0: prompt of 7 tokens -> " + ",".join(map(str, res["generated"][0]))
+    assert check_greedy(plain_models["tiny-c"], res["prompts"][0], res["generated"][0], 4e-2) <= 1
+    bad = subprocess.run([sys.executable, str(root / "bin" / "pyre_generate"), "--model", str(tmp_path / "nothing")],
+                         capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "neither a model folder nor a preset" in bad.stderr
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

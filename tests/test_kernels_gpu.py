@@ -712,6 +712,49 @@ def test_attention_at_a_windows_edge(kernel):
         assert not torch.allclose(out2.double().cpu(), want.expand(n, nq, hd), atol=0.2)
 
 
+@pytest.mark.parametrize("kernel", ["generic32", "generic16", "decode", "decode256", "prefill", "prefill256", "prefill32"])
+@pytest.mark.parametrize("ctx_len", [700, 689, 655])
+def test_attention_ignores_what_a_page_held_before(kernel, ctx_len):
+    """A request's last page is only partly its own: the slots past its last key still hold what
+    the page's previous owner wrote, which may be NaN or Inf (a request that diverged). A kernel
+    that loads whole chunks and weights the hidden keys with 0 must not let such a value through
+    (0 * NaN is NaN). Contexts that end 4, 15 and 1 keys before the end of a 16-key page; pages that the request
+    does not hold are NaN as well."""
+    ops = _ops()
+    big = kernel.endswith("256")
+    nq, nkv, hd, page = (4, 2, 256, 16) if big else (8, 2, 64, 16)
+    dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
+    ql = 34 if kernel.startswith("prefill") else 1
+    ctx_lens, q_lens = [ctx_len, 40], [ql, min(ql, 3)]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=17)
+    held = set(table[table >= 0].tolist())
+    for p in range(kc.shape[0]):
+        if p not in held:
+            kc[p], vc[p] = float("nan"), float("inf")
+    for s, c in enumerate(ctx_lens):                       # the tail of each request's last page
+        last = int(table[s, (c - 1) // page])
+        kc[last, :, c % page or page:, :] = float("nan")
+        vc[last, :, :, c % page or page:] = float("nan")
+        if c % page:
+            vc[last, 0, :, c % page] = float("inf")           # and an infinity right behind the last key
+    scale = hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale)
+    out = torch.zeros_like(q)
+    n = q.shape[0]
+    tiles = [(0, 32), (32, 2), (34, 3)]
+    if kernel.startswith("generic"):
+        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, 0)
+    elif kernel.startswith("decode"):
+        decode_attention(ops, q, out, kc, vc, [0, 1], pos, seq_of, table, nq, nkv, hd, page, scale)
+    elif kernel == "prefill32":
+        ops.attn_prefill_f32(q, out, kc, vc, i32([t for tile in tiles for t in tile]), 3, pos, seq_of, table, nq, nkv, hd, page, scale, 0)
+    else:
+        prefill_attention(ops, q, out, kc, vc, tiles, pos, seq_of, table, nq, nkv, hd, page, scale)
+    assert torch.isfinite(out.float()).all(), kernel
+    tol = 2e-5 if dt == torch.float32 else 2e-2
+    assert torch.allclose(out.double().cpu(), want, atol=tol, rtol=tol), kernel
+
+
 # ----------------------------------------------------------------------------- sampling
 
 def test_argmax_first_of_equals():

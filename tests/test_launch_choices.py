@@ -6,7 +6,7 @@ import random
 
 import numpy as np
 
-from pyre_amd.parts.attention_work import (DECODE_MAX_BLOCKS_PER_REQUEST, DECODE_UNITS, decode_alone, decode_capacity,
+from pyre_amd.parts.attention_work import (DECODE_MAX_BLOCKS_PER_REQUEST, DEFAULT_UNITS, decode_alone, decode_capacity,
                                            decode_work, prefill_slots, prefill_work)
 from pyre_amd.parts.fast import SKINNY_MAX_KSPLIT, skinny_ksplit
 
@@ -127,7 +127,7 @@ def test_prefill_work_lists_cover_every_chunk_once():
             tiles += [(t0, min(32, base + n - t0)) for t0 in range(base, base + n, 32)]
         tiles, positions = np.asarray(tiles, dtype=np.int32), np.asarray(positions, dtype=np.int32)
         work = prefill_work(tiles, positions, window, items)
-        assert len(work) <= len(tiles) + 2 * DECODE_UNITS
+        assert len(work) <= len(tiles) + 2 * DEFAULT_UNITS
         seen, slots = {}, set()
         for t0, ntok, c0, c1, slot0, b, nb, _ in work.tolist():
             assert c0 <= c1 and 0 <= b < nb

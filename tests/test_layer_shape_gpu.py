@@ -15,7 +15,8 @@ import pytest
 import torch
 
 import plain_qwen2 as P
-from helpers import TOL, first_bad, make_engine_from_state, plain_logits, random_ids, replay
+from helpers import (TOL, depth_tol, first_bad, first_layer_off, layer_report, make_engine_from_state, plain_logits,
+                     random_ids, replay)
 
 pytestmark = pytest.mark.gpu
 
@@ -167,4 +168,64 @@ def test_decode_steps_of_few_requests_at_the_1p5b_shape():
     assert bad is None, bad
     plain[1].clear()
     state.clear()
+    torch.cuda.empty_cache()
+
+
+# ----------------------------------------------------------------------------- whole models
+
+class _Widened(dict):
+    """The bfloat16 tensors of a whole model, each widened to float64 when the plain implementation
+    asks for it (61 GB of float64 copies at the 7B shape would fit, but nothing needs them at once)."""
+
+    def __getitem__(self, name):
+        return super().__getitem__(name).to(torch.float64)
+
+
+@pytest.mark.parametrize("shape,dtype", [("qwen2.5-7b", "float32"), ("qwen2.5-7b", "bfloat16"),
+                                         ("qwen2.5-1.5b", "float32"), ("qwen2.5-1.5b", "bfloat16")])
+def test_every_layer_of_the_benchmarked_shapes(shape, dtype):
+    """All 28 layers of the Qwen2.5-7B shape (the one that is benchmarked) and of the Qwen2.5-1.5B
+    shape (tied head), the whole vocabulary: a prompt of 48 tokens whole with logits at every
+    position, then the same prompt as a portion of 32 tokens and 16 single tokens, the single
+    tokens from captured graphs from their third step on, every row against the plain
+    implementation in float64 on the device. The bound was fixed before the first run
+    (``helpers.depth_tol``). If a row is off, the message names the first layer whose hidden rows
+    leave the bound (`scripts/diagnose_parity.py:103-120` of the reference walks its layers so)."""
+    from pyre_amd.config import preset
+    from pyre_amd.weights import model_tensor_specs, random_state
+
+    cfg = preset(shape)
+    assert cfg.num_hidden_layers == 28
+    state = random_state(model_tensor_specs(cfg), seed=9, std=0.02, gain_std=0.1, dtype="bfloat16", device=DEV)
+    plain_cfg = {k: getattr(cfg, k) for k in ("hidden_size", "intermediate_size", "num_hidden_layers",
+                                              "num_attention_heads", "num_key_value_heads", "vocab_size",
+                                              "rms_norm_eps", "rope_theta", "tie_word_embeddings", "head_dim")}
+    weights = _Widened(state)
+    if cfg.tie_word_embeddings:
+        assert "lm_head.weight" not in state
+        dict.__setitem__(weights, "lm_head.weight", state["model.embed_tokens.weight"])   # the tied head, as the plain loader has it
+    plain = (plain_cfg, weights)
+    ids = random_ids(cfg.vocab_size, 48, 77)
+    rounding = torch.bfloat16 if dtype == "bfloat16" else None
+    want = {r: plain_logits(plain, ids, rounding) for r in ("whole", "cut")}
+    tol = depth_tol(dtype, cfg.num_hidden_layers)
+    eng = make_engine_from_state(cfg, state, dtype, use_graphs=True, max_cached_tokens=256, max_num_seqs=2,
+                                 max_num_batched_tokens=64, max_model_len=128)
+    steps = [([("whole", ids, list(range(48)))], ["whole"]), ([("cut", ids[:32], list(range(32)))], [])]
+    steps += [([("cut", ids[i:i + 1], [0])], ["cut"] if i == 47 else []) for i in range(32, 48)]
+    got = replay(eng, steps)
+    assert len(got) == 96 and eng.graph_replays >= 14
+    bad, worst = first_bad(got, want, tol)
+    if bad is not None:
+        bad += " | " + first_layer_off(layer_report(eng, plain, ids, rounding), tol)
+    assert bad is None, bad
+    assert all(torch.isfinite(row).all() for row in got.values())
+    # the walk through the layers itself: every layer's hidden rows within the same bound
+    report = layer_report(eng, plain, ids, rounding)
+    assert len(report) == 28 and all(d <= tol for _, d in report), first_layer_off(report, tol)
+    print(f"{shape} {dtype}: worst row {worst:.2e} of the logit scale (bound {tol:.1e}); layers "
+          f"{report[0][1]:.1e} .. {report[-1][1]:.1e}")
+    weights.clear()
+    state.clear()
+    del eng
     torch.cuda.empty_cache()

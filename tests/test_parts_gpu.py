@@ -212,11 +212,11 @@ def test_block_part(dtype):
     w = {s.name: rnd(*s.shape, seed=i, scale=0.2) + (1 if s.init == "gain" else 0) for i, s in enumerate(block.tensor_specs())}
     assert len(w) == 12
     block.bind({k: dev(v, wt) for k, v in w.items()}, None)
-    rig = Rig([block.mixer.cache_spec()], dtype)
+    rig = Rig([block.cache_specs()], dtype)
     ctx, views, _ = rig.context([("a", [0] * n, [])])
     x = rnd(n, H, seed=99)
     state = Hidden(x.to(DEV))
-    block.forward(ctx, state, views[0])
+    block.forward(ctx, state, views)
     got = state.resid.cpu().double() + state.pending.data.float().sum(0).cpu().double()
     cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": hd, "rms_norm_eps": eps}
     cos, sin = P.rope_tables(n, hd, 1e4)

@@ -278,6 +278,38 @@ def test_decode_steps_beyond_the_weight_streaming_kernels(model, dtype, graphs, 
         assert eng.graph_replays == 8      # of each size: once eagerly, then captured and replayed twice
 
 
+@pytest.mark.parametrize("model,dtype", [("tiny-c", "bfloat16"), ("tiny-c", "float32"), ("tiny-b", "bfloat16")])
+def test_decode_steps_of_more_requests_than_a_captured_step_takes(model, dtype, model_dirs, plain_models):
+    """300, then 257 live requests, one token each per step: more rows than the largest captured
+    step (256) and than the kernels that keep a step's rows in a block take. Such a step runs
+    eagerly at its own size, its products in the BLAS library (or the 32-bit tile kernel), the
+    decode attention's list planned for two blocks a compute unit; every row of every step
+    against the plain implementation. Then 256 of them, which is captured again."""
+    plain = plain_models[model]
+    vocab = plain[0]["vocab_size"]
+    prompt = [2 + (17 * i) % 45 for i in range(300)]
+    reqs = {i: random_ids(vocab, n + 8, 2100 + i) for i, n in enumerate(prompt)}
+    want = _expected(plain, reqs, dtype)
+    eng = make_engine(model_dirs[model], dtype, use_graphs=True, max_num_seqs=300, max_cached_tokens=300 * 64,
+                      max_num_batched_tokens=2048)
+    steps = [([(i, reqs[i][:prompt[i]], []) for i in range(lo, lo + 60)], []) for lo in range(0, 300, 60)]
+    live, counts = list(range(300)), (300, 300, 257, 257, 256, 256, 256)
+    for k, keep in enumerate(counts):
+        end = live[keep:]
+        if end:
+            steps[-1] = (steps[-1][0], end)
+        live = live[:keep]
+        steps.append(([(i, [reqs[i][prompt[i] + k]], [0]) for i in live], []))
+    steps[-1] = (steps[-1][0], list(live))
+    got = replay(eng, steps)
+    assert len(got) == sum(counts)
+    bad, worst = first_bad(got, want, TOL[dtype])
+    assert bad is None, bad
+    eng.cache.check_invariants()
+    assert eng.cache.page_groups[0].allocator.num_used == 0
+    assert eng.graph_replays == 2                                    # the steps of 256: once eagerly, then captured and replayed
+
+
 @pytest.mark.parametrize("model,dtype,page", [("tiny-b", "float32", 8), ("tiny-c", "bfloat16", 16), ("tiny-a", "bfloat16", 16)])
 def test_mixed_with_page_reuse_on_poisoned_pages(model, dtype, page, model_dirs, plain_models):
     """The mixed trace again with the debug mode that fills every freed page with NaN: a

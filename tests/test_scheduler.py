@@ -8,6 +8,7 @@ from dataclasses import dataclass
 import pytest
 
 from pyre_amd.cache import CacheManager
+from pyre_amd.cache.allocator import OutOfPages
 from pyre_amd.engine.scheduler import Scheduler
 from pyre_amd.parts.base import PagedCacheSpec, PagedTensorSpec
 
@@ -323,6 +324,67 @@ def test_steps_with_prompt_portions_run_ahead_too():
         assert sum(n for _, n, _ in step) <= 24 and len(step) <= 3
     for rid, (p, g) in enumerate(zip(prompts, ahead)):
         assert eng1.fed[rid] == p + g[:-1]   # no end token here: nothing surplus
+
+
+class FailingAheadEngine(AheadEngine):
+    """Refuses the steps that run ahead whose number is in ``fail_on`` (before it touches the
+    cache, as the real engine's all-or-nothing preparation does)."""
+
+    def __init__(self, fail_on, error, **kw):
+        super().__init__(**kw)
+        self.fail_on, self.error, self.ahead_calls, self.refused = set(fail_on), error, 0, 0
+
+    def step(self, entries, fed_ids=None):
+        if fed_ids is not None:
+            self.ahead_calls += 1
+            if self.ahead_calls in self.fail_on:
+                self.refused += 1
+                raise self.error("the step that ran ahead is refused")
+        return super().step(entries, fed_ids)
+
+
+@pytest.mark.parametrize("error", [OutOfPages, ValueError])
+def test_a_refused_step_ahead_costs_no_token(error):
+    """If the engine refuses the step that was to run ahead, this step's tokens are still
+    collected, the requests that the refused step had admitted wait again in their order, and
+    the next step is planned as usual: the same tokens as without running ahead."""
+    prompts = [[3, 1], [2] * 70, [9, 8, 7], [5] * 90, [6] * 40, [1, 2, 3, 4]]
+    lens = [40, 10, 25, 6, 12, 9]
+
+    def run(fail_on):
+        eng = FailingAheadEngine(fail_on, error, pages=64, max_num_seqs=3, max_num_batched_tokens=24, prefill_chunk=16)
+        s = Scheduler(eng)
+        s.sampler = AheadSampler(s)
+        s.lookahead = True
+        ids = [s.add_request(p, n) for p, n in zip(prompts, lens)]
+        out = s.run()
+        eng.cache.check_invariants()
+        assert eng.cache.free_pages() == 64 and eng.cache.slots.num_used == 0
+        return eng, [out[i] for i in ids]
+
+    eng0, plain = run(())
+    eng1, got = run({1, 2, 5, 11, 12, 30})
+    assert eng1.refused == 6 and eng1.ahead_steps > 10
+    assert got == plain == [expected(p, n) for p, n in zip(prompts, lens)]
+    first_seen = lambda eng: list(dict.fromkeys(rid for step in eng.steps for rid, _, _ in step))  # noqa: E731
+    assert first_seen(eng1) == first_seen(eng0) == list(range(6))      # first come, first served all the same
+
+
+def test_finished_requests_are_handed_over_and_forgotten():
+    eng, s = make(pages=64, max_num_seqs=4)
+    a = s.add_request([1, 2, 3], 4)
+    b = s.add_request([9] * 20, 2)
+    out = s.run()
+    assert out == {a: expected([1, 2, 3], 4), b: expected([9] * 20, 2)}
+    taken = s.take_finished()
+    assert sorted(taken) == [a, b] and taken[a].finish_reason == "length" and not s.finished
+    assert s.take_finished() == {}
+    # a stream driven by step() whose caller never asks: the oldest are dropped beyond the cap
+    s.max_finished_kept = 3
+    ids = [s.add_request([i + 1], 1) for i in range(8)]
+    results = s.run()
+    assert sorted(results) == ids                                       # run() hands every result over all the same
+    assert list(s.finished) == ids[-3:]
 
 
 @pytest.mark.parametrize("seed", range(12))

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import TOL, plain_logits, random_ids
+from helpers import TOL, cut, plain_logits, random_ids
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
@@ -80,3 +80,54 @@ def test_trace_run(model, dtype, extra, model_dirs, plain_models, tmp_path):
             assert d <= TOL[dtype], f"step {st} request {r} position {pos}: {d:.3e}"
             checked += 1
     assert checked > 50
+
+
+def _check(out, wanted, ref, vocab, dtype):
+    checked = 0
+    for st, rows in wanted.items():
+        got = torch.from_numpy(np.fromfile(out / f"{st}.f32", dtype="<f4").reshape(len(rows), vocab))
+        for i, (r, pos) in enumerate(rows):
+            scale = ref[r][pos].abs().max().item()
+            d = (got[i] - ref[r][pos]).abs().max().item() / scale
+            assert d <= TOL[dtype], f"step {st} request {r} position {pos}: {d:.3e}"
+            checked += 1
+    return checked
+
+
+@pytest.mark.parametrize("mode,extra", [("whole", ()), ("tail", ()), ("tail", ("--graphs",)), ("ragged", ())])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_in_the_replay_modes(mode, extra, dtype, model_dirs, plain_models, tmp_path):
+    """The program itself, with its own sizing of the cache from --max-tokens, through the modes
+    that the engine is tested in: each request alone and whole; most of it in one step and the
+    last 32 tokens one by one (also with those steps captured and replayed); portions of
+    changing size down to two tokens. One request is live at a time and the pool holds just
+    the longest (150 tokens rounded up to 192), so every request after the first gets pages that
+    another one gave back."""
+    plain = plain_models["tiny-c"]
+    vocab = plain[0]["vocab_size"]
+    reqs = {r: random_ids(vocab, n, seed=ord(r) + n) for r, n in (("a", 97), ("b", 64), ("c", 33), ("d", 150))}
+    steps, wanted = [], {}
+
+    def add(r, lo, n, want, end):
+        wanted[len(steps)] = [(r, lo + w) for w in want]
+        steps.append({"step": len(steps), "entries": [{"id": r, "tokens": reqs[r][lo:lo + n], "want": want}],
+                      "end": [r] if end else []})
+
+    for r, ids in reqs.items():
+        n = len(ids)
+        if mode == "whole":
+            add(r, 0, n, list(range(n)), True)
+        elif mode == "tail":
+            add(r, 0, n - 32, [n - 33], False)
+            for i in range(n - 32, n):
+                add(r, i, 1, [0], i == n - 1)
+        else:
+            lo = 0
+            for k in cut(n, [17, 5, 2, 32, 3, 2, 21]):
+                add(r, lo, k, list(range(k)), lo + k == n)
+                lo += k
+    out = tmp_path / "out"
+    run_trace(model_dirs["tiny-c"], dtype, out, 192, steps, extra)
+    ref = {r: plain_logits(plain, ids, torch.bfloat16 if dtype == "bfloat16" else None) for r, ids in reqs.items()}
+    checked = _check(out, wanted, ref, vocab, dtype)
+    assert checked == (sum(len(i) for i in reqs.values()) if mode != "tail" else 33 * len(reqs))

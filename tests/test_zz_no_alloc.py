@@ -21,6 +21,8 @@ def _library():
     P, I, L = ctypes.c_void_p, ctypes.c_int, ctypes.c_long
     lib.pyre_argmax_static.argtypes = [P, L, P, I, I, P]
     lib.pyre_argmax_static.restype = I
+    lib.pyre_argmax_static_init.argtypes = []
+    lib.pyre_argmax_static_init.restype = I
     lib.pyre_argmax.argtypes = [P, L, P, P, I, I, P]
     lib.pyre_argmax.restype = I
     lib.pyre_last_error.restype = ctypes.c_char_p
@@ -64,3 +66,30 @@ def test_argmax_static_twice_then_too_many_rows():
         full = torch.randn(MAX_ROWS, 515, device="cuda:0", generator=gen)
         got, want = _both(lib, full)
         assert torch.equal(got, want)
+
+
+def test_argmax_static_in_a_captured_graph():
+    """The caller that cannot allocate: the entry point under HIP graph capture. The scratch's
+    address is looked up beforehand (``pyre_argmax_static_init``; a lookup during capture is not
+    allowed); the graph is replayed several times on new logits, with eager work and
+    synchronisations of the program's own in between, every replay against torch's argmax."""
+    lib = _library()
+    with torch.cuda.device(0):
+        assert lib.pyre_argmax_static_init() == 0, lib.pyre_last_error().decode()
+        assert lib.pyre_argmax_static_init() == 0                  # any number of times
+        gen = torch.Generator(device="cuda:0").manual_seed(12)
+        logits = torch.randn(9, 4099, device="cuda:0", generator=gen)
+        out = torch.full((9,), -1, dtype=torch.int32, device="cuda:0")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rc = lib.pyre_argmax_static(logits.data_ptr(), logits.stride(0), out.data_ptr(), 9, 4099,
+                                        torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.pyre_last_error().decode()
+        for k in range(4):
+            logits.copy_(torch.randn(9, 4099, device="cuda:0", generator=gen))
+            logits[k, 4098 - k] = 11.0
+            want = logits.argmax(dim=1).cpu()                       # eager work and a synchronisation between replays
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out.cpu().long(), want), k
+            assert int(out[k]) == 4098 - k
