@@ -304,6 +304,7 @@ def main() -> int:
         for kv in args.opt:
             k, v = kv.split("=", 1)
             engine.runtime.options[k] = int(v)
+        sync()
         print(f"[bench] {model}: engine ready in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
         checked = None if args.no_gate else gate(engine, cfg.vocab_size, args.dtype, n_layers, model)
         return engine, cfg, full, n_layers, checked

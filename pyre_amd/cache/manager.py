@@ -31,8 +31,9 @@ slots (the engine passes its fill kernel; without one torch does it). It zeroes 
 slot when a request starts. Debugging aid: with ``poison=True`` every page and every state
 slot that goes back to a pool is filled with NaN at once, and the whole pool at the start,
 so that a read of memory which no live request owns shows in the results instead of hiding
-behind stale, finite data; a page is zeroed when a request takes it (slots of its own pages
-that it has not written yet are read, and weighted with 0, by kernels that load whole chunks).
+behind stale, finite data. A page is handed out as it is (NaN in that mode): a mixer whose
+kernels read slots of its own pages that it has not written yet has to see to it that they are
+harmless (the attention part's writing kernel zeroes the values behind a step's last token).
 """
 
 from __future__ import annotations
@@ -248,11 +249,6 @@ class CacheManager:
                 have = len(table)
                 table.extend(g.allocator.allocate_many(add))
                 arr[have:have + add] = table[have:]
-                if self.poison:
-                    # What a request has not yet written of its own pages reads as zero: the
-                    # attention kernels load whole chunks and weight hidden keys with an exact 0.
-                    for t in g.tensors.values():
-                        self._fill(t, table[have:], 0.0)
         req.reserved = max(req.reserved, new_len)
 
     def slot_mapping(self, rid, group: int, start: int, n: int) -> list[int]:

@@ -56,26 +56,6 @@ __device__ inline bf16x8 zero_b128() {
 }
 __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
-// A hidden key's probability is an exact 0, and 0 times a value is 0 only for a finite value.
-// The slots of a request's last page past its last written key hold whatever the page's
-// previous owner left there (NaN and Inf included), so an operand of V^T that reaches past
-// that key has those elements set to zero. keep2: a word of two elements of which the first
-// `n` stay; zero_after: element e of `a` is key first + e, the keys after `last` go.
-__device__ inline unsigned keep2(unsigned w, int n) { return n >= 2 ? w : n == 1 ? (w & 0xffffu) : 0u; }
-__device__ inline bf16x8 zero_after(bf16x8 a, int first, int last) {
-  uint4 u = __builtin_bit_cast(uint4, a);
-  const int n = last - first + 1;
-  u.x = keep2(u.x, n), u.y = keep2(u.y, n - 2), u.z = keep2(u.z, n - 4), u.w = keep2(u.w, n - 6);
-  return __builtin_bit_cast(bf16x8, u);
-}
-// The same for an operand whose elements 0..3 are keys first0 .. and 4..7 keys first1 ..
-__device__ inline bf16x8 zero_after(bf16x8 a, int first0, int first1, int last) {
-  uint4 u = __builtin_bit_cast(uint4, a);
-  const int n0 = last - first0 + 1, n1 = last - first1 + 1;
-  u.x = keep2(u.x, n0), u.y = keep2(u.y, n0 - 2), u.z = keep2(u.z, n1), u.w = keep2(u.w, n1 - 2);
-  return __builtin_bit_cast(bf16x8, u);
-}
-
 // Addressing of one request's keys and values for one key/value head.
 struct KV {
   const bf16* k;     // layer slab [pages, nkv, page_size, HD]
@@ -100,15 +80,14 @@ struct Bounds {
 //                 tile 0, slots 4..7 = the same keys of tile 1
 //   tile_ok[t]    false for a tile whose page is not there: all its keys are hidden
 // `edge` says that some key of the chunk may be hidden from some column;
-// interior chunks skip all masking. `v_last` (the same in all lanes) is the last key whose
-// value has been written: an edge chunk that reaches past it has the rest of V^T zeroed.
+// interior chunks skip all masking.
 // RUNS8 deals the keys to the tiles differently, so that a lane's eight values of P^T
 // belong to eight consecutive keys and V^T comes in 16-byte loads: row 4 g + j of tile t
 // is key key0 + 8 g + 4 t + j; load_k(t, c) gives lane (r, g) the row of key
 // key0 + 8 (r / 4) + 4 t + r % 4, load_v(dt) the keys 8 g .. 8 g + 7 in its slots, and
 // tile_ok[h] stands for the chunk's keys 16 h .. 16 h + 15.
 template <int HD, int CT, bool RUNS8 = false, typename LoadK, typename LoadV>
-__device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2], const Bounds<CT>& bd, int v_last,
+__device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2], const Bounds<CT>& bd,
                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT],
                                    LoadK&& load_k, LoadV&& load_v) {
@@ -174,11 +153,9 @@ __device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2]
   }
 
   // O^T += V^T P^T.
-  const bool cut = edge && key0 + kChunk - 1 > v_last;
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
-    bf16x8 a = load_v(dt);
-    if (cut) a = RUNS8 ? zero_after(a, key0 + 8 * g, v_last) : zero_after(a, key0 + 4 * g, key0 + 16 + 4 * g, v_last);
+    const bf16x8 a = load_v(dt);
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
       o[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p[ct], o[dt][ct], 0, 0, 0);
@@ -188,7 +165,7 @@ __device__ inline void attend_core(int key0, bool edge, const bool (&tile_ok)[2]
 // The chunk's operands straight from the paged cache (no LDS): K rows as stored,
 // V^T as two runs of four keys, 8 bytes each in the transposed cache.
 template <int HD, int CT>
-__device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bounds<CT>& bd, int v_last,
+__device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bounds<CT>& bd,
                                     float scale_log2, const bf16x8 (&q)[CT][HD / 32],
                                     f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
@@ -205,7 +182,7 @@ __device__ inline void attend_chunk(const KV& kv, int key0, bool edge, const Bou
     vp[t] = kv.v + (base * HD + r) * kv.page_size + off + 4 * g;
   }
   attend_core<HD, CT>(
-      key0, edge, ok, bd, v_last, scale_log2, q, o, m, l,
+      key0, edge, ok, bd, scale_log2, q, o, m, l,
       [&](int t, int c) { return load_b128(kp[t] + 32 * c); },
       [&](int dt) {
         uint2 h[2];
@@ -285,12 +262,12 @@ __device__ inline void load_chunk(const KV& kv, TableWindow& tw, int key0, Chunk
 }
 
 template <int HD, int CT>
-__device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge, const Bounds<CT>& bd, int v_last,
+__device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge, const Bounds<CT>& bd,
                                    float scale_log2, const bf16x8 (&q)[CT][HD / 32],
                                    f32x4 (&o)[HD / 16][CT], float (&m)[CT], float (&l)[CT]) {
   const bool ok[2] = {cr.ok[0], cr.ok[1]};
   attend_core<HD, CT, true>(
-      key0, edge, ok, bd, v_last, scale_log2, q, o, m, l, [&](int t, int c) { return cr.k[t][c]; },
+      key0, edge, ok, bd, scale_log2, q, o, m, l, [&](int t, int c) { return cr.k[t][c]; },
       [&](int dt) { return cr.v[dt]; });
 }
 
@@ -388,15 +365,15 @@ __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) 
     }
     for (int c = begin; c < end; c += 2) {
       if (c + 1 < end) load_chunk<HD, STREAM_V>(kv, tw, (c + 1) * kChunk, rb);
-      attend_regs<HD, 1>(ra, c * kChunk, c == first || c == last, bd, pos, scale_log2, qr, o, m, l);
+      attend_regs<HD, 1>(ra, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
       if (c + 1 < end) {
         if (c + 2 < end) load_chunk<HD, STREAM_V>(kv, tw, (c + 2) * kChunk, ra);
-        attend_regs<HD, 1>(rb, (c + 1) * kChunk, c + 1 == first || c + 1 == last, bd, pos, scale_log2, qr, o, m, l);
+        attend_regs<HD, 1>(rb, (c + 1) * kChunk, c + 1 == first || c + 1 == last, bd, scale_log2, qr, o, m, l);
       }
     }
   } else {
     for (int c = begin; c < end; ++c)
-      attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, pos, scale_log2, qr, o, m, l);
+      attend_chunk<HD, 1>(kv, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
   }
 
   // The block's four waves: sum_w o_w 2^(m_w - M), sum_w l_w 2^(m_w - M), M = max_w m_w, waves in the order 0..3.
@@ -560,7 +537,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   for (int c = first; c <= last; ++c) {
     const int key0 = c * kChunk;
     const bool edge = key0 + kChunk - 1 > pos0 || key0 < lo_max;
-    attend_chunk<HD, CT>(kv, key0, edge, bd, hi_all, scale_log2, qr, o, m, l);
+    attend_chunk<HD, CT>(kv, key0, edge, bd, scale_log2, qr, o, m, l);
   }
 
 #pragma unroll
@@ -603,9 +580,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 //        of keys 8 x .. 8 x + 7 of row d lies in slot x ^ ((d >> 3) & 1).
 // A page that is not there (released, or past the request's end) is read from 16 bytes of
 // zeros instead: all its keys are out of every column's bounds, and a hidden key's value is
-// weighted with an exact 0, which only a finite value survives. For the same reason the
-// values of the last chunk that lie past the tile's last key are zeroed on their way from LDS
-// to the matrix cores (zero_after): nobody has written them since the page changed hands.
+// weighted with an exact 0, which only a finite value survives. The slots of a request's last
+// page after its last key are finite because they are zero: whoever writes a token into a page
+// zeroes the values behind it (pyre_common.h: ends_its_page_run, zero_tail).
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 64;
@@ -819,8 +796,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     }
   };
   // O^T += V^T P^T for the chunk in stage sv; MFMA `pair` takes keys 16 pair .. 16 pair + 15, eight per half-wave.
-  auto weighted_values = [&](int sv, int key0) {
-    const bool cut = key0 + kKeys - 1 > hi_all;  // the chunk reaches past the last key that has been written
+  auto weighted_values = [&](int sv) {
     bf16x8 va[2][HD / 32];
     const int v_lane = r * 32 + 16 * (g ^ ((r >> 3) & 1));
     auto load_v = [&](int slot, int pair) {
@@ -833,11 +809,8 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
 #pragma unroll
     for (int pair = 0; pair < 4; ++pair) {
 #pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt) {
-        bf16x8 a = va[pair & 1][dt];
-        if (cut) a = zero_after(a, key0 + 16 * pair + 8 * g, hi_all);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p[pair >> 1][pair & 1], o[dt], 0, 0, 0);
-      }
+      for (int dt = 0; dt < HD / 32; ++dt)
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[pair & 1][dt], p[pair >> 1][pair & 1], o[dt], 0, 0, 0);
       if (pair + 2 < 4) load_v(pair & 1, pair + 2);
     }
   };
@@ -900,7 +873,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_tile32_kernel(
     lds_barrier();
     const int nx = (st + 1) % NS;
     if (active) {
-      weighted_values(st, (first + c) * kKeys);
+      weighted_values(st);
       if (c + 1 < n) scores(nx);
     }
     st = nx;

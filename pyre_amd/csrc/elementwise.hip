@@ -120,6 +120,7 @@ __global__ void rope_kv_write_kernel(const void* __restrict__ qkv, int qkv_dt, i
   const int half = rotary_dim / 2;
   const int slot = write_kv ? slots[n] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  const bool tail = write_kv && ends_its_page_run(slots, n, gridDim.x, slot, page_size);
 
   auto value = [&](int col) {
     float v = 0.f;
@@ -164,7 +165,9 @@ __global__ void rope_kv_write_kernel(const void* __restrict__ qkv, int qkv_dt, i
       const int e = it - n_rot_items;
       const int kvh = e / hd, d = e % hd;
       const float v = value((nq + nkv) * hd + e);
-      v_cache[((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off] = from_float<TC>(v);
+      TC* row = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size;
+      row[off] = from_float<TC>(v);
+      if (tail) zero_tail(row, off + 1, page_size);  // nothing of the page's previous owner stays behind the last key
     }
   }
 }

@@ -211,11 +211,16 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
     const int e = 4 * (it - n_rot);
     const int kvh = e / hd, d = e % hd;
     const float4 v = value4((nq + nkv) * hd + e);
-    TC* dst = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off;
-    dst[0] = from_float<TC>(v.x);
-    dst[page_size] = from_float<TC>(v.y);
-    dst[2 * static_cast<size_t>(page_size)] = from_float<TC>(v.z);
-    dst[3 * static_cast<size_t>(page_size)] = from_float<TC>(v.w);
+    TC* row = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size;
+    row[off] = from_float<TC>(v.x);
+    row[page_size + off] = from_float<TC>(v.y);
+    row[2 * static_cast<size_t>(page_size) + off] = from_float<TC>(v.z);
+    row[3 * static_cast<size_t>(page_size) + off] = from_float<TC>(v.w);
+    // the step's last token of a page leaves nothing of the page's previous owner behind it
+    if (ends_its_page_run(slots, n, gridDim.x, slot, page_size)) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) zero_tail(row + r * static_cast<size_t>(page_size), off + 1, page_size);
+    }
   }
 }
 

@@ -29,6 +29,12 @@ int pyre_add_rmsnorm(float* resid, const void* delta, int delta_dt, int n_partia
                      int gain_dt, void* out, int out_dt, const int* rows, int n, int hidden,
                      float eps, hipStream_t stream);
 
+// Finishes the q/k/v product (partial sums, bias), rotates queries and keys by position, stores
+// the queries and, with write_kv, keys and values at slots[n] = page * page_size + offset
+// (-1: not stored) of caches k [pages, nkv, page_size, hd] and v [pages, nkv, hd, page_size]. The
+// tokens that one call writes into one page are neighbours in the batch and take consecutive
+// slots in rising order (a request's next positions); the last of them zeroes the values of the
+// slots behind it, so that nothing of the page's previous owner stays behind a request's last key.
 int pyre_rope_kv_write(const void* qkv, int qkv_dt, int n_partials, long partial_stride,
                        const void* bias, int bias_dt, void* q_out, int q_dt, void* k_cache,
                        void* v_cache, int cache_dt, const float* cos_t, const float* sin_t,

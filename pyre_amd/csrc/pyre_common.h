@@ -57,6 +57,42 @@ __device__ inline void rotate_pair(float x1, float x2, float c, float s, float& 
   b = fmaf(x2, c, x1 * s);
 }
 
+// The attention kernels on the matrix cores load whole chunks of values and weight the keys
+// that a query does not see with an exact 0, which only a finite value survives. The slots of a
+// request's last page after its last key hold what the page's previous owner left there (NaN
+// and Inf included), so whoever writes a step's last token into a page also zeroes the values
+// of the slots after it: what follows a request's last key in its page is always zero.
+//   ends_its_page_run: token n of a step of `count` tokens, written to `slot`, is the last one
+//                      that the step writes into its page (the next token, if there is one, does
+//                      not take the next slot), and the page has slots after it;
+//   zero_tail:         row[from .. to) = 0 in as few stores as the alignment allows.
+__device__ inline bool ends_its_page_run(const int* slots, int n, int count, int slot, int page_size) {
+  return slot >= 0 && slot % page_size + 1 < page_size && (n + 1 >= count || slots[n + 1] != slot + 1);
+}
+template <typename T>
+__device__ inline void zero_tail(T* row, int from, int to) {
+  static_assert(sizeof(T) == 2 || sizeof(T) == 4, "cache elements of two or four bytes");
+  char* p = reinterpret_cast<char*>(row + from);
+  char* const end = reinterpret_cast<char*>(row + to);
+  while (p < end) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    const size_t left = static_cast<size_t>(end - p);
+    if (a % 16 == 0 && left >= 16) {
+      *reinterpret_cast<uint4*>(p) = uint4{0u, 0u, 0u, 0u};
+      p += 16;
+    } else if (a % 8 == 0 && left >= 8) {
+      *reinterpret_cast<uint2*>(p) = uint2{0u, 0u};
+      p += 8;
+    } else if (a % 4 == 0 && left >= 4) {
+      *reinterpret_cast<uint32_t*>(p) = 0u;
+      p += 4;
+    } else {
+      *reinterpret_cast<uint16_t*>(p) = 0;
+      p += 2;
+    }
+  }
+}
+
 template <typename T> __host__ __device__ inline T from_float(float v);
 template <> __host__ __device__ inline float from_float<float>(float v) { return v; }
 template <> __host__ __device__ inline bf16 from_float<bf16>(float v) {

@@ -44,27 +44,37 @@ extern "C" const char* pyre_sources_digest() { return PYRE_SOURCES_DIGEST; }
 // ---------------------------------------------------------------------------
 // A plain streaming read of `bytes` (a multiple of 16) for measuring what the
 // memory system delivers: every lane loads 16 bytes per iteration, the loads of
-// one wave are contiguous, and nothing but a checksum is written.
+// one wave are contiguous, and nothing but a checksum is written. The loads are
+// non-temporal, as those of the kernels that stream weights: data that is read once
+// goes past the caches (ordinary loads reach about four fifths of this).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict__ p, size_t n,
+typedef unsigned probe_u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void read_probe_kernel(const probe_u32x4* __restrict__ p, size_t n,
                                                           unsigned* __restrict__ sink) {
+  // A block takes spans of 64 KB (4,096 pieces of 16 bytes), span b, b + blocks, ...: 16 loads
+  // per thread and span, four in flight.
+  constexpr size_t kSpan = 4096;
   unsigned acc = 0;
-  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
-  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  for (; i + 3 * stride < n; i += 4 * stride) {
-    const uint4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
-    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
-  }
-  for (; i < n; i += stride) {
-    const uint4 a = p[i];
-    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  for (size_t s0 = static_cast<size_t>(blockIdx.x) * kSpan; s0 < n; s0 += static_cast<size_t>(gridDim.x) * kSpan) {
+    const size_t end = s0 + kSpan < n ? s0 + kSpan : n;
+    size_t i = s0 + threadIdx.x;
+    for (; i + 768 < end; i += 1024) {
+      const probe_u32x4 a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + 256),
+                        c = __builtin_nontemporal_load(p + i + 512), d = __builtin_nontemporal_load(p + i + 768);
+      acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < end; i += 256) {
+      const probe_u32x4 a = __builtin_nontemporal_load(p + i);
+      acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
   }
   if (acc == 0x9e3779b9u) *sink = acc;  // practically never: keeps the loads alive
 }
 
 extern "C" int pyre_read_probe(const void* p, size_t bytes, int blocks, unsigned* sink, hipStream_t stream) {
   PYRE_REQUIRE(bytes % 16 == 0 && blocks > 0, "read_probe: bytes must be a multiple of 16");
-  hipLaunchKernelGGL(read_probe_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<const uint4*>(p),
+  hipLaunchKernelGGL(read_probe_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<const probe_u32x4*>(p),
                      bytes / 16, sink);
   return pyre::check_launch("read_probe");
 }

@@ -294,8 +294,9 @@ def test_unreserve_gives_back_what_a_step_that_did_not_run_had_taken():
 
 
 def test_poison_mode_marks_what_nobody_holds():
-    """NaN wherever no live request holds the memory, zero in a page just taken, under a
-    random sequence of requests with a window (on the CPU: torch does the filling)."""
+    """NaN wherever no live request holds the memory and in the slots of a held page that its
+    request has not written yet (a page is handed out as it is), under a random sequence of
+    requests with a window (on the CPU: torch does the filling)."""
     import torch
 
     rng = random.Random(5)
@@ -330,10 +331,15 @@ def test_poison_mode_marks_what_nobody_holds():
             live[rid] += n
         m.check_invariants()
         for gi, g in enumerate(m.page_groups):
-            held = {p for r in live for p in m.block_table(r, gi) if p != RELEASED}
+            written = {}                                   # page -> slots of it that its request has written
+            for r, length in live.items():
+                for i, p in enumerate(m.block_table(r, gi)):
+                    if p != RELEASED:
+                        written[p] = max(0, min(16, length - 16 * i))
             for p in range(g.num_pages):
-                nan = torch.isnan(g.tensors["k"][:, p])
-                assert (not nan.any()) if p in held else nan.all(), (step, gi, p)
+                nan = torch.isnan(g.tensors["k"][:, p])    # [layers, kv heads, slots, head]
+                n = written.get(p, 0)
+                assert not nan[:, :, :n].any() and nan[:, :, n:].all(), (step, gi, p)
         free_slots = set(range(3)) - {m.slot(r) for r in live}
         for sl in free_slots:
             assert torch.isnan(m.state_groups[0].tensor[:, sl]).all()

@@ -227,7 +227,10 @@ def test_rope_kv_write(dtype, nq, nkv, hd, rot, page):
     bias = rnd(width, seed=8)
     pos = torch.tensor([0, 1, 2, 40, 41, 7, 100, 3, 64])
     cos, sin = rotary_tables(rot, theta, 128)
-    slots = torch.tensor(random.Random(1).sample(range(npages * page), n))
+    rng = random.Random(1)
+    # every token in a page of its own (the tokens that a call writes into one page are a run of
+    # consecutive slots: the run's last token zeroes the values behind it)
+    slots = torch.tensor([p * page + rng.randrange(page) for p in rng.sample(range(npages), n)])
     slots[4] = -1                                           # this token is not stored
     q = torch.empty(n, nq * hd, device=DEV, dtype=DT[dtype])
     kc = torch.zeros(npages, nkv, page, hd, device=DEV, dtype=DT[dtype])
@@ -716,27 +719,48 @@ def test_attention_at_a_windows_edge(kernel):
 @pytest.mark.parametrize("ctx_len", [700, 689, 655])
 def test_attention_ignores_what_a_page_held_before(kernel, ctx_len):
     """A request's last page is only partly its own: the slots past its last key still hold what
-    the page's previous owner wrote, which may be NaN or Inf (a request that diverged). A kernel
-    that loads whole chunks and weights the hidden keys with 0 must not let such a value through
-    (0 * NaN is NaN). Contexts that end 4, 15 and 1 keys before the end of a 16-key page; pages that the request
-    does not hold are NaN as well."""
+    the page's previous owner wrote, which may be NaN or Inf (a request that diverged). The
+    kernels on the matrix cores load whole chunks and weight the hidden keys with 0, and 0 * NaN
+    is NaN: so the kernel that writes a step's keys and values zeroes the values behind the last
+    token it writes into a page. Every page starts as NaN (keys) and Inf (values) here; the
+    requests' keys and values go in through that kernel in two steps (all but the last tokens,
+    then the last tokens of both requests side by side); then attention. Contexts that end 4,
+    15 and 1 keys before the end of a 16-key page."""
     ops = _ops()
+    from pyre_amd.hip.ops import Partials
+
     big = kernel.endswith("256")
     nq, nkv, hd, page = (4, 2, 256, 16) if big else (8, 2, 64, 16)
     dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
     ql = 34 if kernel.startswith("prefill") else 1
     ctx_lens, q_lens = [ctx_len, 40], [ql, min(ql, 3)]
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=17)
-    held = set(table[table >= 0].tolist())
-    for p in range(kc.shape[0]):
-        if p not in held:
-            kc[p], vc[p] = float("nan"), float("inf")
-    for s, c in enumerate(ctx_lens):                       # the tail of each request's last page
-        last = int(table[s, (c - 1) // page])
-        kc[last, :, c % page or page:, :] = float("nan")
-        vc[last, :, :, c % page or page:] = float("nan")
+    kc.fill_(float("nan"))
+    vc.fill_(float("inf"))
+    tab = table.cpu()
+
+    def write(spans):
+        """The tokens [a, b) of each request (request, a, b), in one call of the writing kernel."""
+        rows, positions, slots = [], [], []
+        for s, a, b in spans:
+            K, V = dense[s]
+            rows.append(torch.cat([torch.zeros(b - a, nq * hd), K[a:b].reshape(b - a, -1).float(),
+                                   V[a:b].reshape(b - a, -1).float()], dim=1))
+            positions += list(range(a, b))
+            slots += [int(tab[s, t // page]) * page + t % page for t in range(a, b)]
+        qkv = Partials(torch.cat(rows).to(DEV).unsqueeze(0).contiguous())
+        n = len(positions)
+        ops.rope_kv_write(qkv, torch.empty(n, nq * hd, device=DEV, dtype=dt), kc, vc, None, None, 0, i32(positions),
+                          i32(slots), n, nq, nkv, hd, page)
+
+    write([(0, 0, ctx_lens[0] - q_lens[0])])
+    write([(1, 0, ctx_lens[1] - q_lens[1])])
+    write([(0, ctx_lens[0] - q_lens[0], ctx_lens[0]), (1, ctx_lens[1] - q_lens[1], ctx_lens[1])])
+    for s, c in enumerate(ctx_lens):                        # what the writer left: its values, then zeros; keys untouched
+        last = int(tab[s, (c - 1) // page])
         if c % page:
-            vc[last, 0, :, c % page] = float("inf")           # and an infinity right behind the last key
+            assert (vc[last, :, :, c % page:] == 0).all() and torch.isnan(kc[last, :, c % page:, :]).all()
+        assert torch.equal(vc[last, :, :, (c - 1) % page].cpu(), dense[s][1][c - 1].to(dt))
     scale = hd ** -0.5
     want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale)
     out = torch.zeros_like(q)
@@ -753,6 +777,38 @@ def test_attention_ignores_what_a_page_held_before(kernel, ctx_len):
     assert torch.isfinite(out.float()).all(), kernel
     tol = 2e-5 if dt == torch.float32 else 2e-2
     assert torch.allclose(out.double().cpu(), want, atol=tol, rtol=tol), kernel
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page,hd", [(16, 128), (8, 12), (5, 40), (6, 10), (32, 64)])
+def test_the_writer_zeroes_the_values_behind_a_steps_last_token(dtype, page, hd):
+    """Page sizes and head sizes of the vectorised and of the general writing kernel: three
+    requests in one step (one run that ends mid-page, one that ends exactly at a page's end, one
+    single token that starts a page); of every page only the slots after the run's last token
+    are zeroed, nothing that an earlier step wrote and nothing of other pages."""
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+
+    nq, nkv, dt = 2, 2, DT[dtype]
+    pages = 6
+    kc = torch.full((pages, nkv, page, hd), 7.0, device=DEV, dtype=dt)
+    vc = torch.full((pages, nkv, hd, page), 7.0, device=DEV, dtype=dt)
+    # request a: slots 2 .. page + 1 of pages (0, 1): its run ends at slot 1 of page 1; request b: the
+    # whole of page 2; request c: slot 0 of page 3; page 4 belongs to nobody
+    runs = [[2 + i for i in range(page)], [2 * page + i for i in range(page)], [3 * page]]
+    slots = [s for r in runs for s in r]
+    n = len(slots)
+    vals = rnd(n, (nq + 2 * nkv) * hd, seed=3)
+    ops.rope_kv_write(Partials(vals.to(DEV).unsqueeze(0).contiguous()), torch.empty(n, nq * hd, device=DEV, dtype=dt), kc, vc,
+                      None, None, 0, i32(list(range(n))), i32(slots), n, nq, nkv, hd, page)
+    v = vals.cpu()[:, (nq + nkv) * hd:].view(n, nkv, hd).to(dt)
+    got = vc.cpu()
+    for i, s in enumerate(slots):
+        assert torch.equal(got[s // page, :, :, s % page], v[i]), (i, s)
+    assert (got[0, :, :, :2] == 7.0).all()                              # before the run: as it was
+    assert (got[1, :, :, 2:] == 0).all()                                # behind the run's end in its last page
+    assert (got[3, :, :, 1:] == 0).all() and (got[4] == 7.0).all() and (got[5] == 7.0).all()
+    assert (kc.cpu()[1, :, 2:, :] == 7.0).all()                         # keys need no zeroing: their scores are masked
 
 
 # ----------------------------------------------------------------------------- sampling
