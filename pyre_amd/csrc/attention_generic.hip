@@ -146,6 +146,139 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
   }
 }
 
+// The same for the query heads that share a key/value head, float32 throughout: one block per
+// (token, key/value head and group of up to kGroupHeads of its query heads, span of keys), so
+// that a span's keys and values are read once for the group and not once per head (a decode
+// step's attention is all memory traffic). Every number is computed exactly as the kernel
+// above computes it, by the same chain of operations in the same order: a score by one thread
+// (the key's, for all heads of the group) over the head's elements in ascending order; a span's sum of probabilities by the same
+// reduction over the same layout of threads (key j in lane j % 64 of wave j / 64, the waves'
+// sums added in their order); an output element over the keys 4 g, 4 g + 1, ... of its thread's
+// set, the sets' sums added in their order. The two kernels give the same bits; this one needs
+// head and page sizes that are multiples of four (VEC above).
+constexpr int kGroupHeads = 8;
+
+__global__ __launch_bounds__(kThreads) void attn_grouped_f32_kernel(
+    const float* __restrict__ q, const float* __restrict__ k_cache, const float* __restrict__ v_cache,
+    float* __restrict__ out, const int* __restrict__ tokens, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride, int nq, int nkv,
+    int hd, int page_size, float scale, int window, float* __restrict__ part) {
+  __shared__ __attribute__((aligned(16))) float sc[kGroupHeads][kSpan];
+  __shared__ float accs[kGroupHeads][kThreads];
+  __shared__ float ml[kGroupHeads][2];  // maximum and sum of each head's span
+  __shared__ float scratch[16];
+
+  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, tid = threadIdx.x;
+  const int n_rep = nq / nkv, per_kv = (n_rep + kGroupHeads - 1) / kGroupHeads;
+  const int kvh = blockIdx.y / per_kv, head0 = kvh * n_rep + (blockIdx.y % per_kv) * kGroupHeads;
+  const int nheads = min(kGroupHeads, kvh * n_rep + n_rep - head0);
+  const int pos = positions[n];
+  const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int base = lo + static_cast<int>(blockIdx.z) * kSpan;  // this block's span
+  if (base > pos) return;
+  const int cnt = min(kSpan, pos - base + 1);
+
+  // Scores: thread j < 128 takes key base + j for every head of the group (each row of keys is read by
+  // one thread only: a wave's load touches 64 lines, and the address unit's time is what this phase
+  // costs). The queries are the same for every lane: they come through scalar loads.
+  const int j = tid;
+  const float* qg = q + (static_cast<size_t>(n) * nq + head0) * hd;
+  float s[kGroupHeads];
+#pragma unroll
+  for (int h = 0; h < kGroupHeads; ++h) s[h] = -INFINITY;
+  if (j < cnt) {
+    const int key = base + j;
+    const int page = table[key / page_size], off = key % page_size;
+    if (page >= 0) {  // a page that is not there (padding rows of a captured step) hides its keys
+      const float* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * hd;
+#pragma unroll
+      for (int h = 0; h < kGroupHeads; ++h) s[h] = 0.f;
+#pragma unroll 8
+      for (int e = 0; e < hd; e += 4) {
+        float kv[4];
+        load4(kp + e, kv);
+#pragma unroll
+        for (int h = 0; h < kGroupHeads; ++h)
+          if (h < nheads) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s[h] = fmaf(qg[h * hd + e + u], kv[u], s[h]);
+          }
+      }
+#pragma unroll
+      for (int h = 0; h < kGroupHeads; ++h) s[h] *= scale;
+    }
+  }
+  // Softmax of the span, head by head: the maximum, the probabilities, their sum (key j in lane
+  // j % 64 of wave j / 64, the other two waves add zeros).
+#pragma unroll
+  for (int h = 0; h < kGroupHeads; ++h) {
+    if (h >= nheads) break;
+    const bool mine = j < cnt;
+    const float m = block_max(mine ? s[h] : -INFINITY, scratch);
+    const float m_use = m == -INFINITY ? 0.f : m;
+    const float p = mine ? expf(s[h] - m_use) : 0.f;
+    if (mine) sc[h][j] = p;
+    const float l = block_sum(p, scratch);  // its barriers publish sc[h][]
+    if (tid == 0) ml[h][0] = m, ml[h][1] = l;
+  }
+
+  // Output: set g of hd threads takes the groups of four keys g, g + groups, ... of the span for element d.
+  const int groups = kThreads / hd;  // >= 1 because hd <= 256
+  const int g = tid / hd, d = tid % hd;
+  float acc[kGroupHeads];
+#pragma unroll
+  for (int h = 0; h < kGroupHeads; ++h) acc[h] = 0.f;
+  if (g < groups) {
+#pragma unroll 2
+    for (int quad = base / 4 + g; quad <= (base + cnt - 1) / 4; quad += groups) {
+      const int key = 4 * quad;
+      const int page = table[key / page_size], off = key % page_size;
+      if (page < 0) continue;
+      float vv[4];
+      load4(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off, vv);
+      if (key >= base && key + 3 < base + cnt && ((key - base) & 3) == 0) {  // the whole group, its probabilities in one read
+#pragma unroll
+        for (int h = 0; h < kGroupHeads; ++h)
+          if (h < nheads) {
+            const float4 p = *reinterpret_cast<const float4*>(&sc[h][key - base]);
+            acc[h] = fmaf(p.x, vv[0], acc[h]);
+            acc[h] = fmaf(p.y, vv[1], acc[h]);
+            acc[h] = fmaf(p.z, vv[2], acc[h]);
+            acc[h] = fmaf(p.w, vv[3], acc[h]);
+          }
+        continue;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (key + u >= base && key + u < base + cnt) {
+#pragma unroll
+          for (int h = 0; h < kGroupHeads; ++h)
+            if (h < nheads) acc[h] = fmaf(sc[h][key + u - base], vv[u], acc[h]);
+        }
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < kGroupHeads; ++h) accs[h][tid] = g < groups ? acc[h] : 0.f;
+  __syncthreads();
+  for (int i = tid; i < nheads * hd; i += kThreads) {
+    const int h = i / hd, dd = i % hd;
+    float total = 0.f;
+    for (int gg = 0; gg < groups; ++gg) total += accs[h][gg * hd + dd];
+    if (part) {  // [token of the list][head][span][hd + 2]: unnormalised output, max, sum
+      float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + head0 + h) * gridDim.z + blockIdx.z) * (hd + 2);
+      dst[dd] = total;
+      if (dd == 0) {
+        dst[hd] = ml[h][0];
+        dst[hd + 1] = ml[h][1];
+      }
+    } else {
+      const float l = ml[h][1];
+      out[(static_cast<size_t>(n) * nq + head0 + h) * hd + dd] = l > 0.f ? total / l : 0.f;
+    }
+  }
+}
+
 // out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the spans that the token has, in their order.
 template <typename TQ>
 __global__ __launch_bounds__(kThreads) void attn_generic_join_kernel(
@@ -184,7 +317,7 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
                                  const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                                  const int* seq_of_token, const int* block_table, int table_stride,
                                  int n, int nq, int nkv, int hd, int page_size, float scale,
-                                 int window, int max_keys, float* part, hipStream_t stream) {
+                                 int window, int max_keys, float* part, int grouped, hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(q_dt) && known_dtype(cache_dt), "attn_generic: unknown dtype");
   PYRE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attn_generic: %d query heads do not divide over %d kv heads", nq, nkv);
   PYRE_REQUIRE(hd > 0 && hd <= kMaxHead, "attn_generic: head_dim %d is outside 1..%d", hd, kMaxHead);
@@ -198,6 +331,19 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
   float* scratch = spans == 1 ? nullptr : part;
   const bool vec = hd % 4 == 0 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+  if (grouped && vec && q_dt == kF32 && cache_dt == kF32) {
+    // the query heads of a key/value head together: the span's keys and values are read once for all of them
+    const int per_kv = (nq / nkv + kGroupHeads - 1) / kGroupHeads;
+    PYRE_REQUIRE(nkv * per_kv <= 65535, "attn_generic: too many heads");
+    hipLaunchKernelGGL(attn_grouped_f32_kernel, dim3(n, nkv * per_kv, spans), dim3(kThreads), 0, stream,
+                       static_cast<const float*>(q), static_cast<const float*>(k_cache),
+                       static_cast<const float*>(v_cache), static_cast<float*>(out), tokens, positions, seq_of_token,
+                       block_table, table_stride, nq, nkv, hd, page_size, scale, window, scratch);
+    if (spans > 1)
+      hipLaunchKernelGGL((attn_generic_join_kernel<float>), dim3(n, nq), dim3(kThreads), 0, stream, scratch,
+                         static_cast<float*>(out), tokens, positions, nq, hd, window, spans);
+    return check_launch("attn_generic");
+  }
 #define PYRE_LAUNCH_GENERIC(VEC)                                                                          \
   PYRE_DISPATCH(q_dt, TQ, PYRE_DISPATCH(cache_dt, TC,                                                     \
       hipLaunchKernelGGL((attn_generic_kernel<TQ, TC, VEC>), dim3(n, nq, spans), dim3(kThreads), 0, stream, \

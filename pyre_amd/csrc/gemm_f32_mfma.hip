@@ -144,20 +144,21 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_f32_mfma_kernel(
   }
 }
 
-// The same product for a decode step's few rows (M <= 8), as a stream over the weights. A block
+// The same product for a decode step's rows (M <= 64), as a stream over the weights. A block
 // is one wave with 32 output columns, so there is no barrier. It has a ring of R slots in LDS, a
-// slot being 32 k (two stages) of its 32 rows of W (4 KB) and of the rows of A (1 KB), filled by
-// loads that go from memory straight into LDS: while slot j is multiplied, slot j + 1 is read
-// from LDS into registers and the R - 2 after it are on their way. A load instruction takes
-// whole 128-byte lines (8 rows x 32 k); the 16-byte pieces of a row are exchanged among
-// themselves by the row's number so that the matrix instruction's operand reads (a lane's row,
-// eight k of a stage) spread over the banks. Stages, steps and parts of k are those of the
-// kernel above: the sums are the same bit for bit. With one row in 32 columns of the matrix
-// instruction the chain of dependent instructions of a wave, not memory, sets the pace (a slot
-// of 4 KB in about 0.6 us); a small ring lets eight blocks share a compute unit.
-constexpr int kStreamRows = 8;
+// slot being 32 k (two stages) of its 32 rows of W (4 KB) and of XR rows of A (XR = 8, 32 or 64,
+// whichever holds M: 1, 4 or 8 KB), filled by loads that go from memory straight into LDS: while
+// slot j is multiplied, slot j + 1 is read from LDS into registers and the R - 2 after it are on
+// their way. A load instruction takes whole 128-byte lines (8 rows x 32 k); the 16-byte pieces
+// of a row are exchanged among themselves by the row's number so that the matrix instruction's
+// operand reads (a lane's row, eight k of a stage) spread over the banks. Stages, steps and
+// parts of k are those of the kernel above, and an element of the result depends on its own
+// row of A and row of W alone: the sums are the same bit for bit, however many of the
+// instruction's 32 columns carry a row. With few rows the chain of dependent instructions of a
+// wave, not memory, sets the pace (a slot of 4 KB in about 0.6 us), and with 64 rows the matrix
+// cores' float32 rate does; a small ring lets several blocks share a compute unit.
+constexpr int kStreamMaxRows = 64;
 constexpr int kSlotK = 32;
-constexpr int kSlotBytes = 5 * 1024;
 
 __device__ inline void load_to_lds(const void* src, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
@@ -168,11 +169,16 @@ __device__ inline void wait_loads() {
 }
 __device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 0u, 0u};
 
-template <int R>
+template <int R, int XR>
 __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
     const float* __restrict__ A, size_t lda, const float* __restrict__ W, size_t ldw,
     const void* __restrict__ bias, int bias_dt, float* __restrict__ out, size_t ldo, size_t part_stride, int M,
     int N, int K, int kper) {
+  constexpr int XL = XR / 8;                    // load instructions for a slot's rows of A
+  constexpr int MT = XR > 32 ? 2 : 1;           // tiles of 32 rows of A
+  constexpr int kSlotBytes = 4096 + XR * 128;
+  constexpr int L = 4 + XL;                     // load instructions per slot
+  static_assert(L * (R - 2) <= 63, "the wait counter holds 63 loads");
   __shared__ __attribute__((aligned(1024))) unsigned char ring[R * kSlotBytes];
   const int lane = threadIdx.x, half = lane >> 5, c = lane & 31;
   const int n0 = blockIdx.x * 32;
@@ -182,9 +188,9 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
   if (blockIdx.z) bias = nullptr;  // the bias belongs to one part only
   const int slots = (K - kbeg + kSlotK - 1) / kSlotK;
 
-  // This lane's share of a slot's five loads: of load i, the piece that lands at row 8 i + lane / 8,
+  // This lane's share of a slot's loads: of load i, the piece that lands at row 8 i + lane / 8,
   // place lane % 8, which is piece (place ^ swizzle of the row) of the row's 32 k. Columns past
-  // the end read the last one's weights and are not stored.
+  // the end read the last one's weights and are not stored; rows of A past M read zeros.
   const int lr = lane >> 3, lp = lane & 7;
   const float* wsrc[4];
   int wk[4];
@@ -194,7 +200,17 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
     wk[i] = 4 * (lp ^ ((r >> 1) & 7));
     wsrc[i] = W + static_cast<size_t>(min(n0 + r, N - 1)) * ldw + kbeg + wk[i];
   }
-  const float* xsrc = A + static_cast<size_t>(lr < M ? lr : 0) * lda + kbeg + 4 * lp;
+  const float* xsrc[XL];
+  int xk[XL];
+  bool xrow[XL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int r = 8 * i + lr;
+    // eight rows or fewer: every lane of the instruction reads row c % 8 (no exchange of pieces needed)
+    xk[i] = XR == 8 ? 4 * lp : 4 * (lp ^ ((r >> 1) & 7));
+    xrow[i] = r < M;
+    xsrc[i] = A + static_cast<size_t>(xrow[i] ? r : 0) * lda + kbeg + xk[i];
+  }
   const unsigned mine = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(ring)));
   const float* zero = reinterpret_cast<const float*>(kZeroPiece);
 
@@ -205,26 +221,32 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
     const int k0 = kSlotK * j, left = j < slots ? K - kbeg - k0 : 0;  // k of this part from the slot's start on
 #pragma unroll
     for (int i = 0; i < 4; ++i) load_to_lds(wk[i] < left ? wsrc[i] + k0 : zero, dst + 1024 * i);
-    load_to_lds(lr < M && 4 * lp < left ? xsrc + k0 : zero, dst + 4096);
+#pragma unroll
+    for (int i = 0; i < XL; ++i) load_to_lds(xrow[i] && xk[i] < left ? xsrc[i] + k0 : zero, dst + 4096 + 1024 * i);
   };
 
-  f32x16 acc;
+  f32x16 acc[MT];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  for (int u = 0; u < MT; ++u)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[u][i] = 0.f;
   const unsigned char* wpiece = ring + c * 128;
-  const unsigned char* xpiece = ring + 4096 + (c & 7) * 128;
-  const int swz = (c >> 1) & 7;
-  const bool has_x = c < M;
+  const unsigned char* xpiece = ring + 4096 + (XR == 8 ? c & 7 : c) * 128;
+  const int swz = (c >> 1) & 7, xswz = XR == 8 ? 0 : swz;  // rows c and 32 + c exchange their pieces alike
+  const bool has_x = XR != 8 || c < M;
   int at = 0;  // ring position of the next slot to read
-  auto read = [&](f32x4 (&a)[2][2], f32x4 (&b)[2][2]) {
+  auto read = [&](f32x4 (&a)[2][2], f32x4 (&b)[MT][2][2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const int piece = 4 * t + 2 * half + h;
         a[t][h] = *reinterpret_cast<const f32x4*>(wpiece + at * kSlotBytes + 16 * (piece ^ swz));
-        b[t][h] = *reinterpret_cast<const f32x4*>(xpiece + at * kSlotBytes + 16 * piece);
-        if (!has_x) b[t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+          b[u][t][h] = *reinterpret_cast<const f32x4*>(xpiece + at * kSlotBytes + 4096 * u + 16 * (piece ^ xswz));
+          if (!has_x) b[u][t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
       }
     at = at + 1 == R ? 0 : at + 1;
   };
@@ -233,44 +255,54 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
   // in registers, one being read and R - 2 on their way.
 #pragma unroll
   for (int j = 0; j < R - 1; ++j) issue(j);
-  f32x4 a[2][2], b[2][2], an[2][2], bn[2][2];
-  wait_loads<5 * (R - 2)>();  // loads finish in the order of issue: slot 0 is there
+  f32x4 a[2][2], b[MT][2][2], an[2][2], bn[MT][2][2];
+  wait_loads<L * (R - 2)>();  // loads finish in the order of issue: slot 0 is there
   read(a, b);
   for (int j = 0; j < slots; ++j) {
     issue(j + R - 1);            // into the position of slot j - 1, read a turn ago
-    wait_loads<5 * (R - 2)>();   // slot j + 1 is there
+    wait_loads<L * (R - 2)>();   // slot j + 1 is there
     read(an, bn);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       if (kSlotK * j + BK * t >= K - kbeg) break;  // a part that ends with half a slot
 #pragma unroll
       for (int s = 0; s < 8; ++s)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s >> 2][s & 3], b[t][s >> 2][s & 3], acc, 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < MT; ++u)
+          acc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s >> 2][s & 3], b[u][t][s >> 2][s & 3], acc[u], 0, 0, 0);
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) a[t][h] = an[t][h], b[t][h] = bn[t][h];
+      for (int h = 0; h < 2; ++h) {
+        a[t][h] = an[t][h];
+#pragma unroll
+        for (int u = 0; u < MT; ++u) b[u][t][h] = bn[u][t][h];
+      }
   }
   wait_loads<0>();  // the loads past the end
 
-  // acc[4 i + j]: output column n = tile row 8 i + 4 half + j, output row m = tile column c.
-  if (c >= M) return;
+  // acc[u][4 i + j]: output column n = tile row 8 i + 4 half + j, output row m = 32 u + tile column c.
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = n0 + 8 * i + 4 * half;
-    if (n >= N) continue;
-    float v[4];
+  for (int u = 0; u < MT; ++u) {
+    const int m = 32 * u + c;
+    if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      v[j] = acc[4 * i + j];
-      if (bias && n + j < N) v[j] += load_as_float(bias, bias_dt, n + j);
-    }
-    float* dst = out + static_cast<size_t>(c) * ldo + n;
-    if (n + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
-      *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-    } else {
-      for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = v[j];
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 8 * i + 4 * half;
+      if (n >= N) continue;
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[j] = acc[u][4 * i + j];
+        if (bias && n + j < N) v[j] += load_as_float(bias, bias_dt, n + j);
+      }
+      float* dst = out + static_cast<size_t>(m) * ldo + n;
+      if (n + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+      } else {
+        for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = v[j];
+      }
     }
   }
 }
@@ -291,11 +323,16 @@ extern "C" int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw,
   // 16-byte loads along k need rows that start on 16 bytes
   const int vec_ok = lda % 4 == 0 && ldw % 4 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(W) % 16 == 0;
-  if (M <= kStreamRows && vec_ok && K % 4 == 0) {  // a decode step's few rows: the weights as a stream
+  if (M <= kStreamMaxRows && vec_ok && K % 4 == 0) {  // a decode step's rows: the weights as a stream
     const dim3 grid((N + 31) / 32, 1, ksplit);
-    hipLaunchKernelGGL((gemm_f32_stream_kernel<4>), grid, dim3(64), 0, stream, A, static_cast<size_t>(lda), W,
-                       static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),
-                       static_cast<size_t>(part_stride), M, N, K, kper);
+#define PYRE_STREAM(R, XR)                                                                                         \
+  hipLaunchKernelGGL((gemm_f32_stream_kernel<R, XR>), grid, dim3(64), 0, stream, A, static_cast<size_t>(lda), W,    \
+                     static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),                       \
+                     static_cast<size_t>(part_stride), M, N, K, kper)
+    if (M <= 8) PYRE_STREAM(4, 8);
+    else if (M <= 32) PYRE_STREAM(4, 32);
+    else PYRE_STREAM(3, 64);
+#undef PYRE_STREAM
   } else if (M <= 32) {  // four waves side by side along n
     const dim3 grid((N + 127) / 128, (M + 31) / 32, ksplit);
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<4, 1, 1, 1>), grid, dim3(256), 0, stream, A, static_cast<size_t>(lda), W,

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 
 class KernelError(RuntimeError):
@@ -30,7 +30,7 @@ _SIGNATURES = {
     "pyre_fill_rows": [P, I, L, I, I, L, P, I, ctypes.c_uint, P],
     "pyre_gemm_generic": [P, I, L, P, P, I, L, P, I, P, I, L, I, I, I, P],
     "pyre_gemm_f32": [P, L, P, L, P, I, P, L, L, I, I, I, I, P],
-    "pyre_attn_generic": [P, P, I, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P],
+    "pyre_attn_generic": [P, P, I, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, I, P],
     "pyre_attn_generic_spans": [I],
     "pyre_attn_prefill_f32": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_mfma_supports": [I, I, I, I],

@@ -126,7 +126,8 @@ def test_gemm_generic(adt, wdt, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 37, 50), (5, 130, 257), (32, 128, 16), (33, 129, 17), (77, 200, 64), (130, 65, 1000),
-                                   (300, 3584, 3584), (8, 1000, 18944)])
+                                   (300, 3584, 3584), (8, 1000, 18944), (20, 777, 3584), (64, 4608, 3584), (48, 96, 40),
+                                   (33, 1000, 1100)])
 def test_gemm_f32_on_the_matrix_cores(m, n, k):
     """float32 in, float32 products and sums (the result is as close to a float64 product as
     plain float32 FMAs are), and a row's result bit for bit the same whatever rows share
@@ -336,6 +337,41 @@ def test_attn_generic(dtype, nq, nkv, hd, page, window):
     if window == 0:
         # one visible key: the output is exactly that key's value (request 0)
         assert torch.allclose(out[0].double().cpu(), dense[0][1][0].double().repeat_interleave(nq // nkv, 0), atol=tol)
+    if dtype == "float32":
+        # one block per head and one block for the heads of a key/value head: the same bits
+        alone = torch.empty_like(q)
+        ops.attn_generic(q, alone, kc, vc, pos, seq_of, table, q.shape[0], nq, nkv, hd, page, scale, window, grouped=False)
+        assert torch.equal(out, alone)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,page", [(28, 4, 128, 16), (40, 8, 128, 16), (12, 2, 128, 32), (9, 1, 64, 8), (20, 2, 256, 16),
+                                            (3, 3, 32, 4), (6, 2, 12, 8), (8, 2, 64, 16)])
+@pytest.mark.parametrize("window", [0, 300])
+def test_attn_of_single_tokens_by_groups_of_heads_in_float32(nq, nkv, hd, page, window):
+    """The 32-bit path's attention of single tokens: one block serves the query heads that share
+    a key/value head (up to eight; nine and ten heads take two blocks) from one read of its keys
+    and values. Bit for bit what one block per head gives, for contexts of one span and of many,
+    with and without a list of tokens, with released pages of a window."""
+    ops = _ops()
+    ctx_lens = [1, 127, 128, 129, 700, 2049, 33]
+    q_lens = [1] * len(ctx_lens)
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.float32, seed=31)
+    if window:                                              # pages that the window has passed are released
+        for s, c in enumerate(ctx_lens):
+            table[s, :max(0, (c - window) // page)] = -1
+    n, scale = q.shape[0], hd ** -0.5
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
+    outs = []
+    for grouped in (True, False):
+        out = torch.full_like(q, float("nan"))
+        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, window, grouped=grouped)
+        assert torch.allclose(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    some = [6, 0, 4]
+    part = torch.full_like(q, float("nan"))
+    ops.attn_generic(q, part, kc, vc, pos, seq_of, table, len(some), nq, nkv, hd, page, scale, window, tokens=i32(some))
+    assert torch.equal(part[some], outs[0][some]) and torch.isnan(part[1]).all()
 
 
 @pytest.mark.parametrize("listed", [False, True])
