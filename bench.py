@@ -250,6 +250,7 @@ def main() -> int:
                          "--context tokens that is fed in such portions (chunked prefill late in a long context)")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-tune", action="store_true", help="keep the BLAS library's default kernels for prefill")
+    ap.add_argument("--no-breakdown", action="store_true", help="no per-kernel times of the decode step in the line")
     ap.add_argument("--no-gate", action="store_true", help="skip the check of the engine's output before timing (profiling runs)")
     ap.add_argument("--extras", default="auto", choices=["auto", "on", "off"],
                     help="the further points of the default run: batch 8 at contexts of 16,384 and 32,768 tokens, a "
@@ -309,15 +310,34 @@ def main() -> int:
         checked = None if args.no_gate else gate(engine, cfg.vocab_size, args.dtype, n_layers, model)
         return engine, cfg, full, n_layers, checked
 
-    def decode(engine, cfg, n_layers: int, batch: int, context: int, steps: int, warmup: int) -> dict:
+    PROFILED = 4  # decode steps under the profiler for the per-kernel breakdown
+
+    def kernel_breakdown(sched) -> dict:
+        """Microseconds per decode step of each kernel (the longest ten, by the part of their names
+        that tells them apart), from the device's own trace of a few more steps of this run."""
+        from torch.profiler import ProfilerActivity, profile
+
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            for _ in range(PROFILED):
+                sched.step()
+            sync()
+        rows = sorted(((e.key, e.device_time_total) for e in prof.key_averages() if e.device_time_total > 0), key=lambda r: -r[1])
+        short = lambda k: k.replace("void ", "").replace("(anonymous namespace)::", "").split("(")[0][:48]  # noqa: E731
+        out = {}
+        for key, total in rows[:10]:
+            out[short(key)] = round(out.get(short(key), 0.0) + total / PROFILED, 1)
+        out["all kernels"] = round(sum(t for _, t in rows) / PROFILED, 1)
+        return out
+
+    def decode(engine, cfg, n_layers: int, batch: int, context: int, steps: int, warmup: int, breakdown: bool = False) -> dict:
         """Three timed blocks of `steps` decode steps at `batch`; the block of median time counts.
-        The last block ends at the full context."""
+        The last block ends at the full context (`breakdown`: a few steps under the profiler follow)."""
         weight_bytes, kv_per_token, _ = model_numbers(cfg, n_layers, dtype_bytes)
         sched = Scheduler(engine, max_batch=batch)
         # Requests whose prompt is done decode while the others are still being
         # prefilled (one step per portion of a prompt), so leave room for those tokens too.
         portions = -(-context // PREFILL_TOKENS)
-        start_ctx = context - (BLOCKS * steps + warmup) - portions * batch - 2
+        start_ctx = context - (BLOCKS * steps + warmup) - portions * batch - 2 - (PROFILED if breakdown else 0)
         for _ in range(batch):
             sched.add_request([rng.randrange(cfg.vocab_size) for _ in range(start_ctx)], max_new_tokens=context - start_ctx)
         t_fill = time.perf_counter()
@@ -338,12 +358,18 @@ def main() -> int:
                 assert len(out) == batch
             sync()
             blocks.append((time.perf_counter() - t, ctx0 + steps / 2))
+        kernels = None
+        if breakdown:
+            try:
+                kernels = kernel_breakdown(sched)
+            except Exception as e:  # noqa: BLE001  (a profiler that is not there costs the run nothing)
+                kernels = {"error": repr(e)[:120]}
         for r in list(sched.running):
             engine.finish(r.seq_id)
         dt, mean_ctx = sorted(blocks)[BLOCKS // 2]
         ms = dt / steps * 1e3
         achieved = (weight_bytes + batch * mean_ctx * kv_per_token) / (ms / 1e3) / 1e9
-        return {"tok_s": batch * steps / dt, "ms": ms, "gbs": achieved, "frac": achieved / HBM_PEAK_GBS}
+        return {"tok_s": batch * steps / dt, "ms": ms, "gbs": achieved, "frac": achieved / HBM_PEAK_GBS, "kernels": kernels}
 
     def prefill_of(engine, cfg, n_layers: int) -> dict:
         _, _, prefill_flops = model_numbers(cfg, n_layers, dtype_bytes)
@@ -401,7 +427,7 @@ def main() -> int:
         print(json.dumps({"metric": "prefill tok/s (%s shape, %d tokens)" % (args.model, PREFILL_TOKENS),
                           "prefill": prefill, "portion": portion, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32"}))
         return 0
-    main_point = decode(engine, cfg, n_layers, args.batch, args.context, args.steps, args.warmup)
+    main_point = decode(engine, cfg, n_layers, args.batch, args.context, args.steps, args.warmup, breakdown=not args.no_breakdown)
     value, ms_per_step, achieved = main_point["tok_s"], main_point["ms"], main_point["gbs"]
     pts, pts_ms, pts_frac = {}, {}, {}
 
@@ -473,7 +499,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "frac_of_measured": round(achieved / measured_read, 4)},
         "points": pts, "points_ms_per_step": pts_ms, "points_hbm_frac": pts_frac,
-        "measured_read_gbs": measured_read, "peak_mem_gb": peak_mem, "pool_pages": pool_pages,
+        "kernels_us_per_step": main_point["kernels"], "measured_read_gbs": measured_read, "peak_mem_gb": peak_mem, "pool_pages": pool_pages,
         "gate": gates, "extras_failed": failed,
         "timing": "median of %d timed blocks of %d steps" % (BLOCKS, args.steps), "env": environment(),
     }
