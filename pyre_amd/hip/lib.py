@@ -105,8 +105,12 @@ def loaded_path() -> str | None:
     return None if _lib is None else _lib._name
 
 
+_entry_points: dict = {}
+
+
 def call(name: str, *args) -> None:
-    handle = lib()
-    rc = getattr(handle, name)(*args)
-    if rc != 0:
-        raise KernelError(handle.pyre_last_error().decode(errors="replace"))
+    fn = _entry_points.get(name)
+    if fn is None:
+        fn = _entry_points[name] = getattr(lib(), name)
+    if fn(*args) != 0:
+        raise KernelError(lib().pyre_last_error().decode(errors="replace"))

@@ -9,6 +9,7 @@ not on a GPU is an error.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from functools import lru_cache
 
 import torch
 
@@ -455,6 +456,7 @@ def feed_tokens(tokens: torch.Tensor, src: torch.Tensor, ids: torch.Tensor, n: i
     call("pyre_feed_tokens", tokens.data_ptr(), src.data_ptr(), ids.data_ptr(), n, _stream())
 
 
+@lru_cache(maxsize=4096)
 def attn_mfma_supports(hd: int, page_size: int, nq: int, nkv: int) -> bool:
     from pyre_amd.hip.lib import lib
 
@@ -506,6 +508,7 @@ def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_o
          block_table.stride(0), nq, nkv, hd, page_size, float(scale), int(window), _stream())
 
 
+@lru_cache(maxsize=4096)
 def attn_prefill_waves(nq: int, nkv: int) -> int:
     from pyre_amd.hip.lib import lib
 
@@ -532,6 +535,7 @@ def attn_prefill_work_bf16(q, out, k_cache, v_cache, work, n_items, partials, co
          nq, nkv, hd, page_size, float(scale), int(window), _stream())
 
 
+@lru_cache(maxsize=4096)
 def gemm_skinny_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
     from pyre_amd.hip.lib import lib
 
@@ -569,6 +573,7 @@ def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.T
          out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
 
 
+@lru_cache(maxsize=4096)
 def gemm_mid_supports(m: int, n: int, k: int, ldx: int, ldw: int) -> bool:
     from pyre_amd.hip.lib import lib
 
@@ -586,6 +591,7 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, k
          w.shape[1], ksplit, int(wide), _stream())
 
 
+@lru_cache(maxsize=4096)
 def gemm_mid_silu_blocks(m: int, two_i: int) -> int:
     from pyre_amd.hip.lib import lib
 
