@@ -465,7 +465,7 @@ def main() -> int:
             try:
                 torch.cuda.reset_peak_memory_stats()
                 eng2, cfg2, _, layers2, gates[other] = build(other, None, args.batch, context, args.batch * context, False)
-                note(f"{tag}_decode_b{args.batch}_ctx{context}", decode(eng2, cfg2, layers2, args.batch, context, short, args.warmup))
+                note(f"{tag}_decode_b{args.batch}_ctx{context}", decode(eng2, cfg2, layers2, args.batch, context, args.steps, args.warmup))
                 peak_mem[other] = round(torch.cuda.max_memory_allocated() / 2**30, 2)
                 del eng2
             except Exception as e:  # noqa: BLE001
