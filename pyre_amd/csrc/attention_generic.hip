@@ -146,135 +146,180 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(
   }
 }
 
-// The same for the query heads that share a key/value head, float32 throughout: one block per
-// (token, key/value head and group of up to kGroupHeads of its query heads, span of keys), so
-// that a span's keys and values are read once for the group and not once per head (a decode
-// step's attention is all memory traffic). Every number is computed exactly as the kernel
-// above computes it, by the same chain of operations in the same order: a score by one thread
-// (the key's, for all heads of the group) over the head's elements in ascending order; a span's sum of probabilities by the same
-// reduction over the same layout of threads (key j in lane j % 64 of wave j / 64, the waves'
-// sums added in their order); an output element over the keys 4 g, 4 g + 1, ... of its thread's
-// set, the sets' sums added in their order. The two kernels give the same bits; this one needs
-// head and page sizes that are multiples of four (VEC above).
-constexpr int kGroupHeads = 8;
+// The same for the query heads that share a key/value head, float32 throughout, on the matrix
+// cores' float32 instruction 16x16x4: one block per (token, key/value head with up to 16 of its
+// query heads, span of keys), so that a span's keys and values are read once for the group and
+// not once per head (a decode step's attention is all memory traffic). The instruction's 16
+// columns are the query heads; its 16 rows are 16 keys (scores) or 16 elements of the head
+// (output). It adds an element's products one after the other with fused multiply-adds, in the
+// order of its four lane groups, so every sum here is a chain in a fixed order too: a score over
+// the head's elements 0, 4, 8, 12, 1, 5, ... of each run of 16 (a lane holds four consecutive
+// elements of its key, one 16-byte load), an output element over the keys of the span in the same
+// order within each run of 16 keys, the runs in ascending order. Keys are taken in runs of 16 that
+// start at multiples of 16 (inside one page: the page size is a multiple of 16); those of a run
+// outside lo..pos get the weight 0, and what they hold is finite (older keys of the request) or zero
+// (behind its last key). A wave issues the loads of all its keys and values before it multiplies, so
+// the whole span is on its way at once. Head sizes that are multiples of 16 up to 128.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+constexpr int kSingleHeads = 16;
 
-__global__ __launch_bounds__(kThreads) void attn_grouped_f32_kernel(
+// ALIGNED: no window, so a span starts at a multiple of 128 and touches eight runs; else nine.
+template <int HT, bool ALIGNED>  // head size / 16
+__global__ __launch_bounds__(kThreads) void attn_single_f32_kernel(
     const float* __restrict__ q, const float* __restrict__ k_cache, const float* __restrict__ v_cache,
     float* __restrict__ out, const int* __restrict__ tokens, const int* __restrict__ positions,
     const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride, int nq, int nkv,
-    int hd, int page_size, float scale, int window, float* __restrict__ part) {
-  __shared__ __attribute__((aligned(16))) float sc[kGroupHeads][kSpan];
-  __shared__ float accs[kGroupHeads][kThreads];
-  __shared__ float ml[kGroupHeads][2];  // maximum and sum of each head's span
-  __shared__ float scratch[16];
+    int page_size, float scale, int window, float* __restrict__ part) {
+  constexpr int hd = 16 * HT;
+  constexpr int kRuns = kSpan / 16 + (ALIGNED ? 0 : 1);
+  constexpr int kScoreLd = kRuns * 16 + 4, kQLd = hd + 4;  // rows that start four banks apart
+  constexpr int kMyRuns = (kRuns + 3) / 4;         // runs of keys whose scores one wave computes
+  constexpr int kMyTiles = (HT + 3) / 4;           // tiles of 16 output elements of one wave
+  constexpr int kEarly = kRuns / 2;                // runs whose values are asked for before the scores are computed
+  __shared__ __attribute__((aligned(16))) float sc[kSingleHeads][kScoreLd];
+  __shared__ __attribute__((aligned(16))) float qs[kSingleHeads][kQLd];
+  __shared__ float ml[kSingleHeads][2];  // maximum and sum of each head's span
 
   const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, tid = threadIdx.x;
-  const int n_rep = nq / nkv, per_kv = (n_rep + kGroupHeads - 1) / kGroupHeads;
-  const int kvh = blockIdx.y / per_kv, head0 = kvh * n_rep + (blockIdx.y % per_kv) * kGroupHeads;
-  const int nheads = min(kGroupHeads, kvh * n_rep + n_rep - head0);
+  const int wave = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+  const int n_rep = nq / nkv, per_kv = (n_rep + kSingleHeads - 1) / kSingleHeads;
+  const int kvh = blockIdx.y / per_kv, head0 = kvh * n_rep + (blockIdx.y % per_kv) * kSingleHeads;
+  const int nheads = min(kSingleHeads, kvh * n_rep + n_rep - head0);
   const int pos = positions[n];
   const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int base = lo + static_cast<int>(blockIdx.z) * kSpan;  // this block's span
   if (base > pos) return;
-  const int cnt = min(kSpan, pos - base + 1);
+  const int last = min(pos, base + kSpan - 1);
+  const int first = base & ~15, nruns = (last >> 4) - (base >> 4) + 1;
 
-  // Scores: thread j < 128 takes key base + j for every head of the group (each row of keys is read by
-  // one thread only: a wave's load touches 64 lines, and the address unit's time is what this phase
-  // costs). The queries are the same for every lane: they come through scalar loads.
-  const int j = tid;
-  const float* qg = q + (static_cast<size_t>(n) * nq + head0) * hd;
-  float s[kGroupHeads];
+  // Where this wave's runs of keys lie; a page that is not there (padding rows of a captured
+  // step) hides its keys. All loads of the keys are issued before anything waits for one.
+  const float* krow[kMyRuns];
 #pragma unroll
-  for (int h = 0; h < kGroupHeads; ++h) s[h] = -INFINITY;
-  if (j < cnt) {
-    const int key = base + j;
-    const int page = table[key / page_size], off = key % page_size;
-    if (page >= 0) {  // a page that is not there (padding rows of a captured step) hides its keys
-      const float* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * hd;
-#pragma unroll
-      for (int h = 0; h < kGroupHeads; ++h) s[h] = 0.f;
-#pragma unroll 8
-      for (int e = 0; e < hd; e += 4) {
-        float kv[4];
-        load4(kp + e, kv);
-#pragma unroll
-        for (int h = 0; h < kGroupHeads; ++h)
-          if (h < nheads) {
-#pragma unroll
-            for (int u = 0; u < 4; ++u) s[h] = fmaf(qg[h * hd + e + u], kv[u], s[h]);
-          }
-      }
-#pragma unroll
-      for (int h = 0; h < kGroupHeads; ++h) s[h] *= scale;
+  for (int i = 0; i < kMyRuns; ++i) {
+    const int r = wave + 4 * i;
+    krow[i] = nullptr;
+    if (r < nruns) {
+      const int key0 = first + 16 * r, page = table[key0 / page_size];
+      if (page >= 0)
+        krow[i] = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + key0 % page_size + c16) * hd + 4 * g;
     }
   }
-  // Softmax of the span, head by head: the maximum, the probabilities, their sum (key j in lane
-  // j % 64 of wave j / 64, the other two waves add zeros).
+  f32x4 kreg[kMyRuns][HT];
 #pragma unroll
-  for (int h = 0; h < kGroupHeads; ++h) {
-    if (h >= nheads) break;
-    const bool mine = j < cnt;
-    const float m = block_max(mine ? s[h] : -INFINITY, scratch);
-    const float m_use = m == -INFINITY ? 0.f : m;
-    const float p = mine ? expf(s[h] - m_use) : 0.f;
-    if (mine) sc[h][j] = p;
-    const float l = block_sum(p, scratch);  // its barriers publish sc[h][]
-    if (tid == 0) ml[h][0] = m, ml[h][1] = l;
-  }
-
-  // Output: set g of hd threads takes the groups of four keys g, g + groups, ... of the span for element d.
-  const int groups = kThreads / hd;  // >= 1 because hd <= 256
-  const int g = tid / hd, d = tid % hd;
-  float acc[kGroupHeads];
+  for (int i = 0; i < kMyRuns; ++i)
+    if (krow[i]) {
 #pragma unroll
-  for (int h = 0; h < kGroupHeads; ++h) acc[h] = 0.f;
-  if (g < groups) {
-#pragma unroll 2
-    for (int quad = base / 4 + g; quad <= (base + cnt - 1) / 4; quad += groups) {
-      const int key = 4 * quad;
-      const int page = table[key / page_size], off = key % page_size;
-      if (page < 0) continue;
-      float vv[4];
-      load4(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + d) * page_size + off, vv);
-      if (key >= base && key + 3 < base + cnt && ((key - base) & 3) == 0) {  // the whole group, its probabilities in one read
+      for (int b = 0; b < HT; ++b) kreg[i][b] = *reinterpret_cast<const f32x4*>(krow[i] + 16 * b);
+    }
+  // The values: tiles wave, wave + 4 of the head's elements, every run of the span; the first runs
+  // now, the others when the keys' registers are free.
+  f32x4 vreg[kRuns][kMyTiles];
+  bool vthere[kRuns];
+  auto ask_values = [&](int r) {
+    vthere[r] = false;
+    if (r < nruns) {
+      const int key0 = first + 16 * r, page = table[key0 / page_size];
+      vthere[r] = page >= 0;
+      if (page >= 0) {
+        const float* vp = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + c16) * page_size + key0 % page_size + 4 * g;
 #pragma unroll
-        for (int h = 0; h < kGroupHeads; ++h)
-          if (h < nheads) {
-            const float4 p = *reinterpret_cast<const float4*>(&sc[h][key - base]);
-            acc[h] = fmaf(p.x, vv[0], acc[h]);
-            acc[h] = fmaf(p.y, vv[1], acc[h]);
-            acc[h] = fmaf(p.z, vv[2], acc[h]);
-            acc[h] = fmaf(p.w, vv[3], acc[h]);
-          }
-        continue;
+        for (int t = 0; t < kMyTiles; ++t)
+          if (wave + 4 * t < HT) vreg[r][t] = *reinterpret_cast<const f32x4*>(vp + static_cast<size_t>(16 * (wave + 4 * t)) * page_size);
       }
+    }
+  };
+#pragma unroll
+  for (int r = 0; r < kEarly; ++r) ask_values(r);
+  // the queries of the group's heads, through LDS (rows of heads that are not there: zeros)
+  for (int i = tid; i < kSingleHeads * (hd / 4); i += kThreads) {
+    const int h = i / (hd / 4), e = 4 * (i % (hd / 4));
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (h < nheads) v = *reinterpret_cast<const f32x4*>(q + (static_cast<size_t>(n) * nq + head0 + h) * hd + e);
+    *reinterpret_cast<f32x4*>(&qs[h][e]) = v;
+  }
+  __syncthreads();
+
+  // Scores: rows are the run's keys, columns the heads; this lane gets keys 4 g .. 4 g + 3 of the run for head c16.
+#pragma unroll
+  for (int i = 0; i < kMyRuns; ++i) {
+    const int r = wave + 4 * i;
+    if (r < nruns) {
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+      if (krow[i]) {
+#pragma unroll
+        for (int b = 0; b < HT; ++b) {
+          const f32x4 qv = *reinterpret_cast<const f32x4*>(&qs[c16][16 * b + 4 * g]);  // head c16, this lane group's elements
+#pragma unroll
+          for (int u = 0; u < 4; ++u) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[i][b][u], qv[u], s, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int key = first + 16 * r + 4 * g + u;
+        s[u] = krow[i] && key >= base && key <= last ? s[u] * scale : -INFINITY;
+      }
+      *reinterpret_cast<f32x4*>(&sc[c16][16 * r + 4 * g]) = s;
+    }
+  }
+#pragma unroll
+  for (int r = kEarly; r < kRuns; ++r) ask_values(r);
+  __syncthreads();
+
+  // Softmax of the span, 16 threads a head: thread t of them takes the keys t, t + 16, ... of the runs.
+  {
+    const int h = tid >> 4, t = tid & 15;
+    float m = -INFINITY;
+    for (int j = t; j < 16 * nruns; j += 16) m = fmaxf(m, sc[h][j]);
+#pragma unroll
+    for (int x = 8; x > 0; x >>= 1) m = fmaxf(m, __shfl_xor(m, x, 16));
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float l = 0.f;
+    for (int j = t; j < 16 * nruns; j += 16) {
+      const float p = expf(sc[h][j] - m_use);  // 0 for the keys outside the span
+      sc[h][j] = p;
+      l += p;
+    }
+#pragma unroll
+    for (int x = 8; x > 0; x >>= 1) l += __shfl_xor(l, x, 16);
+    if (t == 0) ml[h][0] = m, ml[h][1] = l;
+  }
+  __syncthreads();
+
+  // Output: rows are 16 elements of the head, columns the heads; the keys of the span run by run.
+  f32x4 acc[kMyTiles];
+#pragma unroll
+  for (int t = 0; t < kMyTiles; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < kRuns; ++r) {
+    if (r < nruns && vthere[r]) {
+      const f32x4 p = *reinterpret_cast<const f32x4*>(&sc[c16][16 * r + 4 * g]);
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        if (key + u >= base && key + u < base + cnt) {
 #pragma unroll
-          for (int h = 0; h < kGroupHeads; ++h)
-            if (h < nheads) acc[h] = fmaf(sc[h][key + u - base], vv[u], acc[h]);
-        }
+        for (int t = 0; t < kMyTiles; ++t)
+          if (wave + 4 * t < HT) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vreg[r][t][u], p[u], acc[t], 0, 0, 0);
     }
   }
+  if (c16 >= nheads) return;
+  const int h = head0 + c16;
+  const float m = ml[c16][0], l = ml[c16][1];
 #pragma unroll
-  for (int h = 0; h < kGroupHeads; ++h) accs[h][tid] = g < groups ? acc[h] : 0.f;
-  __syncthreads();
-  for (int i = tid; i < nheads * hd; i += kThreads) {
-    const int h = i / hd, dd = i % hd;
-    float total = 0.f;
-    for (int gg = 0; gg < groups; ++gg) total += accs[h][gg * hd + dd];
+  for (int t = 0; t < kMyTiles; ++t) {
+    if (wave + 4 * t >= HT) continue;
+    const int d = 16 * (wave + 4 * t) + 4 * g;  // this lane's four elements
     if (part) {  // [token of the list][head][span][hd + 2]: unnormalised output, max, sum
-      float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + head0 + h) * gridDim.z + blockIdx.z) * (hd + 2);
-      dst[dd] = total;
-      if (dd == 0) {
-        dst[hd] = ml[h][0];
-        dst[hd + 1] = ml[h][1];
-      }
+      float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + h) * gridDim.z + blockIdx.z) * (hd + 2);
+      *reinterpret_cast<f32x2*>(dst + d) = f32x2{acc[t][0], acc[t][1]};  // rows of hd + 2 floats start on 8 bytes
+      *reinterpret_cast<f32x2*>(dst + d + 2) = f32x2{acc[t][2], acc[t][3]};
+      if (d == 0) dst[hd] = m, dst[hd + 1] = l;
     } else {
-      const float l = ml[h][1];
-      out[(static_cast<size_t>(n) * nq + head0 + h) * hd + dd] = l > 0.f ? total / l : 0.f;
+      f32x4 o;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) o[u] = l > 0.f ? acc[t][u] / l : 0.f;
+      *reinterpret_cast<f32x4*>(out + (static_cast<size_t>(n) * nq + h) * hd + d) = o;
     }
   }
 }
@@ -317,7 +362,7 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
                                  const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                                  const int* seq_of_token, const int* block_table, int table_stride,
                                  int n, int nq, int nkv, int hd, int page_size, float scale,
-                                 int window, int max_keys, float* part, int grouped, hipStream_t stream) {
+                                 int window, int max_keys, float* part, int matrix_cores, hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(q_dt) && known_dtype(cache_dt), "attn_generic: unknown dtype");
   PYRE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attn_generic: %d query heads do not divide over %d kv heads", nq, nkv);
   PYRE_REQUIRE(hd > 0 && hd <= kMaxHead, "attn_generic: head_dim %d is outside 1..%d", hd, kMaxHead);
@@ -331,14 +376,27 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
   float* scratch = spans == 1 ? nullptr : part;
   const bool vec = hd % 4 == 0 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
-  if (grouped && vec && q_dt == kF32 && cache_dt == kF32) {
+  const bool aligned = reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                       (!scratch || reinterpret_cast<uintptr_t>(scratch) % 8 == 0);
+  if (matrix_cores && vec && aligned && q_dt == kF32 && cache_dt == kF32 && hd % 16 == 0 && hd <= 128 && page_size % 16 == 0) {
     // the query heads of a key/value head together: the span's keys and values are read once for all of them
-    const int per_kv = (nq / nkv + kGroupHeads - 1) / kGroupHeads;
+    const int per_kv = (nq / nkv + kSingleHeads - 1) / kSingleHeads;
     PYRE_REQUIRE(nkv * per_kv <= 65535, "attn_generic: too many heads");
-    hipLaunchKernelGGL(attn_grouped_f32_kernel, dim3(n, nkv * per_kv, spans), dim3(kThreads), 0, stream,
-                       static_cast<const float*>(q), static_cast<const float*>(k_cache),
-                       static_cast<const float*>(v_cache), static_cast<float*>(out), tokens, positions, seq_of_token,
-                       block_table, table_stride, nq, nkv, hd, page_size, scale, window, scratch);
+#define PYRE_SINGLE_AS(HT, ALIGNED)                                                                                  \
+  hipLaunchKernelGGL((attn_single_f32_kernel<HT, ALIGNED>), dim3(n, nkv * per_kv, spans), dim3(kThreads), 0, stream, \
+                     static_cast<const float*>(q), static_cast<const float*>(k_cache),                               \
+                     static_cast<const float*>(v_cache), static_cast<float*>(out), tokens, positions, seq_of_token,   \
+                     block_table, table_stride, nq, nkv, page_size, scale, window, scratch)
+#define PYRE_SINGLE(HT)                     \
+  case HT:                                  \
+    if (window > 0) PYRE_SINGLE_AS(HT, false); \
+    else PYRE_SINGLE_AS(HT, true);          \
+    break
+    switch (hd / 16) {
+      PYRE_SINGLE(1); PYRE_SINGLE(2); PYRE_SINGLE(3); PYRE_SINGLE(4); PYRE_SINGLE(5); PYRE_SINGLE(6); PYRE_SINGLE(7); PYRE_SINGLE(8);
+    }
+#undef PYRE_SINGLE
+#undef PYRE_SINGLE_AS
     if (spans > 1)
       hipLaunchKernelGGL((attn_generic_join_kernel<float>), dim3(n, nq), dim3(kThreads), 0, stream, scratch,
                          static_cast<float*>(out), tokens, positions, nq, hd, window, spans);

@@ -8,12 +8,16 @@
 // 32 rows of an MFMA tile are output columns n, its 32 columns are rows m, so that a lane
 // holds runs of four consecutive n of one row m and stores them as one float4.
 //
-// k is walked in stages of 16 through LDS; within a stage, MFMA step s (0..7) multiplies k = s
-// in lanes 0..31 and k = 8 + s in lanes 32..63, so that every lane reads its eight values of a
-// stage as two 16-byte LDS loads. The order in which the products of an output element are
-// added is therefore (0, 8), (1, 9), ..., (7, 15), (16, 24), ...: a function of k alone. Both
-// tile shapes below walk k the same way, so an element's value does not depend on the shape,
-// on the number of rows in the step or on where the row lies in it, bit for bit.
+// The instruction adds an element's products one after the other, each with one fused
+// multiply-add, in the order of its k (for 32x32x2: lanes 0..31, then lanes 32..63; for 16x16x4:
+// the four groups of 16 lanes in turn), exactly as a chain of fmaf() does. k is walked in stages
+// of 16 through LDS, and within a stage in the order 0, 4, 8, 12, 1, 5, 9, 13, 2, ..., 15: step s
+// (0..7) of 32x32x2 multiplies k = 8 (s & 1) + (s >> 1) in lanes 0..31 and that k + 4 in lanes
+// 32..63, so that a lane reads its eight values of a stage as two 16-byte LDS loads (pieces
+// `half` and `half` + 2); step i (0..3) of 16x16x4 multiplies k = 4 g + i in its lane group g (one
+// 16-byte load). The order in which an element's products are added is a function of k alone and
+// the same for every tile shape and both instructions below, so an element's value does not depend
+// on the shape, on the number of rows in the step or on where the row lies in it, bit for bit.
 //
 // k may be split into `ksplit` parts (grid.z), each writing a partial sum out[s] that the
 // consumer adds in the order 0..ksplit-1: products with few output columns and a long k would
@@ -102,18 +106,18 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_f32_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < TN; ++t)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) a[t][h] = *reinterpret_cast<const f32x4*>(&Ws[(wn * TN + t) * 32 + c][8 * half + 4 * h]);
+      for (int h = 0; h < 2; ++h) a[t][h] = *reinterpret_cast<const f32x4*>(&Ws[(wn * TN + t) * 32 + c][4 * half + 8 * h]);
 #pragma unroll
     for (int u = 0; u < TM; ++u)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) b[u][h] = *reinterpret_cast<const f32x4*>(&As[(wm * TM + u) * 32 + c][8 * half + 4 * h]);
+      for (int h = 0; h < 2; ++h) b[u][h] = *reinterpret_cast<const f32x4*>(&As[(wm * TM + u) * 32 + c][4 * half + 8 * h]);
 #pragma unroll
     for (int s = 0; s < 8; ++s)
 #pragma unroll
       for (int t = 0; t < TN; ++t)
 #pragma unroll
         for (int u = 0; u < TM; ++u)
-          acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s >> 2][s & 3], b[u][s >> 2][s & 3], acc[t][u], 0, 0, 0);
+          acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s & 1][s >> 1], b[u][s & 1][s >> 1], acc[t][u], 0, 0, 0);
     __syncthreads();
   }
 
@@ -146,8 +150,8 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_f32_mfma_kernel(
 
 // The same product for a decode step's rows (M <= 64), as a stream over the weights. A block
 // is one wave with 32 output columns, so there is no barrier. It has a ring of R slots in LDS, a
-// slot being 32 k (two stages) of its 32 rows of W (4 KB) and of XR rows of A (XR = 8, 32 or 64,
-// whichever holds M: 1, 4 or 8 KB), filled by loads that go from memory straight into LDS: while
+// slot being 32 k (two stages) of its 32 rows of W (4 KB) and of XR rows of A (XR = 8, 16, 32 or 64,
+// whichever holds M: 1 to 8 KB), filled by loads that go from memory straight into LDS: while
 // slot j is multiplied, slot j + 1 is read from LDS into registers and the R - 2 after it are on
 // their way. A load instruction takes whole 128-byte lines (8 rows x 32 k); the 16-byte pieces
 // of a row are exchanged among themselves by the row's number so that the matrix instruction's
@@ -206,8 +210,7 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
 #pragma unroll
   for (int i = 0; i < XL; ++i) {
     const int r = 8 * i + lr;
-    // eight rows or fewer: every lane of the instruction reads row c % 8 (no exchange of pieces needed)
-    xk[i] = XR == 8 ? 4 * lp : 4 * (lp ^ ((r >> 1) & 7));
+    xk[i] = 4 * (lp ^ ((r >> 1) & 7));
     xrow[i] = r < M;
     xsrc[i] = A + static_cast<size_t>(xrow[i] ? r : 0) * lda + kbeg + xk[i];
   }
@@ -225,27 +228,92 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
     for (int i = 0; i < XL; ++i) load_to_lds(xrow[i] && xk[i] < left ? xsrc[i] + k0 : zero, dst + 4096 + 1024 * i);
   };
 
+  if constexpr (XR <= 16) {
+    // Sixteen rows or fewer: 16x16x4, whose 16 columns hold the step's rows and whose 16 rows are
+    // output columns, two tiles of them a wave. It takes a weight once for 16 rows where 32x32x2
+    // takes it once for 32, so that a wave gets through its weights in half the time.
+    const int g = lane >> 4, c16 = lane & 15;
+    f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    const int xr = XR == 8 ? c16 & 7 : c16;  // eight rows: the instruction's columns 8..15 read them again and are not stored
+    const unsigned char* wpiece0 = ring + c16 * 128;
+    const unsigned char* wpiece1 = ring + (16 + c16) * 128;
+    const unsigned char* xpiece = ring + 4096 + xr * 128;
+    const int swz = (c16 >> 1) & 7, xswz = (xr >> 1) & 7;  // rows c16 and 16 + c16 exchange their pieces alike
+    int at = 0;
+    auto read = [&](f32x4 (&a)[2][2], f32x4 (&b)[2]) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int piece = 4 * t + g;
+        a[0][t] = *reinterpret_cast<const f32x4*>(wpiece0 + at * kSlotBytes + 16 * (piece ^ swz));
+        a[1][t] = *reinterpret_cast<const f32x4*>(wpiece1 + at * kSlotBytes + 16 * (piece ^ swz));
+        b[t] = *reinterpret_cast<const f32x4*>(xpiece + at * kSlotBytes + 16 * (piece ^ xswz));
+      }
+      at = at + 1 == R ? 0 : at + 1;
+    };
+#pragma unroll
+    for (int j = 0; j < R - 1; ++j) issue(j);
+    f32x4 a[2][2], b[2], an[2][2], bn[2];
+    wait_loads<L * (R - 2)>();
+    read(a, b);
+    for (int j = 0; j < slots; ++j) {
+      issue(j + R - 1);
+      wait_loads<L * (R - 2)>();
+      read(an, bn);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        if (kSlotK * j + BK * t >= K - kbeg) break;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int u = 0; u < 2; ++u) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][t][i], b[t][i], acc[u], 0, 0, 0);
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        a[0][t] = an[0][t];
+        a[1][t] = an[1][t];
+        b[t] = bn[t];
+      }
+    }
+    wait_loads<0>();
+    // acc[u][j]: output column n = 16 u + 4 g + j, output row m = c16.
+    if (c16 >= M || c16 >= XR) return;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int n = n0 + 16 * u + 4 * g;
+      if (n >= N) continue;
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[j] = acc[u][j];
+        if (bias && n + j < N) v[j] += load_as_float(bias, bias_dt, n + j);
+      }
+      float* dst = out + static_cast<size_t>(c16) * ldo + n;
+      if (n + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+      } else {
+        for (int j = 0; j < 4 && n + j < N; ++j) dst[j] = v[j];
+      }
+    }
+  } else {
   f32x16 acc[MT];
 #pragma unroll
   for (int u = 0; u < MT; ++u)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[u][i] = 0.f;
   const unsigned char* wpiece = ring + c * 128;
-  const unsigned char* xpiece = ring + 4096 + (XR == 8 ? c & 7 : c) * 128;
-  const int swz = (c >> 1) & 7, xswz = XR == 8 ? 0 : swz;  // rows c and 32 + c exchange their pieces alike
-  const bool has_x = XR != 8 || c < M;
+  const unsigned char* xpiece = ring + 4096 + c * 128;
+  const int swz = (c >> 1) & 7;  // rows c and 32 + c exchange their pieces alike
   int at = 0;  // ring position of the next slot to read
   auto read = [&](f32x4 (&a)[2][2], f32x4 (&b)[MT][2][2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int piece = 4 * t + 2 * half + h;
+        const int piece = 4 * t + half + 2 * h;
         a[t][h] = *reinterpret_cast<const f32x4*>(wpiece + at * kSlotBytes + 16 * (piece ^ swz));
 #pragma unroll
         for (int u = 0; u < MT; ++u) {
-          b[u][t][h] = *reinterpret_cast<const f32x4*>(xpiece + at * kSlotBytes + 4096 * u + 16 * (piece ^ xswz));
-          if (!has_x) b[u][t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+          b[u][t][h] = *reinterpret_cast<const f32x4*>(xpiece + at * kSlotBytes + 4096 * u + 16 * (piece ^ swz));
         }
       }
     at = at + 1 == R ? 0 : at + 1;
@@ -269,7 +337,7 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
       for (int s = 0; s < 8; ++s)
 #pragma unroll
         for (int u = 0; u < MT; ++u)
-          acc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s >> 2][s & 3], b[u][t][s >> 2][s & 3], acc[u], 0, 0, 0);
+          acc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s & 1][s >> 1], b[u][t][s & 1][s >> 1], acc[u], 0, 0, 0);
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -305,6 +373,7 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
       }
     }
   }
+  }
 }
 
 }  // namespace
@@ -330,6 +399,7 @@ extern "C" int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw,
                      static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),                       \
                      static_cast<size_t>(part_stride), M, N, K, kper)
     if (M <= 8) PYRE_STREAM(4, 8);
+    else if (M <= 16) PYRE_STREAM(4, 16);
     else if (M <= 32) PYRE_STREAM(4, 32);
     else PYRE_STREAM(3, 64);
 #undef PYRE_STREAM

@@ -92,15 +92,17 @@ int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, long ldw, vo
 // tokens: the n tokens of the flat batch to attend for, or null for tokens 0..n-1. max_keys: a
 // bound on the keys that any of them sees (the block table's width in tokens will do); part:
 // n * nq * pyre_attn_generic_spans(max_keys) * (hd + 2) floats of scratch when that is more than one span.
-// grouped: float32 queries and caches with head and page sizes that are multiples of four go to the
-// form of the kernel that reads a span's keys and values once for all query heads of a key/value
-// head (the same bits as one block per head, which 0 asks for).
+// matrix_cores: float32 queries and caches with a head size of 16, 32, ..., 128 and pages of a multiple
+// of 16 tokens go to the kernel that reads a span's keys and values once for all query heads of a
+// key/value head and multiplies on the float32 matrix instruction (its sums run in another order than
+// those of one block per head, which 0 asks for: a difference of rounding). Which kernel runs depends
+// on these sizes alone, never on the tokens of the call.
 int pyre_attn_generic_spans(int max_keys);
 int pyre_attn_generic(const void* q, void* out, int q_dt, const void* k_cache,
                       const void* v_cache, int cache_dt, const int* tokens, const int* positions,
                       const int* seq_of_token, const int* block_table, int table_stride, int n,
                       int nq, int nkv, int hd, int page_size, float scale, int window, int max_keys,
-                      float* part, int grouped, hipStream_t stream);
+                      float* part, int matrix_cores, hipStream_t stream);
 
 // Prompt portions in true float32 on the matrix cores' float32 instruction: tiles as for
 // pyre_attn_prefill_bf16, float32 queries, caches and output, any head size up to 256, any

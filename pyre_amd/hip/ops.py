@@ -297,13 +297,15 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_ca
                  positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                  n: int, nq: int, nkv: int, hd: int, page_size: int, scale: float,
                  window: int = 0, tokens: torch.Tensor | None = None,
-                 scratch: torch.Tensor | None = None, grouped: bool = True) -> None:
+                 scratch: torch.Tensor | None = None, matrix_cores: bool = True) -> None:
     """Causal attention of n tokens over the paged cache (``tokens``: which of the flat batch,
     else the first n); see attention_generic.hip. ``scratch``: float32 memory of
     ``attn_generic_scratch(...)`` elements for the partial results of the spans of keys; without
-    it the memory is allocated here when the block table is wider than one span. ``grouped``: in
-    float32 the query heads that share a key/value head are served from one read of its keys and
-    values where the sizes allow (the same bits as one block per head, which False asks for)."""
+    it the memory is allocated here when the block table is wider than one span. ``matrix_cores``:
+    float32 queries and caches with a head size of 16, 32, ..., 128 and pages of a multiple of 16
+    tokens go to the kernel that serves the query heads of a key/value head from one read of its
+    keys and values, on the matrix cores' float32 instruction (its sums run in another order than
+    those of one block per head, which False asks for: a difference of rounding)."""
     _dev(q, out, k_cache, v_cache, positions, seq_of_token, block_table, tokens, scratch)
     if q.dtype != out.dtype or q.numel() < n * nq * hd or out.numel() < n * nq * hd:
         raise KernelError("attn: q/out buffers do not fit")
@@ -334,7 +336,7 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_ca
         call("pyre_attn_generic", args[0].data_ptr(), args[1].data_ptr(), dtype_code(q), k_cache.data_ptr(),
              v_cache.data_ptr(), dtype_code(k_cache), _ptr(args[2]), args[3].data_ptr(), args[4].data_ptr(),
              block_table.data_ptr(), block_table.stride(0), rows, nq, nkv, hd, page_size, float(scale),
-             int(window), max_keys, _ptr(scratch) if need else None, int(bool(grouped)), _stream())
+             int(window), max_keys, _ptr(scratch) if need else None, int(bool(matrix_cores)), _stream())
 
 
 ATTN_GENERIC_SCRATCH = 1 << 25   #: float32 elements of scratch that one launch of attn_generic may use

@@ -162,24 +162,10 @@ class Attention(Mixer):
             if len(singles):
                 ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, len(singles),
                                  *geometry, tokens=ctx.arrays["attention.decode_tokens"],
-                                 scratch=self._spans_scratch(ctx, cache, len(singles)),
-                                 grouped=self._heads_together(ctx, len(singles)))
+                                 scratch=self._spans_scratch(ctx, cache, len(singles)))
         else:
             ops.attn_generic(q, o, k_pages, v_pages, ctx.positions, ctx.seq_of_token, cache.table, n, *geometry,
-                             scratch=self._spans_scratch(ctx, cache, n), grouped=self._heads_together(ctx, n))
-
-    def _heads_together(self, ctx, n: int) -> bool:
-        """Whether the 32-bit single-token kernel serves the query heads of a key/value head from one
-        block (the keys and values read once for all of them) or each head from its own: the same
-        bits either way, so this is a matter of speed alone. With few tokens and short contexts the
-        blocks of the first form would not fill the chip (a request of 4,096 keys on four key/value
-        heads: 128 blocks), and the second form's seven times as many are faster."""
-        s = self.spec
-        spans = -(-max(1, ctx.host.max_single_ctx or int(ctx.host.ctx_len.max())) // 128)
-        if s.window:
-            spans = min(spans, -(-s.window // 128) + 1)
-        blocks = n * s.num_kv_heads * -(-(s.num_heads // s.num_kv_heads) // 8) * spans
-        return blocks >= 2 * self.units
+                             scratch=self._spans_scratch(ctx, cache, n))
 
     def _spans_scratch(self, ctx, cache, n):
         """Workspace for the partial results of the spans of keys, if the tables are wider than one."""

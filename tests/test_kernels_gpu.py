@@ -127,7 +127,8 @@ def test_gemm_generic(adt, wdt, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 37, 50), (5, 130, 257), (32, 128, 16), (33, 129, 17), (77, 200, 64), (130, 65, 1000),
                                    (300, 3584, 3584), (8, 1000, 18944), (20, 777, 3584), (64, 4608, 3584), (48, 96, 40),
-                                   (33, 1000, 1100)])
+                                   (33, 1000, 1100), (12, 300, 1024), (16, 4608, 3584), (9, 50, 96), (3, 3584, 3584),
+                                   (17, 131, 3584)])
 def test_gemm_f32_on_the_matrix_cores(m, n, k):
     """float32 in, float32 products and sums (the result is as close to a float64 product as
     plain float32 FMAs are), and a row's result bit for bit the same whatever rows share
@@ -338,22 +339,26 @@ def test_attn_generic(dtype, nq, nkv, hd, page, window):
         # one visible key: the output is exactly that key's value (request 0)
         assert torch.allclose(out[0].double().cpu(), dense[0][1][0].double().repeat_interleave(nq // nkv, 0), atol=tol)
     if dtype == "float32":
-        # one block per head and one block for the heads of a key/value head: the same bits
+        # one block per head, with plain multiply-adds, whatever the sizes
         alone = torch.empty_like(q)
-        ops.attn_generic(q, alone, kc, vc, pos, seq_of, table, q.shape[0], nq, nkv, hd, page, scale, window, grouped=False)
-        assert torch.equal(out, alone)
+        ops.attn_generic(q, alone, kc, vc, pos, seq_of, table, q.shape[0], nq, nkv, hd, page, scale, window,
+                         matrix_cores=False)
+        assert torch.allclose(alone.double().cpu(), want, atol=tol, rtol=tol)
 
 
-@pytest.mark.parametrize("nq,nkv,hd,page", [(28, 4, 128, 16), (40, 8, 128, 16), (12, 2, 128, 32), (9, 1, 64, 8), (20, 2, 256, 16),
-                                            (3, 3, 32, 4), (6, 2, 12, 8), (8, 2, 64, 16)])
-@pytest.mark.parametrize("window", [0, 300])
+@pytest.mark.parametrize("nq,nkv,hd,page", [(28, 4, 128, 16), (40, 8, 128, 64), (12, 2, 128, 32), (9, 1, 64, 48), (18, 1, 48, 16),
+                                            (5, 5, 80, 16), (7, 7, 16, 32), (8, 2, 112, 16), (3, 3, 32, 4), (6, 2, 12, 8),
+                                            (20, 2, 256, 16)])
+@pytest.mark.parametrize("window", [0, 300, 77])
 def test_attn_of_single_tokens_by_groups_of_heads_in_float32(nq, nkv, hd, page, window):
     """The 32-bit path's attention of single tokens: one block serves the query heads that share
-    a key/value head (up to eight; nine and ten heads take two blocks) from one read of its keys
-    and values. Bit for bit what one block per head gives, for contexts of one span and of many,
-    with and without a list of tokens, with released pages of a window."""
+    a key/value head (up to 16; 18 heads take two blocks) from one read of its keys and values, on
+    the matrix cores' float32 instruction where the sizes allow (head sizes 16 to 128 in steps of 16,
+    pages of a multiple of 16), for contexts of one span and of many, with and without a list of
+    tokens, with released pages of a window, with spans that start anywhere (a window of 77). The
+    result for a token does not depend on what else the call holds, bit for bit."""
     ops = _ops()
-    ctx_lens = [1, 127, 128, 129, 700, 2049, 33]
+    ctx_lens = [1, 127, 128, 129, 700, 2049, 33, 16, 17]
     q_lens = [1] * len(ctx_lens)
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.float32, seed=31)
     if window:                                              # pages that the window has passed are released
@@ -361,17 +366,37 @@ def test_attn_of_single_tokens_by_groups_of_heads_in_float32(nq, nkv, hd, page, 
             table[s, :max(0, (c - window) // page)] = -1
     n, scale = q.shape[0], hd ** -0.5
     want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, scale, window)
-    outs = []
-    for grouped in (True, False):
-        out = torch.full_like(q, float("nan"))
-        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, window, grouped=grouped)
-        assert torch.allclose(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
-        outs.append(out)
-    assert torch.equal(outs[0], outs[1])
+    out = torch.full_like(q, float("nan"))
+    ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, window)
+    assert torch.allclose(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
     some = [6, 0, 4]
     part = torch.full_like(q, float("nan"))
     ops.attn_generic(q, part, kc, vc, pos, seq_of, table, len(some), nq, nkv, hd, page, scale, window, tokens=i32(some))
-    assert torch.equal(part[some], outs[0][some]) and torch.isnan(part[1]).all()
+    assert torch.equal(part[some], out[some]) and torch.isnan(part[1]).all()
+
+
+def test_attn_of_single_tokens_in_float32_finds_one_key_among_thousands():
+    """One key of 3,000 fits the query, at a place that is no multiple of anything; its value is the
+    output. Then that key lies just outside a window, and the output is far from its value."""
+    ops = _ops()
+    nq, nkv, hd, page = 14, 2, 128, 16
+    ctx_lens, q_lens = [3000], [1]
+    q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.float32, seed=3)
+    K, V = dense[0]                                          # [T, nkv, hd]
+    at = 1717
+    for h in range(nkv):                                     # make key `at` of every key/value head point along its queries
+        for rep in range(nq // nkv):
+            qs[0][0, h * (nq // nkv) + rep] = K[at, h] * 40.0
+    q = qs[0].to(DEV).contiguous()                           # [1, nq, hd]
+    out = torch.full_like(q, float("nan"))
+    ops.attn_generic(q, out, kc, vc, pos, seq_of, table, 1, nq, nkv, hd, page, 1.0)
+    near = V[at].repeat_interleave(nq // nkv, 0)
+    assert torch.allclose(out[0].cpu(), near, atol=1e-4)
+    window = 3000 - 1 - at                                   # the keys at + 1 .. 2999
+    ops.attn_generic(q, out, kc, vc, pos, seq_of, table, 1, nq, nkv, hd, page, 1.0, window)
+    want = attention_plain(qs, dense, ctx_lens, q_lens, nq, nkv, 1.0, window)
+    assert torch.allclose(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
+    assert (out[0].cpu() - near).abs().max() > 0.1
 
 
 @pytest.mark.parametrize("listed", [False, True])
