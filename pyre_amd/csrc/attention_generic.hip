@@ -18,6 +18,8 @@
 // This is the 32-bit path's attention and the 16-bit path's fallback; it stands
 // where the reference has `forward_paged`'s gather + matmuls (pyre/model.py:274-290)
 // and its decode kernel (pyre/kernels/paged_attn.py:26-71).
+#include <type_traits>
+
 #include "pyre_api.h"
 #include "pyre_common.h"
 
@@ -165,74 +167,84 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 constexpr int kSingleHeads = 16;
 
 // ALIGNED: no window, so a span starts at a multiple of 128 and touches eight runs; else nine.
+// A block takes `per_block` spans of its token one after the other (grid.z blocks cover them all):
+// the keys of the next span are asked for as soon as the scores of the current one are computed,
+// its values as soon as the current output is, so that a block always has loads on their way while
+// it multiplies. What a span's partial result is does not depend on per_block.
+// Every span issues the same loads and the same matrix instructions whatever it holds, so that the
+// waits for loads count exactly: a run past the span's end or in a page that is not there (padding
+// rows of a captured step) reads a run that is there, or page 0, and is made harmless afterwards
+// (its scores are -inf, its values zero).
 template <int HT, bool ALIGNED>  // head size / 16
 __global__ __launch_bounds__(kThreads) void attn_single_f32_kernel(
     const float* __restrict__ q, const float* __restrict__ k_cache, const float* __restrict__ v_cache,
     float* __restrict__ out, const int* __restrict__ tokens, const int* __restrict__ positions,
     const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride, int nq, int nkv,
-    int page_size, float scale, int window, float* __restrict__ part) {
+    int page_size, float scale, int window, float* __restrict__ part, int spans, int per_block) {
   constexpr int hd = 16 * HT;
   constexpr int kRuns = kSpan / 16 + (ALIGNED ? 0 : 1);
   constexpr int kScoreLd = kRuns * 16 + 4, kQLd = hd + 4;  // rows that start four banks apart
   constexpr int kMyRuns = (kRuns + 3) / 4;         // runs of keys whose scores one wave computes
   constexpr int kMyTiles = (HT + 3) / 4;           // tiles of 16 output elements of one wave
-  constexpr int kEarly = kRuns / 2;                // runs whose values are asked for before the scores are computed
   __shared__ __attribute__((aligned(16))) float sc[kSingleHeads][kScoreLd];
   __shared__ __attribute__((aligned(16))) float qs[kSingleHeads][kQLd];
   __shared__ float ml[kSingleHeads][2];  // maximum and sum of each head's span
 
   const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wave, and known to be
+  const int lane = tid & 63, g = lane >> 4, c16 = lane & 15;
   const int n_rep = nq / nkv, per_kv = (n_rep + kSingleHeads - 1) / kSingleHeads;
   const int kvh = blockIdx.y / per_kv, head0 = kvh * n_rep + (blockIdx.y % per_kv) * kSingleHeads;
   const int nheads = min(kSingleHeads, kvh * n_rep + n_rep - head0);
   const int pos = positions[n];
   const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int base = lo + static_cast<int>(blockIdx.z) * kSpan;  // this block's span
-  if (base > pos) return;
-  const int last = min(pos, base + kSpan - 1);
-  const int first = base & ~15, nruns = (last >> 4) - (base >> 4) + 1;
+  const int span0 = static_cast<int>(blockIdx.z) * per_block;
+  const int span_end = min(span0 + per_block, (pos - lo) / kSpan + 1);  // the token's spans end here
+  if (span0 >= span_end) return;
 
-  // Where this wave's runs of keys lie; a page that is not there (padding rows of a captured
-  // step) hides its keys. All loads of the keys are issued before anything waits for one.
-  const float* krow[kMyRuns];
-#pragma unroll
-  for (int i = 0; i < kMyRuns; ++i) {
-    const int r = wave + 4 * i;
-    krow[i] = nullptr;
-    if (r < nruns) {
-      const int key0 = first + 16 * r, page = table[key0 / page_size];
-      if (page >= 0)
-        krow[i] = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + key0 % page_size + c16) * hd + 4 * g;
-    }
-  }
+  // A span: its keys base..last, in `nruns` runs of 16 from `first` on.
+  struct Span { int base, last, first, nruns; };
+  auto span_at = [&](int span) {
+    Span sp;
+    sp.base = lo + span * kSpan;
+    sp.last = min(pos, sp.base + kSpan - 1);
+    sp.first = sp.base & ~15;
+    sp.nruns = (sp.last >> 4) - (sp.base >> 4) + 1;
+    return sp;
+  };
+  // The loads of a span's keys (this wave's runs wave, wave + 4, ...) and values (tiles wave,
+  // wave + 4 of the head's elements, every run). All of them are issued before anything waits for one.
   f32x4 kreg[kMyRuns][HT];
+  bool kthere[kMyRuns];
+  auto ask_keys = [&](const Span& sp) {
 #pragma unroll
-  for (int i = 0; i < kMyRuns; ++i)
-    if (krow[i]) {
+    for (int i = 0; i < kMyRuns; ++i) {
+      const int r = wave + 4 * i, key0 = sp.first + 16 * min(r, sp.nruns - 1);
+      const int page = table[key0 / page_size];
+      kthere[i] = r < sp.nruns && page >= 0;
+      const float* kp = k_cache + ((static_cast<size_t>(max(page, 0)) * nkv + kvh) * page_size + key0 % page_size + c16) * hd + 4 * g;
 #pragma unroll
-      for (int b = 0; b < HT; ++b) kreg[i][b] = *reinterpret_cast<const f32x4*>(krow[i] + 16 * b);
-    }
-  // The values: tiles wave, wave + 4 of the head's elements, every run of the span; the first runs
-  // now, the others when the keys' registers are free.
-  f32x4 vreg[kRuns][kMyTiles];
-  bool vthere[kRuns];
-  auto ask_values = [&](int r) {
-    vthere[r] = false;
-    if (r < nruns) {
-      const int key0 = first + 16 * r, page = table[key0 / page_size];
-      vthere[r] = page >= 0;
-      if (page >= 0) {
-        const float* vp = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * hd + c16) * page_size + key0 % page_size + 4 * g;
-#pragma unroll
-        for (int t = 0; t < kMyTiles; ++t)
-          if (wave + 4 * t < HT) vreg[r][t] = *reinterpret_cast<const f32x4*>(vp + static_cast<size_t>(16 * (wave + 4 * t)) * page_size);
-      }
+      for (int b = 0; b < HT; ++b) kreg[i][b] = *reinterpret_cast<const f32x4*>(kp + 16 * b);
     }
   };
+  f32x4 vreg[kRuns][kMyTiles];
+  bool vthere[kRuns];
+  auto ask_values = [&](const Span& sp) {
 #pragma unroll
-  for (int r = 0; r < kEarly; ++r) ask_values(r);
+    for (int r = 0; r < kRuns; ++r) {
+      const int key0 = sp.first + 16 * min(r, sp.nruns - 1);
+      const int page = table[key0 / page_size];
+      vthere[r] = r < sp.nruns && page >= 0;
+      const float* vp = v_cache + ((static_cast<size_t>(max(page, 0)) * nkv + kvh) * hd + c16) * page_size + key0 % page_size + 4 * g;
+#pragma unroll
+      for (int t = 0; t < kMyTiles; ++t)
+        if (HT % 4 == 0 || wave + 4 * t < HT) vreg[r][t] = *reinterpret_cast<const f32x4*>(vp + static_cast<size_t>(16 * (wave + 4 * t)) * page_size);
+    }
+  };
+  Span now = span_at(span0);
+  ask_keys(now);
+  ask_values(now);
   // the queries of the group's heads, through LDS (rows of heads that are not there: zeros)
   for (int i = tid; i < kSingleHeads * (hd / 4); i += kThreads) {
     const int h = i / (hd / 4), e = 4 * (i % (hd / 4));
@@ -242,86 +254,94 @@ __global__ __launch_bounds__(kThreads) void attn_single_f32_kernel(
   }
   __syncthreads();
 
-  // Scores: rows are the run's keys, columns the heads; this lane gets keys 4 g .. 4 g + 3 of the run for head c16.
+  // One span; `ahead`: another one follows, whose loads are issued on the way.
+  auto take = [&](int span, auto ahead) {
+    const Span next = span_at(span + (ahead ? 1 : 0));
+    // Scores: rows are the run's keys, columns the heads; this lane gets keys 4 g .. 4 g + 3 of the run for head c16.
 #pragma unroll
-  for (int i = 0; i < kMyRuns; ++i) {
-    const int r = wave + 4 * i;
-    if (r < nruns) {
+    for (int i = 0; i < kMyRuns; ++i) {
+      const int r = wave + 4 * i;
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
-      if (krow[i]) {
 #pragma unroll
-        for (int b = 0; b < HT; ++b) {
-          const f32x4 qv = *reinterpret_cast<const f32x4*>(&qs[c16][16 * b + 4 * g]);  // head c16, this lane group's elements
+      for (int b = 0; b < HT; ++b) {
+        const f32x4 qv = *reinterpret_cast<const f32x4*>(&qs[c16][16 * b + 4 * g]);  // head c16, this lane group's elements
 #pragma unroll
-          for (int u = 0; u < 4; ++u) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[i][b][u], qv[u], s, 0, 0, 0);
-        }
+        for (int u = 0; u < 4; ++u) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[i][b][u], qv[u], s, 0, 0, 0);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int key = first + 16 * r + 4 * g + u;
-        s[u] = krow[i] && key >= base && key <= last ? s[u] * scale : -INFINITY;
+        const int key = now.first + 16 * r + 4 * g + u;
+        s[u] = kthere[i] && key >= now.base && key <= now.last ? s[u] * scale : -INFINITY;
       }
-      *reinterpret_cast<f32x4*>(&sc[c16][16 * r + 4 * g]) = s;
+      if (r < kRuns) *reinterpret_cast<f32x4*>(&sc[c16][16 * r + 4 * g]) = s;
     }
-  }
-#pragma unroll
-  for (int r = kEarly; r < kRuns; ++r) ask_values(r);
-  __syncthreads();
+    if (ahead) ask_keys(next);  // into the registers that the scores have just left
+    __syncthreads();
 
-  // Softmax of the span, 16 threads a head: thread t of them takes the keys t, t + 16, ... of the runs.
-  {
-    const int h = tid >> 4, t = tid & 15;
-    float m = -INFINITY;
-    for (int j = t; j < 16 * nruns; j += 16) m = fmaxf(m, sc[h][j]);
+    // Softmax of the span, 16 threads a head: thread t of them takes the keys t, t + 16, ... of the runs.
+    {
+      const int h = tid >> 4, t = tid & 15;
+      float p[kRuns], m = -INFINITY;
 #pragma unroll
-    for (int x = 8; x > 0; x >>= 1) m = fmaxf(m, __shfl_xor(m, x, 16));
-    const float m_use = m == -INFINITY ? 0.f : m;
-    float l = 0.f;
-    for (int j = t; j < 16 * nruns; j += 16) {
-      const float p = expf(sc[h][j] - m_use);  // 0 for the keys outside the span
-      sc[h][j] = p;
-      l += p;
+      for (int j = 0; j < kRuns; ++j) m = fmaxf(m, p[j] = sc[h][t + 16 * j]);
+#pragma unroll
+      for (int x = 8; x > 0; x >>= 1) m = fmaxf(m, __shfl_xor(m, x, 16));
+      const float m_use = m == -INFINITY ? 0.f : m;
+      float l = 0.f;
+#pragma unroll
+      for (int j = 0; j < kRuns; ++j) {
+        p[j] = expf(p[j] - m_use);  // 0 for the keys outside the span
+        sc[h][t + 16 * j] = p[j];
+        l += p[j];
+      }
+#pragma unroll
+      for (int x = 8; x > 0; x >>= 1) l += __shfl_xor(l, x, 16);
+      if (t == 0) ml[h][0] = m, ml[h][1] = l;
     }
-#pragma unroll
-    for (int x = 8; x > 0; x >>= 1) l += __shfl_xor(l, x, 16);
-    if (t == 0) ml[h][0] = m, ml[h][1] = l;
-  }
-  __syncthreads();
+    __syncthreads();
 
-  // Output: rows are 16 elements of the head, columns the heads; the keys of the span run by run.
-  f32x4 acc[kMyTiles];
+    // Output: rows are 16 elements of the head, columns the heads; the keys of the span run by run.
+    f32x4 acc[kMyTiles];
 #pragma unroll
-  for (int t = 0; t < kMyTiles; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < kMyTiles; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int r = 0; r < kRuns; ++r) {
-    if (r < nruns && vthere[r]) {
+    for (int r = 0; r < kRuns; ++r) {
       const f32x4 p = *reinterpret_cast<const f32x4*>(&sc[c16][16 * r + 4 * g]);
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int t = 0; t < kMyTiles; ++t) {
+        if (HT % 4 != 0 && wave + 4 * t >= HT) continue;
+        const f32x4 v = vthere[r] ? vreg[r][t] : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < kMyTiles; ++t)
-          if (wave + 4 * t < HT) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vreg[r][t][u], p[u], acc[t], 0, 0, 0);
+        for (int u = 0; u < 4; ++u) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(v[u], p[u], acc[t], 0, 0, 0);
+      }
     }
-  }
-  if (c16 >= nheads) return;
-  const int h = head0 + c16;
-  const float m = ml[c16][0], l = ml[c16][1];
+    if (ahead) ask_values(next);
+    if (c16 < nheads) {
+      const int h = head0 + c16;
+      const float m = ml[c16][0], l = ml[c16][1];
 #pragma unroll
-  for (int t = 0; t < kMyTiles; ++t) {
-    if (wave + 4 * t >= HT) continue;
-    const int d = 16 * (wave + 4 * t) + 4 * g;  // this lane's four elements
-    if (part) {  // [token of the list][head][span][hd + 2]: unnormalised output, max, sum
-      float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + h) * gridDim.z + blockIdx.z) * (hd + 2);
-      *reinterpret_cast<f32x2*>(dst + d) = f32x2{acc[t][0], acc[t][1]};  // rows of hd + 2 floats start on 8 bytes
-      *reinterpret_cast<f32x2*>(dst + d + 2) = f32x2{acc[t][2], acc[t][3]};
-      if (d == 0) dst[hd] = m, dst[hd + 1] = l;
-    } else {
-      f32x4 o;
+      for (int t = 0; t < kMyTiles; ++t) {
+        if (HT % 4 != 0 && wave + 4 * t >= HT) continue;
+        const int d = 16 * (wave + 4 * t) + 4 * g;  // this lane's four elements
+        if (part) {  // [token of the list][head][span][hd + 2]: unnormalised output, max, sum
+          float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + h) * spans + span) * (hd + 2);
+          *reinterpret_cast<f32x2*>(dst + d) = f32x2{acc[t][0], acc[t][1]};  // rows of hd + 2 floats start on 8 bytes
+          *reinterpret_cast<f32x2*>(dst + d + 2) = f32x2{acc[t][2], acc[t][3]};
+          if (d == 0) dst[hd] = m, dst[hd + 1] = l;
+        } else {
+          f32x4 o;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) o[u] = l > 0.f ? acc[t][u] / l : 0.f;
-      *reinterpret_cast<f32x4*>(out + (static_cast<size_t>(n) * nq + h) * hd + d) = o;
+          for (int u = 0; u < 4; ++u) o[u] = l > 0.f ? acc[t][u] / l : 0.f;
+          *reinterpret_cast<f32x4*>(out + (static_cast<size_t>(n) * nq + h) * hd + d) = o;
+        }
+      }
     }
-  }
+    now = next;
+    if (ahead) __syncthreads();  // the scores and the sums are read; the next span may write them
+  };
+  int span = span0;
+  for (; span + 1 < span_end; ++span) take(span, std::true_type{});
+  take(span, std::false_type{});
 }
 
 // out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the spans that the token has, in their order.
@@ -382,11 +402,14 @@ extern "C" int pyre_attn_generic(const void* q, void* out, int q_dt, const void*
     // the query heads of a key/value head together: the span's keys and values are read once for all of them
     const int per_kv = (nq / nkv + kSingleHeads - 1) / kSingleHeads;
     PYRE_REQUIRE(nkv * per_kv <= 65535, "attn_generic: too many heads");
+    // spans a block: as many as leave two blocks a compute unit (the blocks that fit there at once), up to eight
+    int per_block = static_cast<int>(static_cast<long>(n) * nkv * per_kv * spans / (2L * compute_units()));
+    per_block = max(1, min(8, per_block));
 #define PYRE_SINGLE_AS(HT, ALIGNED)                                                                                  \
-  hipLaunchKernelGGL((attn_single_f32_kernel<HT, ALIGNED>), dim3(n, nkv * per_kv, spans), dim3(kThreads), 0, stream, \
-                     static_cast<const float*>(q), static_cast<const float*>(k_cache),                               \
+  hipLaunchKernelGGL((attn_single_f32_kernel<HT, ALIGNED>), dim3(n, nkv * per_kv, (spans + per_block - 1) / per_block), \
+                     dim3(kThreads), 0, stream, static_cast<const float*>(q), static_cast<const float*>(k_cache),     \
                      static_cast<const float*>(v_cache), static_cast<float*>(out), tokens, positions, seq_of_token,   \
-                     block_table, table_stride, nq, nkv, page_size, scale, window, scratch)
+                     block_table, table_stride, nq, nkv, page_size, scale, window, scratch, spans, per_block)
 #define PYRE_SINGLE(HT)                     \
   case HT:                                  \
     if (window > 0) PYRE_SINGLE_AS(HT, false); \
