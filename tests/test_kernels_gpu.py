@@ -705,7 +705,7 @@ def test_attention_finds_a_far_key(kernel):
     the output is its value."""
     ops = _ops()
     nq, nkv, hd, page = 8, 2, 64, 16
-    dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
+    dt = torch.float32 if kernel in ("generic32", "plain32", "prefill32") else torch.bfloat16
     ctx_lens, q_lens = [900], [1 if not kernel.startswith("prefill") else 34]
     for target in (0, 16 * 20, 16 * 20 + 15, 899 - 34):
         q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=9)
@@ -738,7 +738,7 @@ def test_attention_at_a_windows_edge(kernel):
     be seen at all (an off-by-one at the window's edge would return its value instead)."""
     ops = _ops()
     nq, nkv, hd, page, window = 8, 2, 64, 16, 100
-    dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
+    dt = torch.float32 if kernel in ("generic32", "plain32", "prefill32") else torch.bfloat16
     ql = 34 if kernel.startswith("prefill") else 1
     ctx_lens, q_lens = [700], [ql]
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=13)
@@ -776,7 +776,7 @@ def test_attention_at_a_windows_edge(kernel):
         assert not torch.allclose(out2.double().cpu(), want.expand(n, nq, hd), atol=0.2)
 
 
-@pytest.mark.parametrize("kernel", ["generic32", "generic16", "decode", "decode256", "prefill", "prefill256", "prefill32"])
+@pytest.mark.parametrize("kernel", ["generic32", "plain32", "generic16", "decode", "decode256", "prefill", "prefill256", "prefill32"])
 @pytest.mark.parametrize("ctx_len", [700, 689, 655])
 def test_attention_ignores_what_a_page_held_before(kernel, ctx_len):
     """A request's last page is only partly its own: the slots past its last key still hold what
@@ -792,7 +792,7 @@ def test_attention_ignores_what_a_page_held_before(kernel, ctx_len):
 
     big = kernel.endswith("256")
     nq, nkv, hd, page = (4, 2, 256, 16) if big else (8, 2, 64, 16)
-    dt = torch.float32 if kernel in ("generic32", "prefill32") else torch.bfloat16
+    dt = torch.float32 if kernel in ("generic32", "plain32", "prefill32") else torch.bfloat16
     ql = 34 if kernel.startswith("prefill") else 1
     ctx_lens, q_lens = [ctx_len, 40], [ql, min(ql, 3)]
     q, kc, vc, table, pos, seq_of, dense, qs = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, dt, seed=17)
@@ -827,8 +827,9 @@ def test_attention_ignores_what_a_page_held_before(kernel, ctx_len):
     out = torch.zeros_like(q)
     n = q.shape[0]
     tiles = [(0, 32), (32, 2), (34, 3)]
-    if kernel.startswith("generic"):
-        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, 0)
+    if kernel.startswith("generic") or kernel == "plain32":   # float32: on the matrix cores, or one block per head
+        ops.attn_generic(q, out, kc, vc, pos, seq_of, table, n, nq, nkv, hd, page, scale, 0,
+                         matrix_cores=kernel != "plain32")
     elif kernel.startswith("decode"):
         decode_attention(ops, q, out, kc, vc, [0, 1], pos, seq_of, table, nq, nkv, hd, page, scale)
     elif kernel == "prefill32":
