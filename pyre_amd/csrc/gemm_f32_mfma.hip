@@ -162,6 +162,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_f32_mfma_kernel(
 // wave, not memory, sets the pace (a slot of 4 KB in about 0.6 us), and with 64 rows the matrix
 // cores' float32 rate does; a small ring lets several blocks share a compute unit.
 constexpr int kStreamMaxRows = 64;
+constexpr int kMaxDevices = 64;
 constexpr int kSlotK = 32;
 
 __device__ inline void load_to_lds(const void* src, unsigned lds_addr) {
@@ -173,19 +174,29 @@ __device__ inline void wait_loads() {
 }
 __device__ __attribute__((aligned(16))) const unsigned kZeroPiece[4] = {0u, 0u, 0u, 0u};
 
-template <int R, int XR>
-__global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
+// NW = 4 (steps of 17 to 64 rows): four such waves, one on each SIMD, share the step's rows: a slot
+// holds the four waves' weights and one copy of the rows, of which every wave loads a quarter, and
+// a barrier per slot tells a wave that the others' quarters are there. A wave alone reads the rows
+// from L2 once per 32 output columns, more bytes than its weights at 64 rows, and has LDS for one
+// slot on its way; four waves together have it for four (the ring is dynamic shared memory then).
+extern __shared__ __attribute__((aligned(1024))) unsigned char stream_ring[];
+
+template <int R, int XR, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_f32_stream_kernel(
     const float* __restrict__ A, size_t lda, const float* __restrict__ W, size_t ldw,
     const void* __restrict__ bias, int bias_dt, float* __restrict__ out, size_t ldo, size_t part_stride, int M,
     int N, int K, int kper) {
-  constexpr int XL = XR / 8;                    // load instructions for a slot's rows of A
+  static_assert(NW == 1 || (NW == 4 && XR >= 32), "four waves share 32 or 64 rows");
+  constexpr int XL = XR / 8 / NW;               // this wave's load instructions for a slot's rows of A
   constexpr int MT = XR > 32 ? 2 : 1;           // tiles of 32 rows of A
-  constexpr int kSlotBytes = 4096 + XR * 128;
-  constexpr int L = 4 + XL;                     // load instructions per slot
+  constexpr int kSlotBytes = 4096 * NW + XR * 128;
+  constexpr int L = 4 + XL;                     // a wave's load instructions per slot
   static_assert(L * (R - 2) <= 63, "the wait counter holds 63 loads");
-  __shared__ __attribute__((aligned(1024))) unsigned char ring[R * kSlotBytes];
-  const int lane = threadIdx.x, half = lane >> 5, c = lane & 31;
-  const int n0 = blockIdx.x * 32;
+  __shared__ __attribute__((aligned(1024))) unsigned char own_ring[NW == 1 ? R * kSlotBytes : 16];
+  unsigned char* const ring = NW == 1 ? own_ring : stream_ring;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, half = lane >> 5, c = lane & 31;
+  const int n0 = (blockIdx.x * NW + wave) * 32;
   const int kbeg = blockIdx.z * kper;
   K = min(K, kbeg + kper);  // this part's end
   out += blockIdx.z * part_stride;
@@ -209,7 +220,7 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
   bool xrow[XL];
 #pragma unroll
   for (int i = 0; i < XL; ++i) {
-    const int r = 8 * i + lr;
+    const int r = 8 * (NW * i + wave) + lr;  // of the slot's instructions for A, this wave's are wave, NW + wave, ...
     xk[i] = 4 * (lp ^ ((r >> 1) & 7));
     xrow[i] = r < M;
     xsrc[i] = A + static_cast<size_t>(xrow[i] ? r : 0) * lda + kbeg + xk[i];
@@ -223,9 +234,17 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
     fill = fill + 1 == R ? 0 : fill + 1;
     const int k0 = kSlotK * j, left = j < slots ? K - kbeg - k0 : 0;  // k of this part from the slot's start on
 #pragma unroll
-    for (int i = 0; i < 4; ++i) load_to_lds(wk[i] < left ? wsrc[i] + k0 : zero, dst + 1024 * i);
+    for (int i = 0; i < 4; ++i) load_to_lds(wk[i] < left ? wsrc[i] + k0 : zero, dst + 4096 * wave + 1024 * i);
 #pragma unroll
-    for (int i = 0; i < XL; ++i) load_to_lds(xrow[i] && xk[i] < left ? xsrc[i] + k0 : zero, dst + 4096 + 1024 * i);
+    for (int i = 0; i < XL; ++i)
+      load_to_lds(xrow[i] && xk[i] < left ? xsrc[i] + k0 : zero, dst + 4096 * NW + 1024 * (NW * i + wave));
+  };
+  // The slot that this wave's loads have just filled is whole when the other waves' are there too.
+  auto slot_whole = [&]() {
+    if (NW > 1) {
+      asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // and what this wave read of the slot that is filled next
+      __syncthreads();
+    }
   };
 
   if constexpr (XR <= 16) {
@@ -300,8 +319,8 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
   for (int u = 0; u < MT; ++u)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[u][i] = 0.f;
-  const unsigned char* wpiece = ring + c * 128;
-  const unsigned char* xpiece = ring + 4096 + c * 128;
+  const unsigned char* wpiece = ring + 4096 * wave + c * 128;
+  const unsigned char* xpiece = ring + 4096 * NW + c * 128;
   const int swz = (c >> 1) & 7;  // rows c and 32 + c exchange their pieces alike
   int at = 0;  // ring position of the next slot to read
   auto read = [&](f32x4 (&a)[2][2], f32x4 (&b)[MT][2][2]) {
@@ -325,10 +344,12 @@ __global__ __launch_bounds__(64) void gemm_f32_stream_kernel(
   for (int j = 0; j < R - 1; ++j) issue(j);
   f32x4 a[2][2], b[MT][2][2], an[2][2], bn[MT][2][2];
   wait_loads<L * (R - 2)>();  // loads finish in the order of issue: slot 0 is there
+  slot_whole();
   read(a, b);
   for (int j = 0; j < slots; ++j) {
-    issue(j + R - 1);            // into the position of slot j - 1, read a turn ago
+    issue(j + R - 1);            // into the position of slot j - 1, read a turn ago (by every wave: the barrier since)
     wait_loads<L * (R - 2)>();   // slot j + 1 is there
+    slot_whole();
     read(an, bn);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -395,14 +416,34 @@ extern "C" int pyre_gemm_f32(const float* A, long lda, const float* W, long ldw,
   if (M <= kStreamMaxRows && vec_ok && K % 4 == 0) {  // a decode step's rows: the weights as a stream
     const dim3 grid((N + 31) / 32, 1, ksplit);
 #define PYRE_STREAM(R, XR)                                                                                         \
-  hipLaunchKernelGGL((gemm_f32_stream_kernel<R, XR>), grid, dim3(64), 0, stream, A, static_cast<size_t>(lda), W,    \
+  hipLaunchKernelGGL((gemm_f32_stream_kernel<R, XR, 1>), grid, dim3(64), 0, stream, A, static_cast<size_t>(lda), W, \
                      static_cast<size_t>(ldw), bias, bias_dt, out, static_cast<size_t>(ldo),                       \
                      static_cast<size_t>(part_stride), M, N, K, kper)
+// four waves a block, the ring in dynamic shared memory (asked for once per device and kernel)
+#define PYRE_STREAM4(R, XR)                                                                                        \
+  do {                                                                                                             \
+    constexpr int kBytes = (R) * (4096 * 4 + (XR) * 128);                                                          \
+    static bool asked[kMaxDevices] = {};                                                                           \
+    int dev = 0;                                                                                                   \
+    PYRE_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, "gemm_f32: no device");         \
+    if (!asked[dev]) {                                                                                             \
+      PYRE_REQUIRE(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_f32_stream_kernel<R, XR, 4>),           \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBytes) == hipSuccess,          \
+                   "gemm_f32: %d bytes of LDS a block are refused", kBytes);                                       \
+      asked[dev] = true;                                                                                           \
+    }                                                                                                              \
+    hipLaunchKernelGGL((gemm_f32_stream_kernel<R, XR, 4>), dim3((N + 127) / 128, 1, ksplit), dim3(256), kBytes,    \
+                       stream, A, static_cast<size_t>(lda), W, static_cast<size_t>(ldw), bias, bias_dt, out,       \
+                       static_cast<size_t>(ldo), static_cast<size_t>(part_stride), M, N, K, kper);                 \
+  } while (0)
     if (M <= 8) PYRE_STREAM(4, 8);
     else if (M <= 16) PYRE_STREAM(4, 16);
+    else if (M <= 32 && N >= 128) PYRE_STREAM4(7, 32);
     else if (M <= 32) PYRE_STREAM(4, 32);
+    else if (N >= 128) PYRE_STREAM4(6, 64);
     else PYRE_STREAM(3, 64);
 #undef PYRE_STREAM
+#undef PYRE_STREAM4
   } else if (M <= 32) {  // four waves side by side along n
     const dim3 grid((N + 127) / 128, (M + 31) / 32, ksplit);
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<4, 1, 1, 1>), grid, dim3(256), 0, stream, A, static_cast<size_t>(lda), W,
