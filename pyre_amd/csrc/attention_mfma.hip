@@ -31,6 +31,7 @@
 
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 using namespace pyre;
 
@@ -312,8 +313,36 @@ __device__ inline float load_through(const float* base, int elem) {
   return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_of(base), 4 * elem, 0, kThrough));
 }
 
+
+// A barrier that waits for this wave's LDS traffic only. __syncthreads() also waits for
+// every global load in flight, which would put the latency of the next chunks' loads
+// into each half-step.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// What the kernel needs to finish the step's q/k/v product itself (FUSED): the product's partial
+// sums [n_partials][rows][(nq + 2 nkv) HD] float32 with its bias, the rotary tables, and where each
+// token's key and value go. Every block sums, biases and rotates the queries of its heads into LDS
+// (the arithmetic of rope_kv_write, so the same bits); of the waves that attend for a token and
+// key/value head, the one whose chunks hold the token's own position first writes its rotated key
+// and its value into the cache, zeroes the values behind it in the page as rope_kv_write does, waits
+// for the stores and then loads its chunks: no other wave reads that position. A step of single
+// tokens then needs no kernel between the product and the attention.
+struct RopeIn {
+  const float* qkv;
+  int n_partials;
+  long partial_stride;
+  const void* bias;
+  int bias_dt;
+  const float* cos_t;
+  const float* sin_t;
+  const int* slots;  // the cache slot of each token, -1: not stored
+  int n_rows;        // tokens in the step (rows of the product)
+  int write_kv;      // this layer keeps its keys and values
+};
+
+// k_cache and v_cache carry no __restrict__: the FUSED form writes through them what it reads later.
 #define PYRE_DECODE_WORK_PARAMS                                                                                   \
-  const bf16 *__restrict__ q, const bf16 *__restrict__ k_cache, const bf16 *__restrict__ v_cache,                 \
+  const bf16 *__restrict__ q, bf16 *k_cache, bf16 *v_cache,                                                       \
       const int4 *__restrict__ work, const int *__restrict__ positions, const int *__restrict__ seq_of_token,     \
       const int *__restrict__ block_table, int table_stride, float *__restrict__ part_acc,                        \
       float *__restrict__ part_ml, int *__restrict__ counters, bf16 *__restrict__ out, int nq, int nkv,           \
@@ -322,8 +351,8 @@ __device__ inline float load_through(const float* base, int elem) {
   q, k_cache, v_cache, work, positions, seq_of_token, block_table, table_stride, part_acc, part_ml, counters, out, \
       nq, nkv, page_size, scale_log2, window
 
-template <int HD, bool STREAM_V>
-__device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) {
+template <int HD, bool STREAM_V, bool FUSED>
+__device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS, const RopeIn& rope) {
   const int4 head_of_list = work[0];
   if (static_cast<int>(blockIdx.y) >= head_of_list.x) return;
   const int4 item = work[1 + blockIdx.y];
@@ -342,33 +371,136 @@ __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) 
   KV kv{k_cache, v_cache, block_table + static_cast<size_t>(seq_of_token[tok]) * table_stride, nkv, kvh, page_size};
   Bounds<1> bd{{lo}, {pos}};
 
-  bf16x8 qr[1][HD / 32];
-#pragma unroll
-  for (int c = 0; c < HD / 32; ++c)
-    qr[0][c] = r < nheads ? load_b128(q + (static_cast<size_t>(tok) * nq + head0 + r) * HD + 32 * c + 8 * g) : zero_b128();
+  const int first = lo / kChunk, last = pos / kChunk;
+  const int begin = first + (4 * b + wave) * per, end = min(last + 1, begin + per);  // may be empty
 
+  static_assert(!FUSED || HD <= 128, "the form that finishes the product itself: heads of up to 128 elements");
+  bf16x8 qr[1][HD / 32];
+  if constexpr (!FUSED) {
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c)
+      qr[0][c] = r < nheads ? load_b128(q + (static_cast<size_t>(tok) * nq + head0 + r) * HD + 32 * c + 8 * g) : zero_b128();
+  }
   f32x4 o[HD / 16][1];
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) o[dt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m[1] = {-INFINITY}, l[1] = {0.f};
-
-  const int first = lo / kChunk, last = pos / kChunk;
-  const int begin = first + (4 * b + wave) * per, end = min(last + 1, begin + per);  // may be empty
   if constexpr (HD <= 128) {
-    // Two register sets: while one chunk is multiplied the next one's loads are in flight.
+    // Two register sets: while one chunk is multiplied the next one's loads are in flight; the wave
+    // starts with both on their way.
     ChunkRegs<HD> ra, rb;
     // No entry beyond those of the chunks up to `last` is read.
     TableWindow tw{kv.table, min(table_stride, (last * kChunk + 16) / page_size + 1), 0, -1};
-    if (begin < end) {
-      tw.fill(begin * kChunk / page_size);
+    if (begin < end) tw.fill(begin * kChunk / page_size);
+    // FUSED: of the waves that attend for a token and key/value head (the first group of query heads
+    // only), the one whose chunks hold the token's own position writes its key and value; it loads
+    // that chunk only when its stores have arrived.
+    const bool may_write = FUSED && qt == 0 && rope.write_kv && begin <= last && last < end;
+    bool writes = false;
+    auto arrived = [&](int c) {
+      if (FUSED && writes && c == last) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    };
+    const bool ask_a = begin < end && !(may_write && begin == last);
+    const bool ask_b = begin + 1 < end && !(may_write && begin + 1 == last);
+    if constexpr (FUSED) {
+      constexpr int half = HD / 2;
+      const int width = (nq + 2 * nkv) * HD;
+      const float* row = rope.qkv + static_cast<size_t>(tok) * width;
+      auto value4 = [&](int col) {  // the product's sum with its bias, four columns from `col` (a multiple of 4) on
+        float4 v = sum_partials4<float>(row + col, static_cast<size_t>(rope.partial_stride), rope.n_partials);
+        if (rope.bias)
+          v = add4(v, rope.bias_dt == kF32 ? Vec4<float>::load(static_cast<const float*>(rope.bias) + col)
+                                           : Vec4<bf16>::load(static_cast<const bf16*>(rope.bias) + col));
+        return v;
+      };
+      // elements j..j+3 and half + j.. of the head at `base`: what is loaded, and the rotation of it
+      struct Pairs { float4 x1, x2, c4, s4; };
+      auto pairs_of = [&](int base, int j) {
+        const size_t t = static_cast<size_t>(pos) * half + j;
+        return Pairs{value4(base + j), value4(base + j + half), Vec4<float>::load(rope.cos_t + t), Vec4<float>::load(rope.sin_t + t)};
+      };
+      auto rotate = [&](const Pairs& p, float4& a4, float4& b4) {
+        rotate_pair(p.x1.x, p.x2.x, p.c4.x, p.s4.x, a4.x, b4.x);
+        rotate_pair(p.x1.y, p.x2.y, p.c4.y, p.s4.y, a4.y, b4.y);
+        rotate_pair(p.x1.z, p.x2.z, p.c4.z, p.s4.z, a4.z, b4.z);
+        rotate_pair(p.x1.w, p.x2.w, p.c4.w, p.s4.w, a4.w, b4.w);
+      };
+      // First everything this thread has to load of the product: four pairs of a query (thread it of the
+      // block: head it / (HD / 8)), and in the wave that may write, four pairs of the key (lanes
+      // 0 .. HD / 8 - 1) or four elements of the value (the next HD / 4 lanes). Then the chunks' loads, which
+      // queue behind them; then the arithmetic of rope_kv_write.
+      const int it = threadIdx.x;
+      const bool q_item = it < nheads * (HD / 8);
+      const bool key_lane = may_write && lane < HD / 8, value_lane = may_write && lane >= HD / 8 && lane < HD / 8 + HD / 4;
+      const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
+      Pairs qp{zero4, zero4, zero4, zero4}, kp = qp;
+      float4 vv = zero4;
+      if (q_item) qp = pairs_of((head0 + it / (HD / 8)) * HD, 4 * (it % (HD / 8)));
+      if (key_lane) kp = pairs_of((nq + kvh) * HD, 4 * lane);
+      if (value_lane) vv = value4((nq + nkv + kvh) * HD + 4 * (lane - HD / 8));
+      const int slot = may_write ? rope.slots[tok] : -1;
+      if (ask_a) load_chunk<HD, STREAM_V>(kv, tw, begin * kChunk, ra);
+      if (ask_b) load_chunk<HD, STREAM_V>(kv, tw, (begin + 1) * kChunk, rb);
+      // the queries of this block's heads, rounded to bfloat16 as rope_kv_write stores them
+      __shared__ __attribute__((aligned(16))) bf16 q_s[16][HD + 8];
+      static_assert(16 * (HD / 8) <= 256, "one item of the queries per thread");
+      if (q_item) {
+        float4 a4, b4;
+        rotate(qp, a4, b4);
+        const int h = it / (HD / 8), j = 4 * (it % (HD / 8));
+        Vec4<bf16>::store(&q_s[h][j], a4);
+        Vec4<bf16>::store(&q_s[h][j + half], b4);
+      }
+      lds_barrier();  // waits for LDS alone: the chunks' loads stay on their way
+#pragma unroll
+      for (int c = 0; c < HD / 32; ++c) qr[0][c] = r < nheads ? load_b128(&q_s[r][32 * c + 8 * g]) : zero_b128();
+      // the token's own key and value
+      writes = may_write && slot >= 0;
+      if (writes) {
+        const int page = slot / page_size, off = slot % page_size;
+        if (key_lane) {
+          float4 ka, kb;
+          rotate(kp, ka, kb);
+          bf16* dst = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * HD + 4 * lane;
+          Vec4<bf16>::store(dst, ka);
+          Vec4<bf16>::store(dst + half, kb);
+        } else if (value_lane) {
+          bf16* vrow = v_cache + ((static_cast<size_t>(page) * nkv + kvh) * HD + 4 * (lane - HD / 8)) * page_size;
+          const float vals[4] = {vv.x, vv.y, vv.z, vv.w};
+          const bool ends = ends_its_page_run(rope.slots, tok, rope.n_rows, slot, page_size);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            bf16* one = vrow + u * static_cast<size_t>(page_size);
+            one[off] = from_float<bf16>(vals[u]);
+            // the step's last token of a page leaves nothing of the page's previous owner behind it
+            if (ends) zero_tail(one, off + 1, page_size);
+          }
+        }
+      }
+    } else {
+      if (ask_a) load_chunk<HD, STREAM_V>(kv, tw, begin * kChunk, ra);
+      if (ask_b) load_chunk<HD, STREAM_V>(kv, tw, (begin + 1) * kChunk, rb);
+    }
+    if (begin < end && !ask_a) {
+      arrived(begin);
       load_chunk<HD, STREAM_V>(kv, tw, begin * kChunk, ra);
     }
+    if (begin + 1 < end && !ask_b) {
+      arrived(begin + 1);
+      load_chunk<HD, STREAM_V>(kv, tw, (begin + 1) * kChunk, rb);
+    }
     for (int c = begin; c < end; c += 2) {
-      if (c + 1 < end) load_chunk<HD, STREAM_V>(kv, tw, (c + 1) * kChunk, rb);
       attend_regs<HD, 1>(ra, c * kChunk, c == first || c == last, bd, scale_log2, qr, o, m, l);
+      if (c + 2 < end) {
+        arrived(c + 2);
+        load_chunk<HD, STREAM_V>(kv, tw, (c + 2) * kChunk, ra);
+      }
       if (c + 1 < end) {
-        if (c + 2 < end) load_chunk<HD, STREAM_V>(kv, tw, (c + 2) * kChunk, ra);
         attend_regs<HD, 1>(rb, (c + 1) * kChunk, c + 1 == first || c + 1 == last, bd, scale_log2, qr, o, m, l);
+        if (c + 3 < end) {
+          arrived(c + 3);
+          load_chunk<HD, STREAM_V>(kv, tw, (c + 3) * kChunk, rb);
+        }
       }
     }
   } else {
@@ -474,11 +606,21 @@ __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS) 
 template <int HD, bool STREAM_V>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_decode_work_alone_kernel(
     PYRE_DECODE_WORK_PARAMS) {
-  attn_decode_work_block<HD, STREAM_V>(PYRE_DECODE_WORK_ARGS);
+  attn_decode_work_block<HD, STREAM_V, false>(PYRE_DECODE_WORK_ARGS, RopeIn{});
 }
 template <int HD, bool STREAM_V>
 __global__ __launch_bounds__(256, 2) void attn_decode_work_kernel(PYRE_DECODE_WORK_PARAMS) {
-  attn_decode_work_block<HD, STREAM_V>(PYRE_DECODE_WORK_ARGS);
+  attn_decode_work_block<HD, STREAM_V, false>(PYRE_DECODE_WORK_ARGS, RopeIn{});
+}
+// The same two forms, finishing the q/k/v product themselves (heads of up to 128 elements).
+template <int HD, bool STREAM_V>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_decode_work_rope_alone_kernel(
+    PYRE_DECODE_WORK_PARAMS, RopeIn rope) {
+  attn_decode_work_block<HD, STREAM_V, true>(PYRE_DECODE_WORK_ARGS, rope);
+}
+template <int HD, bool STREAM_V>
+__global__ __launch_bounds__(256, 2) void attn_decode_work_rope_kernel(PYRE_DECODE_WORK_PARAMS, RopeIn rope) {
+  attn_decode_work_block<HD, STREAM_V, true>(PYRE_DECODE_WORK_ARGS, rope);
 }
 #undef PYRE_DECODE_WORK_PARAMS
 #undef PYRE_DECODE_WORK_ARGS
@@ -587,10 +729,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 64;
 
-// A barrier that waits for this wave's LDS traffic only. __syncthreads() also waits for
-// every global load in flight, which would put the latency of the next chunks' loads
-// into each half-step.
-__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // 16 bytes per lane from global memory straight into LDS: lane x's piece lands at
 // lds_addr + 16 x. The compiler does not know of these loads; whoever reads the bytes
@@ -971,12 +1109,12 @@ extern "C" int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv) {
          nq % nkv == 0;
 }
 
-extern "C" int pyre_attn_decode_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
-                                          const int* work, int capacity, const int* positions,
-                                          const int* seq_of_token, const int* block_table, int table_stride,
-                                          float* part_acc, float* part_ml, int* counters, int alone, int nq,
-                                          int nkv, int hd, int page_size, float scale, int window,
-                                          hipStream_t stream) {
+namespace {
+
+int launch_decode_work(const void* q, void* out, void* k_cache, void* v_cache, const int* work, int capacity,
+                       const int* positions, const int* seq_of_token, const int* block_table, int table_stride,
+                       float* part_acc, float* part_ml, int* counters, int alone, int nq, int nkv, int hd,
+                       int page_size, float scale, int window, const RopeIn* rope, hipStream_t stream) {
   PYRE_REQUIRE(pyre_attn_mfma_supports(hd, page_size, nq, nkv),
                "attn_decode_work_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
@@ -987,22 +1125,71 @@ extern "C" int pyre_attn_decode_work_bf16(const void* q, void* out, const void* 
   PYRE_REQUIRE(capacity <= 65535, "attn_decode_work_bf16: a list of %d blocks is too long for one launch", capacity);
   const dim3 grid(nkv * qtiles, capacity);
   const float scale_log2 = scale * kLog2e;
+#define PYRE_DECODE_LAUNCH_ARGS                                                                                    \
+  static_cast<const bf16*>(q), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),                          \
+      reinterpret_cast<const int4*>(work), positions, seq_of_token, block_table, table_stride, part_acc, part_ml, \
+      counters, static_cast<bf16*>(out), nq, nkv, page_size, scale_log2, window
   const int rc = dispatch_head(hd, [&](auto HDc) {
     constexpr int HD = decltype(HDc)::value;
     auto launch = [&](auto stream_v) {
       constexpr bool SV = decltype(stream_v)::value;
-      auto kernel = alone ? attn_decode_work_alone_kernel<HD, SV> : attn_decode_work_kernel<HD, SV>;
-      hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, static_cast<const bf16*>(q),
-                         static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache),
-                         reinterpret_cast<const int4*>(work), positions, seq_of_token, block_table, table_stride,
-                         part_acc, part_ml, counters, static_cast<bf16*>(out), nq, nkv, page_size, scale_log2,
-                         window);
+      if (rope) {
+        if constexpr (HD <= 128) {
+          auto kernel = alone ? attn_decode_work_rope_alone_kernel<HD, SV> : attn_decode_work_rope_kernel<HD, SV>;
+          hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, PYRE_DECODE_LAUNCH_ARGS, *rope);
+        }
+      } else {
+        auto kernel = alone ? attn_decode_work_alone_kernel<HD, SV> : attn_decode_work_kernel<HD, SV>;
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, PYRE_DECODE_LAUNCH_ARGS);
+      }
     };
     if (page_size <= 32) launch(std::true_type{});
     else launch(std::false_type{});
   });
+#undef PYRE_DECODE_LAUNCH_ARGS
   PYRE_REQUIRE(rc == 0, "attn_decode_work_bf16: no kernel for head_dim %d", hd);
   return check_launch("attn_decode_work_bf16");
+}
+
+}  // namespace
+
+extern "C" int pyre_attn_decode_work_bf16(const void* q, void* out, const void* k_cache, const void* v_cache,
+                                          const int* work, int capacity, const int* positions,
+                                          const int* seq_of_token, const int* block_table, int table_stride,
+                                          float* part_acc, float* part_ml, int* counters, int alone, int nq,
+                                          int nkv, int hd, int page_size, float scale, int window,
+                                          hipStream_t stream) {
+  return launch_decode_work(q, out, const_cast<void*>(k_cache), const_cast<void*>(v_cache), work, capacity, positions,
+                            seq_of_token, block_table, table_stride, part_acc, part_ml, counters, alone, nq, nkv, hd,
+                            page_size, scale, window, nullptr, stream);
+}
+
+extern "C" int pyre_attn_decode_work_rope_supports(int hd, int page_size, int nq, int nkv, long partial_stride) {
+  // one group of query heads per key/value head: no other block reads the position that a block writes
+  return pyre_attn_mfma_supports(hd, page_size, nq, nkv) && hd <= 128 && nq / nkv <= 16 && partial_stride % 4 == 0;
+}
+
+extern "C" int pyre_attn_decode_work_rope_bf16(const float* qkv, int n_partials, long partial_stride, const void* bias,
+                                               int bias_dt, const float* cos_t, const float* sin_t, const int* slots,
+                                               int n_rows, int write_kv, void* out, void* k_cache, void* v_cache,
+                                               const int* work, int capacity, const int* positions,
+                                               const int* seq_of_token, const int* block_table, int table_stride,
+                                               float* part_acc, float* part_ml, int* counters, int alone, int nq,
+                                               int nkv, int hd, int page_size, float scale, int window,
+                                               hipStream_t stream) {
+  PYRE_REQUIRE(pyre_attn_decode_work_rope_supports(hd, page_size, nq, nkv, partial_stride),
+               "attn_decode_work_rope_bf16: head_dim %d, page_size %d, heads %d/%d or partial sums %ld apart are not "
+               "supported", hd, page_size, nq, nkv, partial_stride);
+  PYRE_REQUIRE(qkv && n_partials >= 1 && cos_t && sin_t && n_rows > 0, "attn_decode_work_rope_bf16: no product or tables");
+  PYRE_REQUIRE(!bias || known_dtype(bias_dt), "attn_decode_work_rope_bf16: unknown bias dtype");
+  PYRE_REQUIRE(!write_kv || slots, "attn_decode_work_rope_bf16: keys and values to write, but no slots");
+  PYRE_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(sin_t) % 16 == 0 && (!bias || reinterpret_cast<uintptr_t>(bias) % 16 == 0),
+               "attn_decode_work_rope_bf16: the product, its bias and the tables must lie on 16 bytes");
+  const RopeIn rope{qkv, n_partials, partial_stride, bias, bias_dt, cos_t, sin_t, slots, n_rows, write_kv};
+  return launch_decode_work(nullptr, out, k_cache, v_cache, work, capacity, positions, seq_of_token, block_table,
+                            table_stride, part_acc, part_ml, counters, alone, nq, nkv, hd, page_size, scale, window,
+                            &rope, stream);
 }
 
 extern "C" int pyre_attn_prefill_bf16(const void* q, void* out, const void* k_cache,

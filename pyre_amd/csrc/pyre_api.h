@@ -134,6 +134,24 @@ int pyre_attn_decode_work_bf16(const void* q, void* out, const void* k_cache, co
                                float* part_acc, float* part_ml, int* counters, int alone, int nq, int nkv,
                                int hd, int page_size, float scale, int window, hipStream_t stream);
 
+// The same for a step of single tokens straight from the step's q/k/v product (float32 partial sums
+// [n_partials][n_rows][(nq + 2 nkv) hd], partial_stride elements apart, with its bias or null): every
+// block sums, biases and rotates its heads' queries itself, and for every token and key/value head one
+// wave writes the token's rotated key and its value into the cache (slots[token], -1: not stored;
+// write_kv 0: a layer that keeps none) and zeroes the values behind it in its page, all with the
+// arithmetic of pyre_rope_kv_write (the same bits in the cache and in the result), so that no kernel
+// runs between the product and the attention. Full-head rotation (cos_t, sin_t: [positions][hd / 2]),
+// heads of up to 128 elements, up to 16 query heads per key/value head.
+int pyre_attn_decode_work_rope_supports(int hd, int page_size, int nq, int nkv, long partial_stride);
+int pyre_attn_decode_work_rope_bf16(const float* qkv, int n_partials, long partial_stride, const void* bias,
+                                    int bias_dt, const float* cos_t, const float* sin_t, const int* slots,
+                                    int n_rows, int write_kv, void* out, void* k_cache, void* v_cache,
+                                    const int* work, int capacity, const int* positions, const int* seq_of_token,
+                                    const int* block_table, int table_stride, float* part_acc, float* part_ml,
+                                    int* counters, int alone, int nq, int nkv, int hd, int page_size, float scale,
+                                    int window, hipStream_t stream);
+
+
 // Prompt portions. tiles[i] = (first token in the flat batch, token count <= 32),
 // all tokens of a tile from one request at consecutive positions. Every wave reads the
 // cache directly (any head size that pyre_attn_mfma_supports takes).

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 
 class KernelError(RuntimeError):
@@ -35,6 +35,8 @@ _SIGNATURES = {
     "pyre_attn_prefill_f32": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_mfma_supports": [I, I, I, I],
     "pyre_attn_decode_work_bf16": [P, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
+    "pyre_attn_decode_work_rope_supports": [I, I, I, I, L],
+    "pyre_attn_decode_work_rope_bf16": [P, I, L, P, I, P, P, P, I, I, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_bf16": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "pyre_attn_prefill_waves": [I, I],
     "pyre_attn_prefill_work_bf16": [P, P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, P],

@@ -499,6 +499,47 @@ def attn_decode_work_bf16(q, out, k_cache, v_cache, work, capacity, positions, s
          nkv, hd, page_size, float(scale), int(window), _stream())
 
 
+@lru_cache(maxsize=4096)
+def attn_decode_work_rope_supports(hd: int, page_size: int, nq: int, nkv: int, partial_stride: int) -> bool:
+    from pyre_amd.hip.lib import lib
+
+    return bool(lib().pyre_attn_decode_work_rope_supports(hd, page_size, nq, nkv, partial_stride))
+
+
+def attn_decode_work_rope_bf16(qkv: Partials, cos, sin, slots, out, k_cache, v_cache, write_kv, work, capacity,
+                               positions, seq_of_token, block_table, part_acc, part_ml, counters, alone, nq, nkv, hd,
+                               page_size, scale, window=0) -> None:
+    """:func:`attn_decode_work_bf16` for a step of single tokens, straight from the step's q/k/v
+    product (float32 partial sums and bias): the kernel sums, biases and rotates the queries itself and
+    writes each token's rotated key and its value into the cache (``write_kv``) with the arithmetic
+    of :func:`rope_kv_write`, the same bits, so that no kernel runs between product and attention.
+    ``cos``/``sin``: float32 ``[positions, hd / 2]`` (full-head rotation)."""
+    _attn_common(out, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
+    _dev(qkv.data, cos, sin, slots, work, part_acc, part_ml, counters)
+    width = (nq + 2 * nkv) * hd
+    args = qkv._args(width)
+    if qkv.data.dtype != torch.float32:
+        raise KernelError("attn_decode_work_rope: float32 partial sums expected")
+    if not attn_decode_work_rope_supports(hd, page_size, nq, nkv, qkv.stride):
+        raise KernelError(f"attn_decode_work_rope: head_dim {hd}, page_size {page_size}, heads {nq}/{nkv} are not taken")
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.dim() != 2 or cos.shape[1] != hd // 2 \
+            or cos.shape != sin.shape:
+        raise KernelError("attn_decode_work_rope: float32 cos/sin tables [positions, hd / 2] needed")
+    _contig("cos", cos), _contig("sin", sin), _i32("slots", slots, qkv.rows), _i32("work", work, 4 * (1 + capacity))
+    items = nkv * -(-(nq // nkv) // 16)
+    if part_acc.dtype != torch.float32 or part_acc.numel() < capacity * items * 16 * hd:
+        raise KernelError("attn_decode_work: partial accumulators too small")
+    if part_ml.dtype != torch.float32 or part_ml.numel() < capacity * items * 32:
+        raise KernelError("attn_decode_work: partial max/sum buffer too small")
+    if counters.dtype != torch.int32 or counters.numel() < capacity * items:
+        raise KernelError("attn_decode_work: too few counters")
+    call("pyre_attn_decode_work_rope_bf16", args[0], args[2], args[3], args[4], args[5], cos.data_ptr(), sin.data_ptr(),
+         slots.data_ptr(), qkv.rows, int(bool(write_kv)), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         work.data_ptr(), capacity, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+         block_table.stride(0), part_acc.data_ptr(), part_ml.data_ptr(), counters.data_ptr(), int(bool(alone)), nq,
+         nkv, hd, page_size, float(scale), int(window), _stream())
+
+
 def attn_prefill_bf16(q, out, k_cache, v_cache, tiles, n_tiles, positions, seq_of_token, block_table,
                       nq, nkv, hd, page_size, scale, window=0) -> None:
     """Attention of prompt portions, every wave reading the cache directly; ``tiles`` is int32

@@ -140,10 +140,15 @@ class Attention(Mixer):
         q = ws.get("attn.q", (n, self.q_dim), ctx.dtype)
         cos, sin, rot = self.position.rotary(ctx.runtime)
         k_pages, v_pages = cache["k"], cache["v"]
+        o = ws.get("attn.o", (n, self.q_dim), ctx.dtype)
+        if fast.rope_in_attention(self, ctx, qkv, cache, rot):
+            # a step of single tokens: the attention kernel sums, biases and rotates the product's
+            # partial sums itself and writes the new keys and values (one kernel less a layer)
+            fast.attention(self, ctx, q, o, cache, rope=(qkv, cos, sin))
+            return self.out.forward(ctx, o, n)
         ops.rope_kv_write(qkv, q, k_pages if cache.writes else None, v_pages if cache.writes else None,
                           cos, sin, rot, ctx.positions, cache.slots, n, s.num_heads, s.num_kv_heads,
                           s.head_dim, cache.page_size)
-        o = ws.get("attn.o", (n, self.q_dim), ctx.dtype)
         if not fast.attention(self, ctx, q, o, cache):
             self._attend_plainly(ctx, q, o, cache)
         return self.out.forward(ctx, o, n)

@@ -216,7 +216,28 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
 PREFILL_MAX_LAUNCH = 65535
 
 
-def attention(mixer, ctx, q, o, cache) -> bool:
+def rope_in_attention(mixer, ctx, qkv, cache, rotary_dim: int) -> bool:
+    """Whether the step's attention kernel can finish the q/k/v product itself (sum of the partial
+    sums, bias, rotation, the cache write): a step of single tokens only, on the 16-bit path's decode
+    kernel, full-head rotation, heads of up to 128 elements. The kernel between product and attention
+    is then left out; the bits are the same. A function of the step's shape and the model's sizes."""
+    from pyre_amd.hip import ops
+
+    s = mixer.spec
+    hb = ctx.host
+    if ctx.dtype != torch.bfloat16 or cache["k"].dtype != torch.bfloat16 or qkv.data.dtype != torch.float32:
+        return False
+    if not ctx.runtime.options.get("mfma_attention", True) or not ctx.runtime.options.get("rope_in_attention", True):
+        return False
+    if rotary_dim != s.head_dim or len(hb.arrays["attention.prefill_tiles"]) or \
+            len(hb.arrays["attention.decode_tokens"]) != ctx.n_tokens:
+        return False
+    return ops.attn_decode_work_rope_supports(s.head_dim, cache.page_size, s.num_heads, s.num_kv_heads, qkv.stride)
+
+
+def attention(mixer, ctx, q, o, cache, rope=None) -> bool:
+    """``rope``: (the q/k/v product's partial sums, cos, sin) when :func:`rope_in_attention` said that
+    the decode kernel finishes the product; ``q`` is then not read."""
     from pyre_amd.hip import ops
     from pyre_amd.parts.attention_work import (decode_alone, decode_capacity, decode_items, prefill_items,
                                                 prefill_slots)
@@ -246,10 +267,18 @@ def attention(mixer, ctx, q, o, cache) -> bool:
         acc = ctx.workspace.get("attn.part_acc", (capacity, items, 16, s.head_dim), torch.float32)
         ml = ctx.workspace.get("attn.part_ml", (capacity, items, 16, 2), torch.float32)
         counters = ctx.workspace.get("attn.counters", (capacity, items), torch.int32, zeroed=True)
-        ops.attn_decode_work_bf16(q, o, k_pages, v_pages, ctx.arrays[mixer.decode_work_name], capacity, ctx.positions,
-                                  ctx.seq_of_token, cache.table, acc, ml, counters,
-                                  decode_alone(rows, s.num_heads, s.num_kv_heads, units), s.num_heads, s.num_kv_heads,
-                                  s.head_dim, cache.page_size, mixer.scale, cache.window)
+        alone = decode_alone(rows, s.num_heads, s.num_kv_heads, units)
+        if rope is not None:
+            qkv, cos, sin = rope
+            ops.attn_decode_work_rope_bf16(qkv, cos, sin, cache.slots, o, k_pages, v_pages, cache.writes,
+                                           ctx.arrays[mixer.decode_work_name], capacity, ctx.positions,
+                                           ctx.seq_of_token, cache.table, acc, ml, counters, alone, s.num_heads,
+                                           s.num_kv_heads, s.head_dim, cache.page_size, mixer.scale, cache.window)
+        else:
+            ops.attn_decode_work_bf16(q, o, k_pages, v_pages, ctx.arrays[mixer.decode_work_name], capacity,
+                                      ctx.positions, ctx.seq_of_token, cache.table, acc, ml, counters, alone,
+                                      s.num_heads, s.num_kv_heads, s.head_dim, cache.page_size, mixer.scale,
+                                      cache.window)
     if n_tiles and s.head_dim <= 128:
         work = hb.arrays[mixer.prefill_work_name]
         n_slots = prefill_slots(work)

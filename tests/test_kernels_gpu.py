@@ -480,6 +480,67 @@ def work_on_device(work, cap, fill=0):
     return i32(flat.tolist())
 
 
+@pytest.mark.parametrize("nq,nkv,hd,page", [(28, 4, 128, 16), (12, 2, 128, 64), (8, 2, 64, 16), (6, 3, 32, 32), (16, 1, 96, 48)])
+@pytest.mark.parametrize("ks,bias,window,size,alone", [(7, True, 0, None, True), (1, False, 0, 4, False), (3, True, 50, None, False)])
+def test_attn_decode_finishes_the_qkv_product_itself(nq, nkv, hd, page, ks, bias, window, size, alone):
+    """A step of single tokens: the decode kernel given the q/k/v product's partial sums (sum, bias,
+    rotation, the cache write and the zeroes behind the new value are its own work) against the
+    kernel that does these and the decode kernel after it: the same bits in the result and in both
+    caches. Requests of very different lengths, one of them not stored (no slot), pages that hold
+    NaN where nothing was written, contexts that end anywhere in a page."""
+    ops = _ops()
+    from pyre_amd.hip.ops import Partials
+    from pyre_amd.parts.attention_work import decode_alone, decode_capacity, decode_items, decode_work
+    from pyre_amd.parts.rotary import rotary_tables
+
+    ctx_lens = [1, 31, 32, 33, 700, 2049, 129, 5, 64]
+    q_lens = [1] * len(ctx_lens)
+    _, kc, vc, table, pos, seq_of, dense, _ = paged_case(ctx_lens, q_lens, nq, nkv, hd, page, torch.bfloat16, seed=9)
+    n, scale, width = len(ctx_lens), hd ** -0.5, (nq + 2 * nkv) * hd
+    tab = table.cpu()
+    slots = [int(tab[s, (c - 1) // page]) * page + (c - 1) % page for s, c in enumerate(ctx_lens)]
+    slots[3] = -1                                            # a token that is not stored
+    for s, c in enumerate(ctx_lens):                         # the last key's place and what follows it: not written yet
+        last = int(tab[s, (c - 1) // page])
+        kc[last, :, (c - 1) % page:, :] = float("nan")
+        vc[last, :, :, (c - 1) % page:] = float("nan")
+    if slots[3] < 0:                                         # its key is read all the same: leave it finite
+        last = int(tab[3, (ctx_lens[3] - 1) // page])
+        kc[last, :, (ctx_lens[3] - 1) % page, :] = 0.25
+        vc[last, :, :, (ctx_lens[3] - 1) % page:] = 0.5
+    parts = Partials(rnd(ks, n, width, seed=12, scale=0.7), rnd(width, seed=13) if bias else None)
+    cos, sin = (t.to(DEV).contiguous() for t in rotary_tables(hd, 1e4, max(ctx_lens) + 1))
+    slots_d = i32(slots)
+    # the two kernels
+    k1, v1 = kc.clone(), vc.clone()
+    q = torch.empty(n, nq * hd, device=DEV, dtype=torch.bfloat16)
+    ops.rope_kv_write(parts, q, k1, v1, cos, sin, hd, pos, slots_d, n, nq, nkv, hd, page)
+    want = torch.full((n, nq, hd), float("nan"), device=DEV, dtype=torch.bfloat16)
+    decode_attention(ops, q.view(n, nq, hd), want, k1, v1, list(range(n)), pos, seq_of, table, nq, nkv, hd, page, scale,
+                     window, size=size, alone=alone)
+    assert torch.isfinite(want.float()).all()
+    # the one
+    k2, v2 = kc.clone(), vc.clone()
+    work = decode_work(np.arange(n, dtype=np.int32), pos.cpu().numpy(), n, window, nq, nkv, size=size)
+    cap, items = max(decode_capacity(n, nq, nkv), int(work[0, 0])), decode_items(nq, nkv)
+    acc = torch.full((cap * items * 16 * hd,), float("nan"), device=DEV)
+    ml = torch.full((cap * items * 32,), float("nan"), device=DEV)
+    counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
+    got = torch.full((n, nq, hd), float("nan"), device=DEV, dtype=torch.bfloat16)
+    for _ in range(2):                                       # the second call writes what is there already
+        ops.attn_decode_work_rope_bf16(parts, cos, sin, slots_d, got, k2, v2, True, work_on_device(work, cap), cap, pos,
+                                       seq_of, table, acc, ml, counters, decode_alone(n, nq, nkv) if alone is None else alone,
+                                       nq, nkv, hd, page, scale, window)
+        assert int(counters.abs().sum()) == 0
+        assert torch.equal(got, want)
+        assert torch.equal(k1.view(torch.int16), k2.view(torch.int16)) and torch.equal(v1.view(torch.int16), v2.view(torch.int16))
+    # a layer that keeps no keys and values of its own: the caches stay as they are
+    k3, v3 = k1.clone(), v1.clone()
+    ops.attn_decode_work_rope_bf16(parts, cos, sin, slots_d, got, k3, v3, False, work_on_device(work, cap), cap, pos,
+                                   seq_of, table, acc, ml, counters, True, nq, nkv, hd, page, scale, window)
+    assert torch.equal(got, want) and torch.equal(k3.view(torch.int16), k1.view(torch.int16))
+
+
 @pytest.mark.parametrize("nq,nkv,hd,page", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 50])
 @pytest.mark.parametrize("size,alone", [(None, True), (4, False), (12, True), (None, False)])
