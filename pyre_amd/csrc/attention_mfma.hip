@@ -278,10 +278,10 @@ __device__ inline void attend_regs(const ChunkRegs<HD>& cr, int key0, bool edge,
 // of dispatch, so that the list's order, longest first, is the order in which work starts. The host deals the
 // keys of every request to blocks in proportion to its context, so that a step whose
 // requests differ widely in length keeps all compute units busy for the same time:
-//   work[0]     = (blocks in the list, -, -, -)
+//   work[0]     = (blocks in the list, -, -, -, -, -, -, -)
 //   work[1 + i] = (token in the flat batch, block b of its request + 65536 * blocks nb of its
 //                  request, chunks of 32 keys per wave of this request, first partial slot of
-//                  the request)
+//                  the request, the token's position, its request's row of the block table, -, -)
 // Block b takes the chunks first + 4 b per .. of its request, a run of `per` chunks for each
 // of its four waves, and joins their results through LDS. A request with one block is
 // finished by it. Otherwise each block stores its joined partial result (max, sum,
@@ -355,7 +355,7 @@ template <int HD, bool STREAM_V, bool FUSED>
 __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS, const RopeIn& rope) {
   const int4 head_of_list = work[0];
   if (static_cast<int>(blockIdx.y) >= head_of_list.x) return;
-  const int4 item = work[1 + blockIdx.y];
+  const int4 item = work[2 * (1 + blockIdx.y)], place = work[2 * (1 + blockIdx.y) + 1];
   const int tok = item.x, b = item.y & 0xffff, nb = item.y >> 16, per = item.z, slot0 = item.w;
   // a list that does not fit the launch is not followed
   if (nb < 1 || nb > kMaxBlocksPerRequest || b < 0 || b >= nb || slot0 < 0 || slot0 + nb > static_cast<int>(gridDim.y) || per < 1)
@@ -365,10 +365,12 @@ __device__ __forceinline__ void attn_decode_work_block(PYRE_DECODE_WORK_PARAMS, 
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
   const int kvh = blockIdx.x / qtiles, qt = blockIdx.x % qtiles;
   const int head0 = kvh * n_rep + qt * 16, nheads = min(16, n_rep - qt * 16);
-  const int pos = positions[tok];
+  // the token's position and its request's row of the block table come with the list: nothing else
+  // stands between the list and the first loads of keys
+  const int pos = place.x;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
 
-  KV kv{k_cache, v_cache, block_table + static_cast<size_t>(seq_of_token[tok]) * table_stride, nkv, kvh, page_size};
+  KV kv{k_cache, v_cache, block_table + static_cast<size_t>(place.y) * table_stride, nkv, kvh, page_size};
   Bounds<1> bd{{lo}, {pos}};
 
   const int first = lo / kChunk, last = pos / kChunk;
@@ -1119,7 +1121,7 @@ int launch_decode_work(const void* q, void* out, void* k_cache, void* v_cache, c
                "attn_decode_work_bf16: head_dim %d (multiples of 32 up to 256), page_size %d (multiples of 16), "
                "heads %d/%d are not supported", hd, page_size, nq, nkv);
   PYRE_REQUIRE(table_stride > 0 && capacity >= 0, "attn_decode_work_bf16: bad table or capacity");
-  PYRE_REQUIRE(reinterpret_cast<uintptr_t>(work) % 16 == 0, "attn_decode_work_bf16: the work list must lie on 16 bytes");
+  PYRE_REQUIRE(reinterpret_cast<uintptr_t>(work) % 16 == 0, "attn_decode_work_bf16: the work list must lie on 16 bytes");  // rows of 8 ints
   if (capacity == 0) return 0;
   const int n_rep = nq / nkv, qtiles = (n_rep + 15) / 16;
   PYRE_REQUIRE(capacity <= 65535, "attn_decode_work_bf16: a list of %d blocks is too long for one launch", capacity);

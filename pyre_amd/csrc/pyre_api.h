@@ -117,9 +117,11 @@ int pyre_attn_mfma_supports(int hd, int page_size, int nq, int nkv);
 
 // One new token per request, from a work list that deals every request's keys to blocks of
 // four waves:
-// work[0] = (blocks in the list, 0, 0, 0), work[1 + i] = (token in the flat batch, block b of
-// its request + 65536 * blocks nb of its request (<= 64), chunks `per` of 32 keys that a wave
-// of this request takes, the request's first partial slot); block b takes chunks 4 b per ..
+// rows of eight ints: work[0] = (blocks in the list, 0, ...), work[1 + i] = (token in the flat batch,
+// block b of its request + 65536 * blocks nb of its request (<= 64), chunks `per` of 32 keys that a
+// wave of this request takes, the request's first partial slot, the token's position, its request's
+// row of the block table, 0, 0: the kernel takes position and row from the list, `positions` and
+// `seq_of_token` are not read); block b takes chunks 4 b per ..
 // 4 (b + 1) per - 1 of its request, counted from the first chunk that the token sees, and the
 // nb blocks of a request cover all of them. The slots of the requests are disjoint runs of nb
 // within 0..capacity-1. `alone`: a compute unit runs one block at a time (for steps of so few

@@ -37,7 +37,7 @@ int compute_units() {
 }  // namespace pyre
 
 extern "C" const char* pyre_last_error() { return pyre::error_buffer(); }
-extern "C" int pyre_abi_version() { return 18; }
+extern "C" int pyre_abi_version() { return 19; }
 extern "C" int pyre_compute_units() { return pyre::compute_units(); }
 extern "C" const char* pyre_sources_digest() { return PYRE_SOURCES_DIGEST; }
 

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 
 class KernelError(RuntimeError):

@@ -481,11 +481,11 @@ def _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table,
 def attn_decode_work_bf16(q, out, k_cache, v_cache, work, capacity, positions, seq_of_token, block_table,
                           part_acc, part_ml, counters, alone, nq, nkv, hd, page_size, scale, window=0) -> None:
     """Attention of single new tokens over the paged cache from a work list (int32
-    ``[1 + blocks, 4]``: see ``pyre_attn_decode_work_bf16`` in pyre_api.h) in a launch of
+    ``[1 + blocks, 8]``: see ``pyre_attn_decode_work_bf16`` in pyre_api.h) in a launch of
     ``capacity`` blocks per key/value head, one (``alone``) or two to a compute unit.
     ``counters`` must be zero and is left at zero."""
     _attn_common(q, out, k_cache, v_cache, positions, seq_of_token, block_table, nq, nkv, hd, page_size)
-    _i32("work", work, 4 * (1 + capacity))
+    _i32("work", work, 8 * (1 + capacity))
     items = nkv * -(-(nq // nkv) // 16)
     if part_acc.dtype != torch.float32 or part_acc.numel() < capacity * items * 16 * hd:
         raise KernelError("attn_decode_work: partial accumulators too small")
@@ -525,7 +525,7 @@ def attn_decode_work_rope_bf16(qkv: Partials, cos, sin, slots, out, k_cache, v_c
     if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.dim() != 2 or cos.shape[1] != hd // 2 \
             or cos.shape != sin.shape:
         raise KernelError("attn_decode_work_rope: float32 cos/sin tables [positions, hd / 2] needed")
-    _contig("cos", cos), _contig("sin", sin), _i32("slots", slots, qkv.rows), _i32("work", work, 4 * (1 + capacity))
+    _contig("cos", cos), _contig("sin", sin), _i32("slots", slots, qkv.rows), _i32("work", work, 8 * (1 + capacity))
     items = nkv * -(-(nq // nkv) // 16)
     if part_acc.dtype != torch.float32 or part_acc.numel() < capacity * items * 16 * hd:
         raise KernelError("attn_decode_work: partial accumulators too small")

@@ -92,15 +92,16 @@ class Attention(Mixer):
         s = self.spec
 
         def work(hb):
-            return plan.decode_work(hb.arrays["attention.decode_tokens"], hb.positions, hb.decode_shape()[0],
-                                    s.window, s.num_heads, s.num_kv_heads, units=self.units)
+            listed = plan.decode_work(hb.arrays["attention.decode_tokens"], hb.positions, hb.decode_shape()[0],
+                                      s.window, s.num_heads, s.num_kv_heads, units=self.units)
+            return plan.decode_work_with_places(listed, hb.positions, hb.seq_of_token)
 
         def portions(hb):
             return plan.prefill_work(hb.arrays["attention.prefill_tiles"], hb.positions, s.window,
                                      plan.prefill_items(s.num_heads, s.num_kv_heads), units=self.units)
 
         def decode_cap(n_cap, s_cap):
-            return 4 * (1 + plan.decode_capacity(s_cap, s.num_heads, s.num_kv_heads, self.units))
+            return 8 * (1 + plan.decode_capacity(s_cap, s.num_heads, s.num_kv_heads, self.units))
 
         def prefill_cap(n_cap, s_cap):
             return 8 * plan.prefill_capacity(n_cap, s_cap, TILE, plan.prefill_items(s.num_heads, s.num_kv_heads), self.units)

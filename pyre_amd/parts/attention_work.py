@@ -68,7 +68,8 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
     slot has to work off in all, and the list starts with the longest requests, so that the
     rounds stay full to the end. Row 0 is (blocks, 0, 0, 0), row 1 + i is (token, block of its
     request + 65536 * blocks of its request, chunks per wave, first partial slot of the
-    request). ``size`` fixes the block size instead (for tests of the kernel)."""
+    request). ``size`` fixes the block size instead (for tests of the kernel). The device gets the
+    list from :func:`decode_work_with_places`."""
     n = len(tokens)
     if n == 0:
         return np.zeros((1, 4), dtype=np.int32)
@@ -110,6 +111,18 @@ def decode_work(tokens: np.ndarray, positions: np.ndarray, rows: int, window: in
     work[1:, 2] = per[order][which]
     work[1:, 3] = first[which]
     return work
+
+
+def decode_work_with_places(work: np.ndarray, positions: np.ndarray, seq_of_token: np.ndarray) -> np.ndarray:
+    """The list as the kernel reads it (int32 ``[1 + blocks, 8]``): each row of :func:`decode_work`
+    followed by (position of its token, row of its request's block table, 0, 0), so that a block
+    finds them with the row itself and not by two more loads that depend on it."""
+    out = np.zeros((len(work), 8), dtype=np.int32)
+    out[:, :4] = work
+    tok = work[1:, 0]
+    out[1:, 4] = positions[tok]
+    out[1:, 5] = seq_of_token[tok]
+    return out
 
 
 #: keys per chunk of the prompt-portion kernel; a block of it fills a compute unit (its LDS)

@@ -467,16 +467,20 @@ def decode_attention(ops, q, out, kc, vc, tokens, pos, seq_of, table, nq, nkv, h
     ml = torch.full((cap * items * 32,), float("nan"), device=DEV)
     counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
     alone = decode_alone(rows, nq, nkv) if alone is None else alone
-    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap), cap, pos, seq_of, table, acc, ml, counters,
+    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap, pos, seq_of), cap, pos, seq_of, table, acc, ml, counters,
                               alone, nq, nkv, hd, page, scale, window)
     assert int(counters.abs().sum()) == 0
     return work
 
 
-def work_on_device(work, cap, fill=0):
-    """The list in a buffer as large as the launch: the rows past its end are never read."""
-    flat = np.full(4 * (1 + cap), fill, dtype=np.int32)
-    flat[:work.size] = work.reshape(-1)
+def work_on_device(work, cap, pos, seq_of, fill=0):
+    """The list as the kernel reads it (each row with its token's position and table row behind
+    it), in a buffer as large as the launch: the rows past its end are never read."""
+    from pyre_amd.parts.attention_work import decode_work_with_places
+
+    wide = decode_work_with_places(work, pos.cpu().numpy(), seq_of.cpu().numpy())
+    flat = np.full(8 * (1 + cap), fill, dtype=np.int32)
+    flat[:wide.size] = wide.reshape(-1)
     return i32(flat.tolist())
 
 
@@ -528,7 +532,7 @@ def test_attn_decode_finishes_the_qkv_product_itself(nq, nkv, hd, page, ks, bias
     counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
     got = torch.full((n, nq, hd), float("nan"), device=DEV, dtype=torch.bfloat16)
     for _ in range(2):                                       # the second call writes what is there already
-        ops.attn_decode_work_rope_bf16(parts, cos, sin, slots_d, got, k2, v2, True, work_on_device(work, cap), cap, pos,
+        ops.attn_decode_work_rope_bf16(parts, cos, sin, slots_d, got, k2, v2, True, work_on_device(work, cap, pos, seq_of), cap, pos,
                                        seq_of, table, acc, ml, counters, decode_alone(n, nq, nkv) if alone is None else alone,
                                        nq, nkv, hd, page, scale, window)
         assert int(counters.abs().sum()) == 0
@@ -536,7 +540,7 @@ def test_attn_decode_finishes_the_qkv_product_itself(nq, nkv, hd, page, ks, bias
         assert torch.equal(k1.view(torch.int16), k2.view(torch.int16)) and torch.equal(v1.view(torch.int16), v2.view(torch.int16))
     # a layer that keeps no keys and values of its own: the caches stay as they are
     k3, v3 = k1.clone(), v1.clone()
-    ops.attn_decode_work_rope_bf16(parts, cos, sin, slots_d, got, k3, v3, False, work_on_device(work, cap), cap, pos,
+    ops.attn_decode_work_rope_bf16(parts, cos, sin, slots_d, got, k3, v3, False, work_on_device(work, cap, pos, seq_of), cap, pos,
                                    seq_of, table, acc, ml, counters, True, nq, nkv, hd, page, scale, window)
     assert torch.equal(got, want) and torch.equal(k3.view(torch.int16), k1.view(torch.int16))
 
@@ -572,7 +576,7 @@ def test_attn_decode_from_a_work_list(nq, nkv, hd, page, window, size, alone):
     outs = []
     for _ in range(2):
         out = torch.full_like(q, float("nan"))
-        ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap), cap, pos, seq_of, table, acc, ml,
+        ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap, pos, seq_of), cap, pos, seq_of, table, acc, ml,
                                   counters, alone, nq, nkv, hd, page, scale, window)
         assert torch.allclose(out.double().cpu(), want, atol=2e-2, rtol=2e-2)
         assert int(counters.abs().sum()) == 0
@@ -580,7 +584,7 @@ def test_attn_decode_from_a_work_list(nq, nkv, hd, page, window, size, alone):
     assert torch.equal(outs[0], outs[1])
     # what lies past the list's end is not followed
     out = torch.full_like(q, float("nan"))
-    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap, fill=-7), cap, pos, seq_of, table, acc, ml,
+    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap, pos, seq_of, fill=-7), cap, pos, seq_of, table, acc, ml,
                               counters, alone, nq, nkv, hd, page, scale, window)
     assert torch.equal(out, outs[0])
 
@@ -603,7 +607,7 @@ def test_attn_decode_work_list_in_a_mixed_batch():
     ml = torch.empty(cap * items * 32, device=DEV)
     counters = torch.zeros(cap * items, dtype=torch.int32, device=DEV)
     out = torch.full_like(q, 7.0)
-    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap), cap, pos, seq_of, table, acc, ml, counters,
+    ops.attn_decode_work_bf16(q, out, kc, vc, work_on_device(work, cap, pos, seq_of), cap, pos, seq_of, table, acc, ml, counters,
                               True, nq, nkv, hd, page, scale)
     got = out.double().cpu()
     assert torch.allclose(got[singles.tolist()], want[singles.tolist()], atol=2e-2, rtol=2e-2)

@@ -85,6 +85,20 @@ def test_decode_work_lists_cover_every_key_once():
     assert (decode_work(np.zeros(0, np.int32), np.zeros(4, np.int32), 8, 0, 4, 2) == 0).all()
 
 
+def test_decode_work_carries_position_and_table_row_to_the_device():
+    from pyre_amd.parts.attention_work import decode_work_with_places
+
+    positions = np.asarray([5, 900, 0, 4000, 33], dtype=np.int32)
+    seq_of = np.asarray([3, 0, 4, 1, 2], dtype=np.int32)
+    tokens = np.asarray([1, 3, 4], dtype=np.int32)
+    work = decode_work(tokens, positions, 4, 0, 8, 2)
+    wide = decode_work_with_places(work, positions, seq_of)
+    assert wide.shape == (len(work), 8) and wide.dtype == np.int32
+    assert (wide[:, :4] == work).all() and (wide[0, 4:] == 0).all() and (wide[:, 6:] == 0).all()
+    for tok, pos, seq in wide[1:, [0, 4, 5]].tolist():
+        assert pos == positions[tok] and seq == seq_of[tok]
+
+
 def test_decode_work_of_known_shapes():
     # 7B heads (28 query, 4 key/value: 64 blocks per key/value head at once), 4,096 tokens of context
     pos = lambda n, ctx: np.full(n, ctx, dtype=np.int32)  # noqa: E731
