@@ -335,6 +335,34 @@ def test_long_decoding_against_plain(model, dtype, page, model_dirs, plain_model
     assert eng.graph_replays > 200
 
 
+@pytest.mark.parametrize("graphs", [False, True])
+def test_single_tokens_with_and_without_the_kernel_between_product_and_attention(graphs, model_dirs, plain_models):
+    """Steps of single tokens leave the rotary kernel out on the 16-bit path (the attention kernel
+    finishes the q/k/v product itself); with the option off they run it. Three requests decoded side
+    by side after prompts of different lengths, one joining late, pages filling up: the same bits
+    either way, in the logits of every step."""
+    plain = plain_models["tiny-c"]
+    vocab = plain[0]["vocab_size"]
+    reqs = {r: random_ids(vocab, n, seed=n) for r, n in (("a", 70), ("b", 41), ("c", 90))}
+    steps = [([(r, reqs[r][:n], [n - 1])], []) for r, n in (("a", 20), ("b", 9))]
+    steps += [([("a", reqs["a"][20 + i:21 + i], [0]), ("b", reqs["b"][9 + i:10 + i], [0])], []) for i in range(12)]
+    steps += [([("c", reqs["c"][:50], [49])], [])]
+    steps += [([("a", reqs["a"][32 + i:33 + i], [0]), ("b", reqs["b"][21 + i:22 + i], [0]), ("c", reqs["c"][50 + i:51 + i], [0])],
+               ["b"] if i == 19 else []) for i in range(20)]
+    steps += [([("a", reqs["a"][52 + i:53 + i], [0]), ("c", reqs["c"][70 + i:71 + i], [0])], ["a", "c"] if i == 17 else [])
+              for i in range(18)]
+    outs = []
+    for fused in (True, False):
+        eng = make_engine(model_dirs["tiny-c"], "bfloat16", use_graphs=graphs, page_size=16)
+        eng.runtime.options["rope_in_attention"] = fused
+        outs.append(replay(eng, steps))
+    assert outs[0].keys() == outs[1].keys() and len(outs[0]) == 3 + 24 + 60 + 36
+    assert all(torch.equal(outs[0][k], outs[1][k]) for k in outs[0])
+    want = {r: plain_logits(plain, ids, torch.bfloat16) for r, ids in reqs.items()}
+    bad, _ = first_bad(outs[0], want, TOL["bfloat16"])
+    assert bad is None, bad
+
+
 def test_weights_stored_in_32_bits_run_in_either_mode(tmp_path, plain_models):
     """A tensor stored in 32 bits stays so: a float32 checkpoint runs in the 16-bit
     mode with float32 weights (mixed products), and exactly in the 32-bit mode."""
